@@ -1,0 +1,202 @@
+/*
+ * lumen_hip.h -- C ABI of liblumen_hip.so: Lumen's batch-1 inference path on
+ * one AMD Instinct MI355X (gfx950), hand-written HIP kernels.
+ *
+ * The reference (chen-197/Lumen) is pure Rust with no FFI seam; its operator
+ * API is its public Rust function surface.  Each entry point below replaces
+ * one of those functions and cites it (paths relative to the reference
+ * checkout).  A Rust `extern "C"` block binding these symbols is all the
+ * reference needs to route its hot path here.
+ *
+ * Conventions
+ *  - every function returns an int status (LUMEN_OK == 0); nothing throws or
+ *    aborts across the boundary.  Status codes 1..5 map one-to-one to the
+ *    reference's panics.  lumen_last_error() gives the message of the last
+ *    failure on the calling thread.
+ *  - pointers named *_dev are device pointers (from lumen_malloc or any HIP
+ *    allocation, 16-byte aligned); *_host are host pointers, borrowed for the
+ *    duration of the call only.
+ *  - a lumen_ctx owns one HIP stream; all work of its objects is enqueued on
+ *    it in call order.  Functions that return data to the host synchronise;
+ *    the others only enqueue.  A ctx and its objects are not thread-safe.
+ *  - linear weights are [N, K] row-major = [out_features, in_features]
+ *    (src/layers/basic/linear.rs:8), never transposed.
+ */
+#ifndef LUMEN_HIP_H
+#define LUMEN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------ status */
+#define LUMEN_OK 0
+#define LUMEN_ERR_SHAPE 1        /* src/ops/matmul.rs:24-38 (RHS not 2-D, K mismatch)            */
+#define LUMEN_ERR_KV_OVERFLOW 2  /* src/layers/attention/self_attention.rs:144-149, 341-346      */
+#define LUMEN_ERR_ROPE_RANGE 3   /* src/layers/attention/encoding.rs:63-68, 176-181, 209-214     */
+#define LUMEN_ERR_EMBED_OOB 4    /* src/layers/basic/embedding.rs:55                             */
+#define LUMEN_ERR_CACHE_COUNT 5  /* src/models/llama.rs:182-188                                  */
+#define LUMEN_ERR_INVALID 6      /* null pointer, bad enum, unknown parameter name               */
+#define LUMEN_ERR_HIP 7          /* a HIP runtime call failed                                    */
+#define LUMEN_ERR_NO_DEVICE 8    /* no usable gfx950 device                                      */
+#define LUMEN_ERR_UNSUPPORTED 9  /* shape outside what the kernels are built for                 */
+
+#define LUMEN_DTYPE_F32 0
+#define LUMEN_DTYPE_BF16 1
+
+typedef struct lumen_ctx lumen_ctx;
+typedef struct lumen_rope lumen_rope;
+typedef struct lumen_kv_cache lumen_kv_cache;
+typedef struct lumen_llama lumen_llama;
+
+const char *lumen_last_error(void);
+const char *lumen_version(void);
+
+/* ----------------------------------------------------------------- context */
+int lumen_ctx_create(int device, lumen_ctx **out);
+int lumen_ctx_destroy(lumen_ctx *ctx);
+/* run on a caller-owned hipStream_t instead of the ctx's own (NULL restores it) */
+int lumen_ctx_set_stream(lumen_ctx *ctx, void *hip_stream);
+int lumen_ctx_synchronize(lumen_ctx *ctx);
+/* HIP-event stopwatch on the ctx stream: start enqueues an event, stop
+ * enqueues a second one, waits for it and returns the elapsed milliseconds */
+int lumen_timer_start(lumen_ctx *ctx);
+int lumen_timer_stop(lumen_ctx *ctx, float *ms_out);
+
+/* device memory: stands in for the storage behind the reference's Tensor
+ * (src/autograd.rs:53-64, ArcArray<f32>) */
+int lumen_malloc(lumen_ctx *ctx, size_t bytes, void **dev_out);
+int lumen_free(lumen_ctx *ctx, void *dev);
+int lumen_upload(lumen_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);
+int lumen_download(lumen_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes);
+
+/* --------------------------------------------------------------------- ops */
+/* ops::matmul::matmul forward, src/ops/matmul.rs:10-99.  A [M, K_a] @ W[N, K_w]^T
+ * -> C [M, N].  K_a != K_w -> LUMEN_ERR_SHAPE (:33-38).  M == 1 takes the
+ * memory-bound GEMV (:42-69), M > 1 the MFMA GEMM (:70-92). */
+int lumen_matmul_f32(lumen_ctx *ctx, const float *A_dev, const float *W_dev, float *C_dev,
+                     int M, int N, int K_a, int K_w);
+/* the two branches on their own */
+int lumen_gemv_f32(lumen_ctx *ctx, const float *W_dev, const float *x_dev, float *y_dev, int N, int K);
+int lumen_gemm_f32(lumen_ctx *ctx, const float *A_dev, const float *W_dev, float *C_dev,
+                   int M, int N, int K);
+/* same products with W stored as bf16 bits and widened on load, f32 accumulate:
+ * the device-side form of the reference's load-time upcast, src/loader.rs:50-64 */
+int lumen_gemv_bf16w(lumen_ctx *ctx, const uint16_t *W_dev, const float *x_dev, float *y_dev, int N, int K);
+int lumen_gemm_bf16w(lumen_ctx *ctx, const float *A_dev, const uint16_t *W_dev, float *C_dev,
+                     int M, int N, int K);
+
+/* RMSNorm::forward, src/layers/norm/rms_norm.rs:24-62.  x [rows, dim], w [dim] */
+int lumen_rmsnorm_f32(lumen_ctx *ctx, const float *x_dev, const float *w_dev, float *out_dev,
+                      int rows, int dim, float eps);
+/* SiLU::forward, src/layers/activation.rs:139-146 */
+int lumen_silu_f32(lumen_ctx *ctx, const float *x_dev, float *out_dev, size_t n);
+/* Tensor + Tensor and Tensor * Tensor, same shape, src/ops/arithmetic.rs:48-51, 105-108 */
+int lumen_add_f32(lumen_ctx *ctx, const float *a_dev, const float *b_dev, float *out_dev, size_t n);
+int lumen_mul_f32(lumen_ctx *ctx, const float *a_dev, const float *b_dev, float *out_dev, size_t n);
+/* silu(gate) * up in one pass: the three elementwise ops of LlamaMLP::forward,
+ * src/models/llama.rs:60-63 */
+int lumen_swiglu_f32(lumen_ctx *ctx, const float *gate_dev, const float *up_dev, float *out_dev, size_t n);
+/* Embedding::forward, src/layers/basic/embedding.rs:21-57.  ids are f32 on
+ * the host like the reference's (src/main.rs:143-152), cast as `as usize`;
+ * idx >= vocab -> LUMEN_ERR_EMBED_OOB.  out [n_ids, dim] */
+int lumen_embedding_f32(lumen_ctx *ctx, const float *W_dev, const float *ids_host, int n_ids,
+                        int vocab, int dim, float *out_dev);
+/* greedy pick, lowest index on ties (the reference samples top-p from an
+ * unseeded RNG, src/main.rs:74-137; greedy is this build's deterministic stand-in) */
+int lumen_argmax_f32(lumen_ctx *ctx, const float *x_dev, int n, int *index_host_out);
+
+/* ------------------------------------------------------------------- RoPE */
+/* RotaryEmbedding::new + precompute_freqs_cis, src/layers/attention/encoding.rs:17-54.
+ * Tables are computed on the host with the reference's exact f32 formula and
+ * uploaded once: [max_seq, dim] cos and sin. */
+int lumen_rope_create(lumen_ctx *ctx, int dim, int max_seq, float theta, lumen_rope **out);
+int lumen_rope_destroy(lumen_rope *rope);
+int lumen_rope_tables_download(lumen_rope *rope, float *cos_host, float *sin_host);
+/* RotaryEmbedding::forward, encoding.rs:56-123.  x, out [B, H, S, D]; offset + S > max_seq
+ * -> LUMEN_ERR_ROPE_RANGE (:62-68) */
+int lumen_rope_forward_f32(lumen_rope *rope, const float *x_dev, float *out_dev,
+                           int b, int h, int s, int d, int offset);
+/* RotaryEmbedding::rope_1token_copy, encoding.rs:173-204.  src, dst [D] */
+int lumen_rope_1token_copy_f32(lumen_rope *rope, const float *src_dev, float *dst_dev, int d, int pos);
+
+/* --------------------------------------------------------------- KV cache */
+/* KVCacheInner, src/layers/attention/self_attention.rs:24-44: k, v
+ * [B, H_kv, max_seq, D] f32 zero-initialised in HBM, plus len.  Allocated
+ * once; nothing is allocated per token. */
+int lumen_kv_cache_create(lumen_ctx *ctx, int b, int h_kv, int max_seq, int d, lumen_kv_cache **out);
+int lumen_kv_cache_destroy(lumen_kv_cache *cache);
+int lumen_kv_cache_reset(lumen_kv_cache *cache);               /* :41-43, len = 0, data kept */
+int lumen_kv_cache_len(const lumen_kv_cache *cache, int *len_out);
+int lumen_kv_cache_ptrs(const lumen_kv_cache *cache, float **k_dev_out, float **v_dev_out);
+/* legacy LlamaKVCache::update / get_view, src/kv_cache.rs:31-59: k, v
+ * [B, H_kv, S, D] written at start_pos (overflow -> LUMEN_ERR_KV_OVERFLOW);
+ * get_view copies the first current_len positions out, [B, H_kv, current_len, D] */
+int lumen_kv_cache_update(lumen_kv_cache *cache, const float *k_dev, const float *v_dev, int s, int start_pos);
+int lumen_kv_cache_get_view(const lumen_kv_cache *cache, int current_len, float *k_out_dev, float *v_out_dev);
+
+/* -------------------------------------------------------------- attention */
+/* SelfAttention::forward decode core, S == 1, self_attention.rs:125-297:
+ * q3 [B, H, D], k3/v3 [B, H_kv, D] un-rotated projections.  Writes RoPE(k)
+ * and v into the cache at position len, sets len += 1, rotates q, runs the
+ * online-softmax GQA attention over the cache, out [B, 1, H, D]. */
+int lumen_attn_decode_f32(lumen_kv_cache *cache, lumen_rope *rope, const float *q3_dev,
+                          const float *k3_dev, const float *v3_dev, float *out_dev,
+                          int h, float scale, int causal);
+/* SelfAttention::forward prefill core, S > 1, self_attention.rs:308-419 with
+ * gqa_attention_no_repeat_bshd_view :519-641 and softmax_inplace_view :643-678:
+ * q [B, S, H, D], k/v [B, S, H_kv, D] un-rotated; appends S positions to the
+ * cache (which may already hold past_len > 0), out [B, S, H, D]. */
+int lumen_attn_prefill_f32(lumen_kv_cache *cache, lumen_rope *rope, const float *q_dev,
+                           const float *k_dev, const float *v_dev, float *out_dev,
+                           int s, int h, float scale, int causal);
+
+/* ------------------------------------------------------------------ model */
+/* LlamaConfig, src/models/llama.rs:11-37, plus what the other benchmark
+ * shapes need and the reference lacks (head_dim, qk_norm, tie_embeddings,
+ * weight_dtype). */
+typedef struct {
+    int vocab_size, hidden_size, intermediate_size, num_hidden_layers;
+    int num_attention_heads, num_key_value_heads;
+    float rms_norm_eps;
+    int max_seq_len;
+    float rope_theta;
+    int head_dim;        /* 0 => hidden_size / num_attention_heads (llama.rs:162) */
+    int qk_norm;         /* per-head RMSNorm on q and k before RoPE               */
+    int tie_embeddings;  /* lm_head shares model.embed_tokens.weight              */
+    int weight_dtype;    /* LUMEN_DTYPE_F32, or LUMEN_DTYPE_BF16 for the linear weights */
+} lumen_llama_config;
+
+/* LlamaModel::new + init_kv_caches(1), llama.rs:138-169: allocates weights,
+ * the static KV caches of all layers and every activation buffer once. */
+int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg, lumen_llama **out);
+int lumen_llama_destroy(lumen_llama *model);
+/* ModelLoader::load_llama_weights for one tensor, src/loader.rs:23-68, by its
+ * HF name (LlamaModel::named_parameters, llama.rs:218-279).  dtype f32 or
+ * bf16 bits (widened like loader.rs:58 when the model stores f32); shape must
+ * match -> LUMEN_ERR_SHAPE; unknown name -> LUMEN_ERR_INVALID. */
+int lumen_llama_set_param(lumen_llama *model, const char *name, const void *data_host,
+                          int dtype, const int64_t *shape, int ndim);
+/* LlamaModel::forward, llama.rs:181-206: ids_host [S] as f32 (main.rs:143-152);
+ * S == 1 takes the decode path, S > 1 prefill (appending to the live cache).
+ * logits_host receives [S, V] when all_rows != 0 (what the reference computes)
+ * or just the last position [V] (what its caller keeps, main.rs:155-163). */
+int lumen_llama_forward(lumen_llama *model, const float *ids_host, int s, float *logits_host, int all_rows);
+/* the generation loop of src/main.rs:340-378 with greedy picks: feeds
+ * first_id, then each argmax, for n steps, without leaving the GPU.
+ * ids_out_host [n] receives the picks; logits_out_host [n, V] is optional. */
+int lumen_llama_decode_greedy(lumen_llama *model, int first_id, int n, int32_t *ids_out_host,
+                              float *logits_out_host);
+int lumen_llama_reset(lumen_llama *model);                      /* reset_kv_caches, llama.rs:172-176 */
+int lumen_llama_kv_len(const lumen_llama *model, int *len_out);
+int lumen_llama_cache_download(lumen_llama *model, int layer, float *k_host, float *v_host);
+/* bytes of weights + KV prefix one decode step at cache length len must read */
+int lumen_llama_decode_bytes(const lumen_llama *model, int len, double *bytes_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,607 @@
+// Static KV cache and GQA attention over it.
+//
+//  * decode (S == 1), src/layers/attention/self_attention.rs:125-297: one
+//    workgroup per (KV head, slice of the cached positions).  The n_rep query
+//    heads of the KV group are rotated once into LDS; every K/V row is read
+//    from HBM exactly once per group as 16-byte pieces (D/4 lanes per row)
+//    and used for all n_rep heads from registers.  Each lane group keeps an
+//    online-softmax state (m, l, ctx); states are merged across lane groups
+//    with shuffles, across wavefronts through LDS and across slices through
+//    a small global scratch by the last workgroup to finish (fixed order, so
+//    results are reproducible run to run).
+//  * prefill (S > 1), self_attention.rs:308-419 + :519-678: rotate q/k and
+//    append to the cache, then one workgroup per (query position, KV group)
+//    runs the same row loop over the causal prefix.
+#include "internal.h"
+
+#include <cmath>
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+#define ATT_THREADS 256
+#define ATT_WAVES 4
+
+template <int NREP>
+struct AttnState {
+    float m[NREP], l[NREP];
+    v4f acc[NREP];
+};
+
+template <int NREP>
+__device__ __forceinline__ void state_init(AttnState<NREP> &st) {
+#pragma unroll
+    for (int r = 0; r < NREP; ++r) {
+        st.m[r] = -INFINITY;
+        st.l[r] = 0.f;
+        st.acc[r] = (v4f){0.f, 0.f, 0.f, 0.f};
+    }
+}
+
+// One K/V row piece per lane: score for each of the NREP heads, online-softmax update.
+template <int D, int NREP>
+__device__ __forceinline__ void attn_step(AttnState<NREP> &st, const v4f (&q)[NREP], const v4f kv, const v4f vv,
+                                          bool valid, float scale) {
+    constexpr int LPR = D / 4;
+#pragma unroll
+    for (int r = 0; r < NREP; ++r) {
+        float s = q[r].x * kv.x;
+        s = fmaf(q[r].y, kv.y, s);
+        s = fmaf(q[r].z, kv.z, s);
+        s = fmaf(q[r].w, kv.w, s);
+#pragma unroll
+        for (int off = LPR / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+        s = valid ? s * scale : -INFINITY;
+        const float m_new = fmaxf(st.m[r], s);
+        if (m_new > -INFINITY) {
+            const float alpha = expf(st.m[r] - m_new);  // exp(-inf) = 0 on the first row
+            const float p = expf(s - m_new);
+            st.l[r] = fmaf(st.l[r], alpha, p);
+            st.acc[r].x = fmaf(st.acc[r].x, alpha, p * vv.x);
+            st.acc[r].y = fmaf(st.acc[r].y, alpha, p * vv.y);
+            st.acc[r].z = fmaf(st.acc[r].z, alpha, p * vv.z);
+            st.acc[r].w = fmaf(st.acc[r].w, alpha, p * vv.w);
+            st.m[r] = m_new;
+        }
+    }
+}
+
+// Rows [p0, p1) of one KV head (Kb/Vb point at row 0), spread over the
+// workgroup's 4 wavefronts x (64/LPR) lane groups.
+template <int D, int NREP>
+__device__ __forceinline__ void attn_rows(AttnState<NREP> &st, const v4f (&q)[NREP], const float *__restrict__ Kb,
+                                          const float *__restrict__ Vb, int p0, int p1, float scale) {
+    constexpr int LPR = D / 4;
+    constexpr int RPW = 64 / LPR;
+    constexpr int RPI = ATT_WAVES * RPW;  // rows per workgroup iteration
+    constexpr int U = 4;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int slot = lane / LPR, c = lane % LPR;
+    const int off = wave * RPW + slot;
+    for (int base = p0; base < p1; base += RPI * U) {  // trip count is uniform over the workgroup
+        v4f kv[U], vv[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int j = base + u * RPI + off;
+            kv[u] = (v4f){0.f, 0.f, 0.f, 0.f};
+            vv[u] = (v4f){0.f, 0.f, 0.f, 0.f};
+            if (j < p1) {
+                kv[u] = *(const v4f *)(Kb + (size_t)j * D + c * 4);
+                vv[u] = *(const v4f *)(Vb + (size_t)j * D + c * 4);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            // uniform test: every lane of the wavefront takes the step (it shuffles), rows past p1 are masked
+            if (base + u * RPI < p1) attn_step<D, NREP>(st, q, kv[u], vv[u], base + u * RPI + off < p1, scale);
+        }
+    }
+}
+
+// Merge the lane-group states of each wavefront and publish one state per
+// wavefront in LDS (sm, sl [ATT_WAVES][NREP]; sacc [ATT_WAVES][NREP][D]).
+// Ends with a workgroup barrier; wave_fold() then combines the wavefronts.
+template <int D, int NREP>
+__device__ __forceinline__ void block_merge(AttnState<NREP> &st, float *sm, float *sl, float *sacc) {
+    constexpr int LPR = D / 4;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int slot = lane / LPR, c = lane % LPR;
+#pragma unroll
+    for (int r = 0; r < NREP; ++r) {
+#pragma unroll
+        for (int off = LPR; off < 64; off <<= 1) {
+            const float mo = __shfl_xor(st.m[r], off, 64);
+            const float lo = __shfl_xor(st.l[r], off, 64);
+            v4f ao;
+            ao.x = __shfl_xor(st.acc[r].x, off, 64);
+            ao.y = __shfl_xor(st.acc[r].y, off, 64);
+            ao.z = __shfl_xor(st.acc[r].z, off, 64);
+            ao.w = __shfl_xor(st.acc[r].w, off, 64);
+            const float mn = fmaxf(st.m[r], mo);
+            const float a = (mn > -INFINITY) ? expf(st.m[r] - mn) : 0.f;
+            const float b = (mn > -INFINITY) ? expf(mo - mn) : 0.f;
+            st.l[r] = st.l[r] * a + lo * b;
+            st.acc[r].x = st.acc[r].x * a + ao.x * b;
+            st.acc[r].y = st.acc[r].y * a + ao.y * b;
+            st.acc[r].z = st.acc[r].z * a + ao.z * b;
+            st.acc[r].w = st.acc[r].w * a + ao.w * b;
+            st.m[r] = mn;
+        }
+        if (slot == 0) {
+            if (c == 0) {
+                sm[wave * NREP + r] = st.m[r];
+                sl[wave * NREP + r] = st.l[r];
+            }
+            *(v4f *)(sacc + ((size_t)(wave * NREP + r)) * D + c * 4) = st.acc[r];
+        }
+    }
+    __syncthreads();
+}
+
+// (max, sum, ctx) of head r, dim dd over the wavefront states in LDS
+template <int D, int NREP>
+__device__ __forceinline__ void wave_fold(const float *sm, const float *sl, const float *sacc, int r, int dd,
+                                          float &mm, float &ls, float &cx) {
+    mm = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < ATT_WAVES; ++w) mm = fmaxf(mm, sm[w * NREP + r]);
+    ls = 0.f;
+    cx = 0.f;
+    if (mm > -INFINITY) {
+#pragma unroll
+        for (int w = 0; w < ATT_WAVES; ++w) {
+            const float ex = expf(sm[w * NREP + r] - mm);
+            ls = fmaf(sl[w * NREP + r], ex, ls);
+            cx = fmaf(sacc[((size_t)(w * NREP + r)) * D + dd], ex, cx);
+        }
+    }
+}
+
+// Optional per-head RMSNorm (gain g) then half-split RoPE of NH contiguous
+// heads held raw in LDS `raw` ([NH][D]) into `rot`.  cs/sn: table rows at the
+// token's position.  q: (x1*c - x2*s, x1*s + x2*c), self_attention.rs:220-227;
+// k: same values, encoding.rs:196-203.
+template <int D>
+__device__ __forceinline__ void norm_rope_heads(const float *raw, float *rot, int nh, const float *__restrict__ cs,
+                                                const float *__restrict__ sn, const float *__restrict__ g,
+                                                float eps) {
+    constexpr int HALF = D / 2;
+    for (int p = threadIdx.x; p < nh * HALF; p += ATT_THREADS) {
+        const int r = p / HALF, j = p % HALF;
+        float x1 = raw[r * D + j], x2 = raw[r * D + j + HALF];
+        if (g) {
+            float ss = 0.f;
+            for (int i = 0; i < D; ++i) ss = fmaf(raw[r * D + i], raw[r * D + i], ss);
+            const float inv = 1.0f / sqrtf(ss / (float)D + eps);
+            x1 = x1 * inv * g[j];
+            x2 = x2 * inv * g[j + HALF];
+        }
+        const float c = cs[j], s = sn[j];
+        rot[r * D + j] = __fsub_rn(__fmul_rn(x1, c), __fmul_rn(x2, s));
+        rot[r * D + j + HALF] = __fadd_rn(__fmul_rn(x1, s), __fmul_rn(x2, c));
+    }
+}
+
+template <int D, int NREP>
+__global__ __launch_bounds__(ATT_THREADS) void attn_decode_kernel(AttnDecodeArgs a) {
+    constexpr int LPR = D / 4;
+    constexpr int RPW = 64 / LPR;
+    constexpr int RPI = ATT_WAVES * RPW;
+    __shared__ __align__(16) float q_raw[NREP * D];
+    __shared__ __align__(16) float q_rot[NREP * D];
+    __shared__ __align__(16) float k_raw[D];
+    __shared__ __align__(16) float k_new[D];
+    __shared__ __align__(16) float v_new[D];
+    __shared__ __align__(16) float sacc[ATT_WAVES * NREP * D];
+    __shared__ float sm[ATT_WAVES * NREP], sl[ATT_WAVES * NREP];
+    __shared__ int s_last;
+
+    const int split = blockIdx.x, hk = blockIdx.y, bb = blockIdx.z;
+    const int nsplit = gridDim.x;
+    const int pos = a.pos_dev ? *a.pos_dev : a.pos_host;  // == past_len
+    const bool has_new = (split == nsplit - 1);
+    const float *cs = a.cos_t + (size_t)pos * D, *sn = a.sin_t + (size_t)pos * D;
+    const size_t head_base = ((size_t)bb * a.hkv + hk) * a.max_seq * D;
+
+    // stage raw q heads of this KV group (contiguous: hq = hk*NREP + r) and the new k / v
+    const float *q_src = a.q + ((size_t)bb * a.hq + (size_t)hk * NREP) * D;
+    for (int i = threadIdx.x; i < NREP * D; i += ATT_THREADS) q_raw[i] = q_src[i];
+    if (has_new) {
+        const float *k_src = a.k_new + ((size_t)bb * a.hkv + hk) * D;
+        const float *v_src = a.v_new + ((size_t)bb * a.hkv + hk) * D;
+        for (int i = threadIdx.x; i < D; i += ATT_THREADS) {
+            k_raw[i] = k_src[i];
+            v_new[i] = v_src[i];
+        }
+    }
+    __syncthreads();
+    norm_rope_heads<D>(q_raw, q_rot, NREP, cs, sn, a.q_norm_w, a.norm_eps);
+    if (has_new) norm_rope_heads<D>(k_raw, k_new, 1, cs, sn, a.k_norm_w, a.norm_eps);
+    __syncthreads();
+    if (has_new) {
+        // self_attention.rs:161-176: rotated k and raw v go to cache row `pos`
+        for (int i = threadIdx.x; i < D; i += ATT_THREADS) {
+            a.k_cache[head_base + (size_t)pos * D + i] = k_new[i];
+            a.v_cache[head_base + (size_t)pos * D + i] = v_new[i];
+        }
+    }
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int slot = lane / LPR, c = lane % LPR;
+    v4f q[NREP];
+#pragma unroll
+    for (int r = 0; r < NREP; ++r) q[r] = *(const v4f *)(q_rot + r * D + c * 4);
+
+    // this slice's share of the cached rows [0, pos)
+    int chunk = (pos + nsplit - 1) / nsplit;
+    chunk = (chunk + RPI - 1) / RPI * RPI;
+    const int p0 = min(pos, split * chunk), p1 = min(pos, p0 + chunk);
+
+    AttnState<NREP> st;
+    state_init<NREP>(st);
+    attn_rows<D, NREP>(st, q, a.k_cache + head_base, a.v_cache + head_base, p0, p1, a.scale);
+    if (has_new) {
+        // the new token's row comes from LDS (lane group 0 of wavefront 0)
+        const bool mine = (wave == 0 && slot == 0);
+        const v4f kv = *(const v4f *)(k_new + c * 4);
+        const v4f vv = *(const v4f *)(v_new + c * 4);
+        if (wave == 0) attn_step<D, NREP>(st, q, kv, vv, mine, a.scale);
+    }
+
+    block_merge<D, NREP>(st, sm, sl, sacc);
+    const int t = threadIdx.x;
+    for (int e = t; e < NREP * D; e += ATT_THREADS) {
+        const int r = e / D, dd = e % D;
+        float mm, ls, cx;
+        wave_fold<D, NREP>(sm, sl, sacc, r, dd, mm, ls, cx);
+        const int hq = hk * NREP + r;
+        if (nsplit == 1) {
+            // out = ctx / (l + 1e-9), self_attention.rs:287-290
+            a.out[((size_t)bb * a.hq + hq) * D + dd] = cx * (1.0f / (ls + 1e-9f));
+        } else {
+            float *pp = a.part + (((size_t)bb * a.hq + hq) * nsplit + split) * (D + 2);
+            pp[dd] = cx;
+            if (dd == 0) {
+                pp[D] = mm;
+                pp[D + 1] = ls;
+            }
+        }
+    }
+    if (nsplit == 1) return;
+
+    // last workgroup of this (batch, KV head) to arrive folds the slices in index order
+    __threadfence();
+    __syncthreads();
+    if (t == 0) {
+        const int old = atomicAdd(&a.counters[bb * a.hkv + hk], 1);
+        s_last = (old == nsplit - 1);
+    }
+    __syncthreads();
+    if (!s_last) return;
+    __threadfence();
+    for (int e = t; e < NREP * D; e += ATT_THREADS) {
+        const int r = e / D, dd = e % D;
+        const int hq = hk * NREP + r;
+        const float *pp = a.part + (((size_t)bb * a.hq + hq) * nsplit) * (D + 2);
+        float mm = -INFINITY;
+        for (int s = 0; s < nsplit; ++s)
+            mm = fmaxf(mm, __hip_atomic_load(pp + (size_t)s * (D + 2) + D, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        float ls = 0.f, cx = 0.f;
+        for (int s = 0; s < nsplit; ++s) {
+            const float ms = __hip_atomic_load(pp + (size_t)s * (D + 2) + D, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (ms > -INFINITY) {
+                const float ex = expf(ms - mm);
+                ls = fmaf(__hip_atomic_load(pp + (size_t)s * (D + 2) + D + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), ex, ls);
+                cx = fmaf(__hip_atomic_load(pp + (size_t)s * (D + 2) + dd, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), ex, cx);
+            }
+        }
+        a.out[((size_t)bb * a.hq + hq) * D + dd] = cx * (1.0f / (ls + 1e-9f));
+    }
+    if (t == 0) a.counters[bb * a.hkv + hk] = 0;  // ready for the next launch
+}
+
+int attn_decode_nsplit(int max_seq) {
+    int n = max_seq / 64;
+    if (n < 1) n = 1;
+    if (n > 64) n = 64;
+    return n;
+}
+
+size_t attn_decode_part_floats(int b, int hq, int d, int nsplit) { return (size_t)b * hq * nsplit * (d + 2); }
+
+template <int D>
+static int launch_decode_d(lumen_ctx *ctx, const AttnDecodeArgs &a) {
+    dim3 grid(a.nsplit, a.hkv, a.b), block(ATT_THREADS);
+    const int nrep = a.hq / a.hkv;
+    switch (nrep) {
+        case 1: hipLaunchKernelGGL((attn_decode_kernel<D, 1>), grid, block, 0, ctx->stream, a); break;
+        case 2: hipLaunchKernelGGL((attn_decode_kernel<D, 2>), grid, block, 0, ctx->stream, a); break;
+        case 4: hipLaunchKernelGGL((attn_decode_kernel<D, 4>), grid, block, 0, ctx->stream, a); break;
+        case 8: hipLaunchKernelGGL((attn_decode_kernel<D, 8>), grid, block, 0, ctx->stream, a); break;
+        default: LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "decode attention: n_rep=%d (supported 1, 2, 4, 8)", nrep);
+    }
+    LUMEN_CHECK_LAUNCH();
+    return LUMEN_OK;
+}
+
+int launch_attn_decode(lumen_ctx *ctx, const AttnDecodeArgs &a) {
+    if (a.hkv <= 0 || a.hq % a.hkv) LUMEN_FAIL(LUMEN_ERR_SHAPE, "heads %d not a multiple of kv heads %d", a.hq, a.hkv);
+    switch (a.d) {
+        case 16: return launch_decode_d<16>(ctx, a);
+        case 32: return launch_decode_d<32>(ctx, a);
+        case 64: return launch_decode_d<64>(ctx, a);
+        case 128: return launch_decode_d<128>(ctx, a);
+        default: LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "decode attention: head_dim=%d (supported 16, 32, 64, 128)", a.d);
+    }
+}
+
+// ------------------------------------------------------------------- prefill
+// q/k-norm + RoPE + cache append for S new positions.
+// q_rot [B,S,Hq,D] = rope(q); cache.k[b,hk,past+s,:] = rope(k); cache.v[...] = v
+// (encoding.rs:56-123 at offset past_len; self_attention.rs:397-402)
+template <int D>
+__global__ __launch_bounds__(ATT_THREADS) void prefill_rope_kernel(AttnPrefillArgs a) {
+    __shared__ __align__(16) float raw[8 * D];
+    __shared__ __align__(16) float rot[8 * D];
+    const int ss = blockIdx.x, bb = blockIdx.y;
+    const int pos = a.past_len + ss;
+    const float *cs = a.cos_t + (size_t)pos * D, *sn = a.sin_t + (size_t)pos * D;
+    const float *qrow = a.q + ((size_t)bb * a.s + ss) * a.q_stride;
+    const float *krow = a.k + ((size_t)bb * a.s + ss) * a.k_stride;
+    const float *vrow = a.v + ((size_t)bb * a.s + ss) * a.v_stride;
+    float *qo = a.q_rot + ((size_t)bb * a.s + ss) * (size_t)a.hq * D;
+    for (int h0 = 0; h0 < a.hq; h0 += 8) {
+        const int nh = min(8, a.hq - h0);
+        __syncthreads();
+        for (int i = threadIdx.x; i < nh * D; i += ATT_THREADS) raw[i] = qrow[(size_t)h0 * D + i];
+        __syncthreads();
+        norm_rope_heads<D>(raw, rot, nh, cs, sn, a.q_norm_w, a.norm_eps);
+        __syncthreads();
+        for (int i = threadIdx.x; i < nh * D; i += ATT_THREADS) qo[(size_t)h0 * D + i] = rot[i];
+    }
+    for (int h0 = 0; h0 < a.hkv; h0 += 8) {
+        const int nh = min(8, a.hkv - h0);
+        __syncthreads();
+        for (int i = threadIdx.x; i < nh * D; i += ATT_THREADS) raw[i] = krow[(size_t)h0 * D + i];
+        __syncthreads();
+        norm_rope_heads<D>(raw, rot, nh, cs, sn, a.k_norm_w, a.norm_eps);
+        __syncthreads();
+        for (int i = threadIdx.x; i < nh * D; i += ATT_THREADS) {
+            const int hk = h0 + i / D, dd = i % D;
+            const size_t dst = (((size_t)bb * a.hkv + hk) * a.max_seq + pos) * D + dd;
+            a.k_cache[dst] = rot[i];
+            a.v_cache[dst] = vrow[(size_t)hk * D + dd];
+        }
+    }
+}
+
+// One workgroup per (query position, KV group): scores over the causal prefix
+// j <= past_len + i (softmax_inplace_view, self_attention.rs:643-678), ctx = P V,
+// out [B,S,Hq,D] (BSHD, :534).
+template <int D, int NREP>
+__global__ __launch_bounds__(ATT_THREADS) void attn_prefill_kernel(AttnPrefillArgs a) {
+    constexpr int LPR = D / 4;
+    __shared__ __align__(16) float sacc[ATT_WAVES * NREP * D];
+    __shared__ float sm[ATT_WAVES * NREP], sl[ATT_WAVES * NREP];
+    const int i = blockIdx.x, hk = blockIdx.y, bb = blockIdx.z;
+    const int L = a.past_len + a.s;
+    const int q_abs = a.past_len + i;
+    const int p1 = a.causal ? min(L, q_abs + 1) : L;
+    const size_t head_base = ((size_t)bb * a.hkv + hk) * a.max_seq * D;
+    const int lane = threadIdx.x & 63;
+    const int c = lane % LPR;
+    const float *qr = a.q_rot + (((size_t)bb * a.s + i) * a.hq + (size_t)hk * NREP) * D;
+    v4f q[NREP];
+#pragma unroll
+    for (int r = 0; r < NREP; ++r) q[r] = *(const v4f *)(qr + r * D + c * 4);
+    AttnState<NREP> st;
+    state_init<NREP>(st);
+    attn_rows<D, NREP>(st, q, a.k_cache + head_base, a.v_cache + head_base, 0, p1, a.scale);
+    block_merge<D, NREP>(st, sm, sl, sacc);
+    for (int e = threadIdx.x; e < NREP * D; e += ATT_THREADS) {
+        const int r = e / D, dd = e % D;
+        float mm, ls, cx;
+        wave_fold<D, NREP>(sm, sl, sacc, r, dd, mm, ls, cx);
+        a.out[(((size_t)bb * a.s + i) * a.hq + hk * NREP + r) * D + dd] = cx * (1.0f / (ls + 1e-9f));
+    }
+}
+
+template <int D>
+static int launch_prefill_d(lumen_ctx *ctx, const AttnPrefillArgs &a) {
+    hipLaunchKernelGGL(prefill_rope_kernel<D>, dim3(a.s, a.b), dim3(ATT_THREADS), 0, ctx->stream, a);
+    LUMEN_CHECK_LAUNCH();
+    dim3 grid(a.s, a.hkv, a.b), block(ATT_THREADS);
+    const int nrep = a.hq / a.hkv;
+    switch (nrep) {
+        case 1: hipLaunchKernelGGL((attn_prefill_kernel<D, 1>), grid, block, 0, ctx->stream, a); break;
+        case 2: hipLaunchKernelGGL((attn_prefill_kernel<D, 2>), grid, block, 0, ctx->stream, a); break;
+        case 4: hipLaunchKernelGGL((attn_prefill_kernel<D, 4>), grid, block, 0, ctx->stream, a); break;
+        case 8: hipLaunchKernelGGL((attn_prefill_kernel<D, 8>), grid, block, 0, ctx->stream, a); break;
+        default: LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "prefill attention: n_rep=%d (supported 1, 2, 4, 8)", nrep);
+    }
+    LUMEN_CHECK_LAUNCH();
+    return LUMEN_OK;
+}
+
+int launch_attn_prefill(lumen_ctx *ctx, const AttnPrefillArgs &a) {
+    if (a.hkv <= 0 || a.hq % a.hkv) LUMEN_FAIL(LUMEN_ERR_SHAPE, "heads %d not a multiple of kv heads %d", a.hq, a.hkv);
+    if (a.s <= 0) return LUMEN_OK;
+    switch (a.d) {
+        case 16: return launch_prefill_d<16>(ctx, a);
+        case 32: return launch_prefill_d<32>(ctx, a);
+        case 64: return launch_prefill_d<64>(ctx, a);
+        case 128: return launch_prefill_d<128>(ctx, a);
+        default: LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "prefill attention: head_dim=%d (supported 16, 32, 64, 128)", a.d);
+    }
+}
+
+// ------------------------------------------------------------------ KV cache
+// legacy LlamaKVCache::update, src/kv_cache.rs:31-49: [B,Hkv,S,D] -> cache[.., start..start+S, ..]
+__global__ __launch_bounds__(256) void kv_update_kernel(const float *__restrict__ src, float *__restrict__ dst, int s,
+                                                        int d, int max_seq, int start, size_t n) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const size_t dd = i % d, ss = (i / d) % s, bh = i / ((size_t)d * s);
+        dst[(bh * max_seq + start + ss) * d + dd] = src[i];
+    }
+}
+
+// legacy LlamaKVCache::get_view, src/kv_cache.rs:51-59: copy of the first cur positions
+__global__ __launch_bounds__(256) void kv_view_kernel(const float *__restrict__ src, float *__restrict__ dst, int cur,
+                                                      int d, int max_seq, size_t n) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const size_t dd = i % d, ss = (i / d) % cur, bh = i / ((size_t)d * cur);
+        dst[i] = src[(bh * max_seq + ss) * d + dd];
+    }
+}
+
+static unsigned ew_blocks(lumen_ctx *ctx, size_t n) {
+    size_t blocks = (n + 255) / 256;
+    const size_t cap = (size_t)ctx->num_cus * 16;
+    return (unsigned)(blocks > cap ? cap : (blocks ? blocks : 1));
+}
+
+extern "C" int lumen_kv_cache_create(lumen_ctx *ctx, int b, int h_kv, int max_seq, int d, lumen_kv_cache **out) {
+    if (!ctx || !out) LUMEN_FAIL(LUMEN_ERR_INVALID, "kv_cache_create: null argument");
+    if (b <= 0 || h_kv <= 0 || max_seq <= 0 || d <= 0)
+        LUMEN_FAIL(LUMEN_ERR_SHAPE, "kv_cache_create: b=%d h_kv=%d max_seq=%d d=%d", b, h_kv, max_seq, d);
+    lumen_kv_cache *c = new lumen_kv_cache();
+    c->ctx = ctx; c->b = b; c->h_kv = h_kv; c->max_seq = max_seq; c->d = d; c->len = 0; c->owns = true;
+    const size_t bytes = sizeof(float) * (size_t)b * h_kv * max_seq * d;
+    if (hipMalloc((void **)&c->k, bytes) != hipSuccess || hipMalloc((void **)&c->v, bytes) != hipSuccess) {
+        hipFree(c->k);
+        delete c;
+        LUMEN_FAIL(LUMEN_ERR_HIP, "kv_cache_create: hipMalloc of 2 x %zu bytes failed", bytes);
+    }
+    // zero-initialised like Array4::zeros (self_attention.rs:35-36); eager, never graph-captured
+    HIP_TRY(hipMemsetAsync(c->k, 0, bytes, ctx->stream));
+    HIP_TRY(hipMemsetAsync(c->v, 0, bytes, ctx->stream));
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    *out = c;
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_kv_cache_destroy(lumen_kv_cache *c) {
+    if (!c) return LUMEN_OK;
+    hipStreamSynchronize(c->ctx->stream);
+    if (c->owns) {
+        hipFree(c->k);
+        hipFree(c->v);
+    }
+    hipFree(c->part);
+    hipFree(c->counters);
+    delete c;
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_kv_cache_reset(lumen_kv_cache *c) {
+    if (!c) LUMEN_FAIL(LUMEN_ERR_INVALID, "kv_cache_reset: null");
+    c->len = 0;  // self_attention.rs:41-43
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_kv_cache_len(const lumen_kv_cache *c, int *len_out) {
+    if (!c || !len_out) LUMEN_FAIL(LUMEN_ERR_INVALID, "kv_cache_len: null");
+    *len_out = c->len;
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_kv_cache_ptrs(const lumen_kv_cache *c, float **k_out, float **v_out) {
+    if (!c || !k_out || !v_out) LUMEN_FAIL(LUMEN_ERR_INVALID, "kv_cache_ptrs: null");
+    *k_out = c->k;
+    *v_out = c->v;
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_kv_cache_update(lumen_kv_cache *c, const float *k, const float *v, int s, int start_pos) {
+    if (!c || !k || !v) LUMEN_FAIL(LUMEN_ERR_INVALID, "kv_cache_update: null");
+    if (s < 0 || start_pos < 0) LUMEN_FAIL(LUMEN_ERR_SHAPE, "kv_cache_update: negative argument");
+    if (start_pos + s > c->max_seq)  // kv_cache.rs:33-36
+        LUMEN_FAIL(LUMEN_ERR_KV_OVERFLOW, "KV Cache overflow! Max: %d, Current: %d", c->max_seq, start_pos + s);
+    const size_t n = (size_t)c->b * c->h_kv * s * c->d;
+    if (!n) return LUMEN_OK;
+    hipLaunchKernelGGL(kv_update_kernel, dim3(ew_blocks(c->ctx, n)), dim3(256), 0, c->ctx->stream, k, c->k, s, c->d,
+                       c->max_seq, start_pos, n);
+    hipLaunchKernelGGL(kv_update_kernel, dim3(ew_blocks(c->ctx, n)), dim3(256), 0, c->ctx->stream, v, c->v, s, c->d,
+                       c->max_seq, start_pos, n);
+    LUMEN_CHECK_LAUNCH();
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_kv_cache_get_view(const lumen_kv_cache *c, int cur, float *k_out, float *v_out) {
+    if (!c || !k_out || !v_out) LUMEN_FAIL(LUMEN_ERR_INVALID, "kv_cache_get_view: null");
+    if (cur < 0 || cur > c->max_seq) LUMEN_FAIL(LUMEN_ERR_SHAPE, "kv_cache_get_view: current_len %d outside [0,%d]", cur, c->max_seq);
+    const size_t n = (size_t)c->b * c->h_kv * cur * c->d;
+    if (!n) return LUMEN_OK;
+    hipLaunchKernelGGL(kv_view_kernel, dim3(ew_blocks(c->ctx, n)), dim3(256), 0, c->ctx->stream, c->k, k_out, cur, c->d,
+                       c->max_seq, n);
+    hipLaunchKernelGGL(kv_view_kernel, dim3(ew_blocks(c->ctx, n)), dim3(256), 0, c->ctx->stream, c->v, v_out, cur, c->d,
+                       c->max_seq, n);
+    LUMEN_CHECK_LAUNCH();
+    return LUMEN_OK;
+}
+
+static int ensure_split_scratch(lumen_kv_cache *c, int hq, int nsplit) {
+    if (c->part && c->part_heads >= hq) return LUMEN_OK;
+    hipStreamSynchronize(c->ctx->stream);
+    hipFree(c->part);
+    hipFree(c->counters);
+    c->part = nullptr;
+    c->counters = nullptr;
+    HIP_TRY(hipMalloc((void **)&c->part, sizeof(float) * attn_decode_part_floats(c->b, hq, c->d, nsplit)));
+    HIP_TRY(hipMalloc((void **)&c->counters, sizeof(int) * (size_t)c->b * c->h_kv));
+    HIP_TRY(hipMemsetAsync(c->counters, 0, sizeof(int) * (size_t)c->b * c->h_kv, c->ctx->stream));
+    c->part_heads = hq;
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_attn_decode_f32(lumen_kv_cache *c, lumen_rope *rope, const float *q3, const float *k3,
+                                     const float *v3, float *out, int h, float scale, int causal) {
+    (void)causal;  // the causal test `j > past_len` never fires for S == 1 (self_attention.rs:256)
+    if (!c || !rope || !q3 || !k3 || !v3 || !out) LUMEN_FAIL(LUMEN_ERR_INVALID, "attn_decode: null argument");
+    if (rope->dim != c->d) LUMEN_FAIL(LUMEN_ERR_SHAPE, "RoPE dimension mismatch: %d vs head_dim %d", rope->dim, c->d);
+    if (h <= 0 || h % c->h_kv) LUMEN_FAIL(LUMEN_ERR_SHAPE, "attn_decode: %d heads over %d kv heads", h, c->h_kv);
+    const int past_len = c->len, new_len = past_len + 1;
+    if (new_len > c->max_seq)  // self_attention.rs:144-149
+        LUMEN_FAIL(LUMEN_ERR_KV_OVERFLOW, "KV cache overflow: new_len=%d > max_seq=%d", new_len, c->max_seq);
+    if (past_len >= rope->max_seq)  // encoding.rs:176-181
+        LUMEN_FAIL(LUMEN_ERR_ROPE_RANGE, "RoPE index out of range: pos %d >= max %d", past_len, rope->max_seq);
+    const int nsplit = attn_decode_nsplit(c->max_seq);
+    LUMEN_TRY(ensure_split_scratch(c, h, nsplit));
+    AttnDecodeArgs a = {};
+    a.q = q3; a.k_new = k3; a.v_new = v3; a.out = out;
+    a.k_cache = c->k; a.v_cache = c->v; a.cos_t = rope->cos_dev; a.sin_t = rope->sin_dev;
+    a.pos_dev = nullptr; a.pos_host = past_len;
+    a.b = c->b; a.hq = h; a.hkv = c->h_kv; a.d = c->d; a.max_seq = c->max_seq; a.scale = scale;
+    a.q_norm_w = nullptr; a.k_norm_w = nullptr; a.norm_eps = 0.f;
+    a.part = c->part; a.counters = c->counters; a.nsplit = nsplit;
+    LUMEN_TRY(launch_attn_decode(c->ctx, a));
+    c->len = new_len;
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_attn_prefill_f32(lumen_kv_cache *c, lumen_rope *rope, const float *q, const float *k,
+                                      const float *v, float *out, int s, int h, float scale, int causal) {
+    if (!c || !rope || !q || !k || !v || !out) LUMEN_FAIL(LUMEN_ERR_INVALID, "attn_prefill: null argument");
+    if (rope->dim != c->d) LUMEN_FAIL(LUMEN_ERR_SHAPE, "RoPE dimension mismatch: %d vs head_dim %d", rope->dim, c->d);
+    if (h <= 0 || h % c->h_kv || s < 0) LUMEN_FAIL(LUMEN_ERR_SHAPE, "attn_prefill: s=%d, %d heads over %d kv heads", s, h, c->h_kv);
+    const int past_len = c->len, new_len = past_len + s;
+    if (past_len + s > rope->max_seq)  // encoding.rs:62-68
+        LUMEN_FAIL(LUMEN_ERR_ROPE_RANGE, "RoPE index out of range: offset %d + len %d > max %d", past_len, s, rope->max_seq);
+    if (new_len > c->max_seq)  // self_attention.rs:341-346
+        LUMEN_FAIL(LUMEN_ERR_KV_OVERFLOW, "KV cache overflow: new_len=%d > max_seq=%d", new_len, c->max_seq);
+    if (s == 0) return LUMEN_OK;
+    float *q_rot = nullptr;
+    HIP_TRY(hipMalloc((void **)&q_rot, sizeof(float) * (size_t)c->b * s * h * c->d));
+    AttnPrefillArgs a = {};
+    a.q = q; a.k = k; a.v = v; a.out = out; a.k_cache = c->k; a.v_cache = c->v;
+    a.cos_t = rope->cos_dev; a.sin_t = rope->sin_dev;
+    a.b = c->b; a.s = s; a.hq = h; a.hkv = c->h_kv; a.d = c->d; a.max_seq = c->max_seq; a.past_len = past_len;
+    a.q_stride = h * c->d; a.k_stride = c->h_kv * c->d; a.v_stride = c->h_kv * c->d;
+    a.scale = scale; a.causal = causal; a.q_rot = q_rot;
+    int rc = launch_attn_prefill(c->ctx, a);
+    hipStreamSynchronize(c->ctx->stream);
+    hipFree(q_rot);
+    if (rc == LUMEN_OK) c->len = new_len;
+    return rc;
+}

@@ -1,0 +1,112 @@
+// Context, device memory, stopwatch and error reporting of liblumen_hip.so.
+#include "internal.h"
+
+#include <cstring>
+
+static thread_local char g_err[512] = "";
+
+void lumen_set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+extern "C" const char *lumen_last_error(void) { return g_err; }
+
+extern "C" const char *lumen_version(void) { return "lumen-hip 0.1 (gfx950)"; }
+
+extern "C" int lumen_ctx_create(int device, lumen_ctx **out) {
+    if (!out) LUMEN_FAIL(LUMEN_ERR_INVALID, "lumen_ctx_create: out is null");
+    *out = nullptr;
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= 0)
+        LUMEN_FAIL(LUMEN_ERR_NO_DEVICE, "no HIP device visible (%s)", hipGetErrorString(e));
+    if (device < 0 || device >= n) LUMEN_FAIL(LUMEN_ERR_INVALID, "device %d out of range [0,%d)", device, n);
+    HIP_TRY(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        LUMEN_FAIL(LUMEN_ERR_NO_DEVICE, "device %d is %s; this library is built for gfx950 only", device,
+                   prop.gcnArchName);
+    lumen_ctx *c = new lumen_ctx();
+    c->device = device;
+    c->num_cus = prop.multiProcessorCount;
+    HIP_TRY(hipStreamCreateWithFlags(&c->own_stream, hipStreamNonBlocking));
+    c->stream = c->own_stream;
+    HIP_TRY(hipEventCreate(&c->ev0));
+    HIP_TRY(hipEventCreate(&c->ev1));
+    HIP_TRY(hipMalloc((void **)&c->d_scratch_int, 64 * sizeof(int)));
+    *out = c;
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_ctx_destroy(lumen_ctx *ctx) {
+    if (!ctx) return LUMEN_OK;
+    hipSetDevice(ctx->device);
+    hipStreamSynchronize(ctx->stream);
+    hipFree(ctx->d_scratch_int);
+    hipEventDestroy(ctx->ev0);
+    hipEventDestroy(ctx->ev1);
+    hipStreamDestroy(ctx->own_stream);
+    delete ctx;
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_ctx_set_stream(lumen_ctx *ctx, void *hip_stream) {
+    if (!ctx) LUMEN_FAIL(LUMEN_ERR_INVALID, "ctx is null");
+    ctx->stream = hip_stream ? (hipStream_t)hip_stream : ctx->own_stream;
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_ctx_synchronize(lumen_ctx *ctx) {
+    if (!ctx) LUMEN_FAIL(LUMEN_ERR_INVALID, "ctx is null");
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_timer_start(lumen_ctx *ctx) {
+    if (!ctx) LUMEN_FAIL(LUMEN_ERR_INVALID, "ctx is null");
+    HIP_TRY(hipEventRecord(ctx->ev0, ctx->stream));
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_timer_stop(lumen_ctx *ctx, float *ms_out) {
+    if (!ctx || !ms_out) LUMEN_FAIL(LUMEN_ERR_INVALID, "null argument");
+    HIP_TRY(hipEventRecord(ctx->ev1, ctx->stream));
+    HIP_TRY(hipEventSynchronize(ctx->ev1));
+    HIP_TRY(hipEventElapsedTime(ms_out, ctx->ev0, ctx->ev1));
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_malloc(lumen_ctx *ctx, size_t bytes, void **dev_out) {
+    if (!ctx || !dev_out) LUMEN_FAIL(LUMEN_ERR_INVALID, "null argument");
+    HIP_TRY(hipSetDevice(ctx->device));
+    HIP_TRY(hipMalloc(dev_out, bytes ? bytes : 16));
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_free(lumen_ctx *ctx, void *dev) {
+    if (!ctx) LUMEN_FAIL(LUMEN_ERR_INVALID, "ctx is null");
+    if (!dev) return LUMEN_OK;
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    HIP_TRY(hipFree(dev));
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_upload(lumen_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes) {
+    if (!ctx || (bytes && (!dst_dev || !src_host))) LUMEN_FAIL(LUMEN_ERR_INVALID, "null argument");
+    if (!bytes) return LUMEN_OK;
+    HIP_TRY(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, ctx->stream));
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_download(lumen_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes) {
+    if (!ctx || (bytes && (!dst_host || !src_dev))) LUMEN_FAIL(LUMEN_ERR_INVALID, "null argument");
+    if (!bytes) return LUMEN_OK;
+    HIP_TRY(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return LUMEN_OK;
+}

@@ -1,0 +1,280 @@
+// Memory-bound vector-matrix product y = W x for the M == 1 branch of
+// ops::matmul::matmul (src/ops/matmul.rs:42-69), W [N, K] row-major f32 or
+// bf16 bits, x and y f32, f32 accumulation.
+//
+// Mapping: x is staged once per workgroup in LDS (optionally RMS-normalised
+// on the way in).  One 64-lane wavefront owns R whole rows at a time; each
+// lane streams 16-byte pieces of the rows (a wavefront covers 1 KiB of a row
+// per load instruction, fully coalesced), multiplies them with its slice of x
+// from LDS and the 64 partial sums are folded with cross-lane shuffles.  The
+// row loop keeps 8 independent 16-byte loads per lane in flight.
+#include "internal.h"
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+
+#define GEMV_THREADS 256
+#define GEMV_WAVES (GEMV_THREADS / 64)
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+__device__ __forceinline__ float silu_f(float g) {
+    // x * (1 / (1 + exp(-x))), src/layers/activation.rs:143-146
+    float sig = 1.0f / (1.0f + expf(-g));
+    return g * sig;
+}
+
+// 16 bytes of weights times the matching slice of x
+template <bool BF16>
+__device__ __forceinline__ float dot16(const v4u raw, const float *xs) {
+    if (BF16) {
+        // eight bf16 values; widening is a 16-bit shift (src/loader.rs:58)
+        const v4f xa = *(const v4f *)xs;
+        const v4f xb = *(const v4f *)(xs + 4);
+        float s = __uint_as_float(raw.x << 16) * xa.x;
+        s = fmaf(__uint_as_float(raw.x & 0xffff0000u), xa.y, s);
+        s = fmaf(__uint_as_float(raw.y << 16), xa.z, s);
+        s = fmaf(__uint_as_float(raw.y & 0xffff0000u), xa.w, s);
+        s = fmaf(__uint_as_float(raw.z << 16), xb.x, s);
+        s = fmaf(__uint_as_float(raw.z & 0xffff0000u), xb.y, s);
+        s = fmaf(__uint_as_float(raw.w << 16), xb.z, s);
+        s = fmaf(__uint_as_float(raw.w & 0xffff0000u), xb.w, s);
+        return s;
+    } else {
+        const v4f xa = *(const v4f *)xs;
+        float s = __uint_as_float(raw.x) * xa.x;
+        s = fmaf(__uint_as_float(raw.y), xa.y, s);
+        s = fmaf(__uint_as_float(raw.z), xa.z, s);
+        s = fmaf(__uint_as_float(raw.w), xa.w, s);
+        return s;
+    }
+}
+
+// Stages x (optionally RMS-normalised: (x * inv_rms) * g, src/layers/norm/rms_norm.rs:45-58)
+// into LDS, zero-padded to kpad.  All threads of the workgroup must call it.
+template <int PRO>
+__device__ __forceinline__ void stage_x(float *xs, const float *__restrict__ x, const float *__restrict__ g,
+                                        float eps, int K, int kpad) {
+    __shared__ float red[GEMV_WAVES];
+    const int tid = threadIdx.x;
+    float inv = 1.0f;
+    if (PRO == PRO_RMSNORM) {
+        float ss = 0.f;
+        for (int k = tid * 4; k < K; k += GEMV_THREADS * 4) {
+            const v4f v = *(const v4f *)(x + k);
+            ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+        }
+        ss = wave_sum(ss);
+        if ((tid & 63) == 0) red[tid >> 6] = ss;
+        __syncthreads();
+        float tot = 0.f;
+#pragma unroll
+        for (int w = 0; w < GEMV_WAVES; ++w) tot += red[w];
+        const float rms = sqrtf(tot / (float)K + eps);
+        inv = 1.0f / rms;
+    }
+    for (int k = tid * 4; k < kpad; k += GEMV_THREADS * 4) {
+        v4f v = {0.f, 0.f, 0.f, 0.f};
+        if (k < K) {
+            v = *(const v4f *)(x + k);
+            if (PRO == PRO_RMSNORM) {
+                const v4f gg = *(const v4f *)(g + k);
+                v.x = v.x * inv * gg.x;
+                v.y = v.y * inv * gg.y;
+                v.z = v.z * inv * gg.z;
+                v.w = v.w * inv * gg.w;
+            }
+        }
+        *(v4f *)(xs + k) = v;
+    }
+    __syncthreads();
+}
+
+template <bool BF16, int R, int PRO, int EPI>
+__global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(GemvArgs a) {
+    extern __shared__ __align__(16) float xs[];
+    constexpr int VEC = BF16 ? 8 : 4;          // elements per 16-byte load
+    constexpr int SWEEP = 64 * VEC;            // elements one wavefront covers per load
+    constexpr int U = 8 / R;                   // loads in flight per lane per row
+    constexpr int ESZ = BF16 ? 2 : 4;
+    const int K = a.K, N = a.N;
+    const int kpad = (K + SWEEP - 1) / SWEEP * SWEEP;
+
+    stage_x<PRO>(xs, a.x, a.norm_w, a.eps, K, kpad);
+
+    const int lane = threadIdx.x & 63;
+    const int gw = blockIdx.x * GEMV_WAVES + (threadIdx.x >> 6);
+    const int nw = gridDim.x * GEMV_WAVES;
+    const int nunits = (N + R - 1) / R;
+    const char *Wb = (const char *)a.W;
+    const size_t row_bytes = (size_t)K * ESZ;
+
+    for (int u = gw; u < nunits; u += nw) {
+        const char *wp[R];
+        float acc[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            int row = u * R + r;
+            if (row >= N) row = N - 1;  // odd N with R == 2: result discarded below
+            wp[r] = Wb + (size_t)row * row_bytes + (size_t)lane * 16;
+            acc[r] = 0.f;
+        }
+        for (int k0 = 0; k0 < K; k0 += SWEEP * U) {
+            v4u raw[R][U];
+#pragma unroll
+            for (int uu = 0; uu < U; ++uu) {
+                const int kk = k0 + uu * SWEEP + lane * VEC;
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    raw[r][uu] = (v4u){0u, 0u, 0u, 0u};
+                    if (kk < K)
+                        raw[r][uu] = __builtin_nontemporal_load((const v4u *)(wp[r] + (size_t)(k0 + uu * SWEEP) * ESZ));
+                }
+            }
+#pragma unroll
+            for (int uu = 0; uu < U; ++uu) {
+                const int kk = k0 + uu * SWEEP + lane * VEC;
+                if (kk < kpad) {
+#pragma unroll
+                    for (int r = 0; r < R; ++r) acc[r] += dot16<BF16>(raw[r][uu], xs + kk);
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
+        if (lane == 0) {
+            if (EPI == EPI_SWIGLU) {
+                // rows (2u, 2u+1) hold (gate_u, up_u): silu(gate) * up, src/models/llama.rs:60-63
+                a.y[u] = silu_f(acc[0]) * acc[R - 1];
+            } else {
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const int row = u * R + r;
+                    if (row < N) {
+                        // residual: x + y, src/ops/arithmetic.rs:48-51 via src/models/llama.rs:110,115
+                        a.y[row] = (EPI == EPI_RESIDUAL) ? a.residual[row] + acc[r] : acc[r];
+                    }
+                }
+            }
+        }
+    }
+}
+
+// Any K, any alignment: one wavefront per row, scalar loads, x from global memory.
+template <bool BF16>
+__global__ __launch_bounds__(GEMV_THREADS) void gemv_generic_kernel(GemvArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int gw = blockIdx.x * GEMV_WAVES + (threadIdx.x >> 6);
+    const int nw = gridDim.x * GEMV_WAVES;
+    for (int row = gw; row < a.N; row += nw) {
+        float acc = 0.f;
+        for (int k = lane; k < a.K; k += 64) {
+            float w;
+            if (BF16)
+                w = __uint_as_float((unsigned int)((const uint16_t *)a.W)[(size_t)row * a.K + k] << 16);
+            else
+                w = ((const float *)a.W)[(size_t)row * a.K + k];
+            acc = fmaf(w, a.x[k], acc);
+        }
+        acc = wave_sum(acc);
+        if (lane == 0) a.y[row] = acc;
+    }
+}
+
+template <bool BF16, int R, int PRO>
+static void launch_epi(const GemvArgs &a, dim3 grid, size_t lds, hipStream_t s) {
+    switch (a.epi) {
+        case EPI_STORE:
+            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_STORE>), grid, dim3(GEMV_THREADS), lds, s, a);
+            break;
+        case EPI_RESIDUAL:
+            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_RESIDUAL>), grid, dim3(GEMV_THREADS), lds, s, a);
+            break;
+        default:
+            hipLaunchKernelGGL((gemv_kernel<BF16, 2, PRO, EPI_SWIGLU>), grid, dim3(GEMV_THREADS), lds, s, a);
+            break;
+    }
+}
+
+template <bool BF16, int R>
+static void launch_pro(const GemvArgs &a, dim3 grid, size_t lds, hipStream_t s) {
+    if (a.pro == PRO_RMSNORM)
+        launch_epi<BF16, R, PRO_RMSNORM>(a, grid, lds, s);
+    else
+        launch_epi<BF16, R, PRO_NONE>(a, grid, lds, s);
+}
+
+int launch_gemv(lumen_ctx *ctx, const GemvArgs &a) {
+    if (a.N <= 0 || a.K <= 0) return LUMEN_OK;
+    const int vec = a.w_bf16 ? 8 : 4;
+    const int sweep = 64 * vec;
+    const int kpad = (a.K + sweep - 1) / sweep * sweep;
+    const size_t lds = (size_t)kpad * sizeof(float);
+    const bool aligned = (((uintptr_t)a.W | (uintptr_t)a.x) & 15) == 0 &&
+                         (a.pro != PRO_RMSNORM || ((uintptr_t)a.norm_w & 15) == 0);
+    const bool fast = (a.K % vec == 0) && aligned && lds <= 64 * 1024;
+    if (!fast) {
+        if (a.pro != PRO_NONE || a.epi != EPI_STORE)
+            LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "fused GEMV needs K %% %d == 0, 16-byte alignment and K <= %d (K=%d)", vec,
+                       16384, a.K);
+        int blocks = (a.N + GEMV_WAVES - 1) / GEMV_WAVES;
+        if (blocks > ctx->num_cus * 8) blocks = ctx->num_cus * 8;
+        if (a.w_bf16)
+            hipLaunchKernelGGL(gemv_generic_kernel<true>, dim3(blocks), dim3(GEMV_THREADS), 0, ctx->stream, a);
+        else
+            hipLaunchKernelGGL(gemv_generic_kernel<false>, dim3(blocks), dim3(GEMV_THREADS), 0, ctx->stream, a);
+        LUMEN_CHECK_LAUNCH();
+        return LUMEN_OK;
+    }
+    if (a.epi == EPI_SWIGLU && (a.N & 1)) LUMEN_FAIL(LUMEN_ERR_SHAPE, "SwiGLU epilogue needs an even row count, got %d", a.N);
+    const int R = (a.epi == EPI_SWIGLU || a.N >= 8192) ? 2 : 1;
+    const int nunits = (a.N + R - 1) / R;
+    int blocks = (nunits + GEMV_WAVES - 1) / GEMV_WAVES;
+    const int cap = ctx->num_cus * 4;
+    if (blocks > cap) blocks = cap;
+    dim3 grid(blocks);
+    if (a.w_bf16) {
+        if (R == 2) launch_pro<true, 2>(a, grid, lds, ctx->stream);
+        else launch_pro<true, 1>(a, grid, lds, ctx->stream);
+    } else {
+        if (R == 2) launch_pro<false, 2>(a, grid, lds, ctx->stream);
+        else launch_pro<false, 1>(a, grid, lds, ctx->stream);
+    }
+    LUMEN_CHECK_LAUNCH();
+    return LUMEN_OK;
+}
+
+// --------------------------------------------------------------------- C ABI
+static int check_gemv(lumen_ctx *ctx, const void *W, const float *x, float *y, int N, int K) {
+    if (!ctx || !W || !x || !y) LUMEN_FAIL(LUMEN_ERR_INVALID, "gemv: null argument");
+    if (N < 0 || K < 0) LUMEN_FAIL(LUMEN_ERR_SHAPE, "gemv: negative dimension N=%d K=%d", N, K);
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_gemv_f32(lumen_ctx *ctx, const float *W, const float *x, float *y, int N, int K) {
+    LUMEN_TRY(check_gemv(ctx, W, x, y, N, K));
+    GemvArgs a = {};
+    a.W = W; a.x = x; a.y = y; a.N = N; a.K = K; a.w_bf16 = 0; a.pro = PRO_NONE; a.epi = EPI_STORE;
+    return launch_gemv(ctx, a);
+}
+
+extern "C" int lumen_gemv_bf16w(lumen_ctx *ctx, const uint16_t *W, const float *x, float *y, int N, int K) {
+    LUMEN_TRY(check_gemv(ctx, W, x, y, N, K));
+    GemvArgs a = {};
+    a.W = W; a.x = x; a.y = y; a.N = N; a.K = K; a.w_bf16 = 1; a.pro = PRO_NONE; a.epi = EPI_STORE;
+    return launch_gemv(ctx, a);
+}
+
+extern "C" int lumen_matmul_f32(lumen_ctx *ctx, const float *A, const float *W, float *C, int M, int N, int K_a,
+                                int K_w) {
+    if (!ctx || !A || !W || !C) LUMEN_FAIL(LUMEN_ERR_INVALID, "matmul: null argument");
+    if (K_a != K_w)  // src/ops/matmul.rs:33-38
+        LUMEN_FAIL(LUMEN_ERR_SHAPE, "MatMul shape mismatch: a (K=%d) vs b (K=%d)", K_a, K_w);
+    if (M < 0 || N < 0 || K_a < 0) LUMEN_FAIL(LUMEN_ERR_SHAPE, "matmul: negative dimension");
+    if (M == 1) return lumen_gemv_f32(ctx, W, A, C, N, K_a);  // src/ops/matmul.rs:42
+    return lumen_gemm_f32(ctx, A, W, C, M, N, K_a);
+}

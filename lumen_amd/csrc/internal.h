@@ -1,0 +1,152 @@
+// Internal declarations shared by the translation units of liblumen_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <string>
+#include <vector>
+
+#include "../../include/lumen_hip.h"
+
+// ---------------------------------------------------------------- errors
+void lumen_set_error(const char *fmt, ...);
+
+#define LUMEN_FAIL(code, ...)           \
+    do {                                \
+        lumen_set_error(__VA_ARGS__);   \
+        return (code);                  \
+    } while (0)
+
+#define HIP_TRY(expr)                                                                      \
+    do {                                                                                   \
+        hipError_t e_ = (expr);                                                            \
+        if (e_ != hipSuccess)                                                              \
+            LUMEN_FAIL(LUMEN_ERR_HIP, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), \
+                       __FILE__, __LINE__);                                                \
+    } while (0)
+
+#define LUMEN_TRY(expr)              \
+    do {                             \
+        int rc_ = (expr);            \
+        if (rc_ != LUMEN_OK) return rc_; \
+    } while (0)
+
+#define LUMEN_CHECK_LAUNCH() HIP_TRY(hipGetLastError())
+
+// ---------------------------------------------------------------- objects
+struct lumen_ctx {
+    int device = 0;
+    int num_cus = 0;
+    hipStream_t own_stream = nullptr;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    int *d_scratch_int = nullptr;  // small device scratch (argmax result etc.)
+};
+
+struct lumen_rope {
+    lumen_ctx *ctx = nullptr;
+    int dim = 0, max_seq = 0;
+    float theta = 0.f;
+    float *cos_dev = nullptr, *sin_dev = nullptr;  // [max_seq, dim]
+    std::vector<float> cos_host, sin_host;
+};
+
+struct lumen_kv_cache {
+    lumen_ctx *ctx = nullptr;
+    int b = 0, h_kv = 0, max_seq = 0, d = 0;
+    int len = 0;            // host mirror of the position counter
+    float *k = nullptr, *v = nullptr;
+    bool owns = true;       // false when k/v are slices of a model-wide slab
+    // decode-attention split-L scratch
+    float *part = nullptr;  // [b*h_q_max, nsplit, d + 2]
+    int *counters = nullptr;
+    int part_heads = 0;
+};
+
+// ---------------------------------------------------------------- launchers
+// Every launcher validates nothing: callers check shapes first.
+
+enum GemvPro { PRO_NONE = 0, PRO_RMSNORM = 1 };
+enum GemvEpi { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2 };
+
+struct GemvArgs {
+    const void *W;        // [N, K] f32 or bf16 bits
+    const float *x;       // [K]
+    float *y;             // [N] (EPI_SWIGLU: [N/2])
+    int N, K;
+    int w_bf16;
+    int pro, epi;
+    const float *norm_w;  // PRO_RMSNORM: gain [K]
+    float eps;
+    const float *residual;  // EPI_RESIDUAL: [N]
+};
+int launch_gemv(lumen_ctx *ctx, const GemvArgs &a);
+
+struct GemmArgs {
+    const float *A;   // [M, K]
+    const void *W;    // [N, K]
+    float *C;         // [M, N] (EPI_SWIGLU: [M, N/2])
+    int M, N, K;
+    int w_bf16;
+    int epi;
+    const float *residual;  // [M, N]
+};
+int launch_gemm(lumen_ctx *ctx, const GemmArgs &a);
+
+int launch_rmsnorm(lumen_ctx *ctx, const float *x, const float *w, float *out, int rows, int dim, float eps);
+int launch_silu(lumen_ctx *ctx, const float *x, float *out, size_t n);
+int launch_add(lumen_ctx *ctx, const float *a, const float *b, float *out, size_t n);
+int launch_mul(lumen_ctx *ctx, const float *a, const float *b, float *out, size_t n);
+int launch_swiglu(lumen_ctx *ctx, const float *g, const float *u, float *out, size_t n);
+// ids_dev int32 [n]; out [n, dim]
+int launch_embedding(lumen_ctx *ctx, const float *W, const int *ids_dev, int n, int dim, int vocab, float *out);
+// writes the index of the first maximum to *out_dev; if next_id/pos are given
+// (device ints) also stores the index there and increments *pos by one
+int launch_argmax(lumen_ctx *ctx, const float *x, int n, int *out_dev, int *pos_inc_dev);
+// x, out [B, H, S, D], positions offset..offset+S-1
+int launch_rope_bhsd(lumen_ctx *ctx, const float *x, float *out, const float *cos_t, const float *sin_t,
+                     int b, int h, int s, int d, int offset);
+
+struct AttnDecodeArgs {
+    const float *q;     // [B, Hq, D] un-rotated (row stride q_stride floats per batch)
+    const float *k_new; // [B, Hkv, D] un-rotated
+    const float *v_new; // [B, Hkv, D]
+    float *out;         // [B, Hq, D]
+    float *k_cache, *v_cache;  // [B, Hkv, max_seq, D]
+    const float *cos_t, *sin_t;
+    const int *pos_dev; // device int: position of the new token (== past_len), or null
+    int pos_host;       // used when pos_dev is null
+    int b, hq, hkv, d, max_seq;
+    float scale;
+    const float *q_norm_w, *k_norm_w;  // per-head RMSNorm gains [D] or null
+    float norm_eps;
+    float *part;        // split scratch
+    int *counters;
+    int nsplit;
+};
+int launch_attn_decode(lumen_ctx *ctx, const AttnDecodeArgs &a);
+
+struct AttnPrefillArgs {
+    const float *q;  // [B, S, Hq, D] un-rotated
+    const float *k;  // [B, S, Hkv, D] un-rotated
+    const float *v;  // [B, S, Hkv, D]
+    float *out;      // [B, S, Hq, D]
+    float *k_cache, *v_cache;
+    const float *cos_t, *sin_t;
+    int b, s, hq, hkv, d, max_seq, past_len;
+    int q_stride, k_stride, v_stride;  // floats between consecutive positions
+    float scale;
+    int causal;
+    const float *q_norm_w, *k_norm_w;
+    float norm_eps;
+    float *q_rot;    // scratch [B, S, Hq, D]
+};
+int launch_attn_prefill(lumen_ctx *ctx, const AttnPrefillArgs &a);
+
+int attn_decode_nsplit(int max_seq);
+size_t attn_decode_part_floats(int b, int hq, int d, int nsplit);
+
+void rope_tables_host(std::vector<float> &cos_t, std::vector<float> &sin_t, int dim, int max_seq, float theta);

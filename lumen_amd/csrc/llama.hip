@@ -1,0 +1,577 @@
+// LlamaModel on one GPU: src/models/llama.rs:129-280.
+//
+// Everything a decode step touches is allocated once at create time: the
+// weights (q|k|v rows concatenated, gate/up rows interleaved so that their
+// GEMVs run as one launch each), one KV slab for all layers, the activation
+// vectors, the token id and the position counter.  A decode step is a fixed
+// sequence of 5 kernels per layer that reads the token id and position from
+// device memory, so the whole step is captured once as a HIP graph and
+// replayed per token; greedy generation never returns to the host between
+// tokens.
+#include "internal.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <string>
+
+struct LayerW {
+    void *wqkv = nullptr, *wo = nullptr, *wgu = nullptr, *wdown = nullptr;  // weight dtype
+    float *in_norm = nullptr, *post_norm = nullptr, *q_norm = nullptr, *k_norm = nullptr;
+};
+
+struct lumen_llama {
+    lumen_ctx *ctx = nullptr;
+    lumen_llama_config cfg = {};
+    int D = 0, qd = 0, kvd = 0, qkvd = 0;
+    bool bf16 = false;
+    size_t esz = 4;
+    float scale = 0.f;
+    float *embed = nullptr;    // [V,H] f32 (bf16 sources are widened: same values)
+    void *lm_head = nullptr;   // [V,H] weight dtype; aliases embed when tied and f32
+    bool lm_head_owned = false;
+    float *final_norm = nullptr;
+    std::vector<LayerW> layers;
+    float *cos_dev = nullptr, *sin_dev = nullptr;
+    float *k_slab = nullptr, *v_slab = nullptr;  // [layers][1][Hkv][max_seq][D]
+    size_t cache_stride = 0;
+    int len = 0;  // host mirror of *d_pos
+    // decode state
+    float *x = nullptr, *h = nullptr, *qkv = nullptr, *attn = nullptr, *act = nullptr, *logits = nullptr;
+    int *d_tok = nullptr, *d_pos = nullptr;
+    float *part = nullptr;
+    int *counters = nullptr;
+    int nsplit = 1;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t graph_exec = nullptr;
+    // prefill buffers (grown on demand, kept)
+    int pf_cap = 0, pf_logit_cap = 0;
+    float *p_x = nullptr, *p_h = nullptr, *p_n = nullptr, *p_qkv = nullptr, *p_qrot = nullptr, *p_attn = nullptr,
+          *p_act = nullptr, *p_logits = nullptr;
+    int *p_ids = nullptr;
+    std::vector<void *> allocs;
+};
+
+static int dmalloc(lumen_llama *m, void **p, size_t bytes) {
+    HIP_TRY(hipMalloc(p, bytes ? bytes : 16));
+    m->allocs.push_back(*p);
+    return LUMEN_OK;
+}
+
+template <typename T>
+static int dmalloc_t(lumen_llama *m, T **p, size_t count) { return dmalloc(m, (void **)p, count * sizeof(T)); }
+
+static int fill_ones(lumen_llama *m, float *dst, size_t n) {
+    std::vector<float> ones(n, 1.0f);
+    return lumen_upload(m->ctx, dst, ones.data(), n * sizeof(float));
+}
+
+extern "C" int lumen_llama_destroy(lumen_llama *m) {
+    if (!m) return LUMEN_OK;
+    hipStreamSynchronize(m->ctx->stream);
+    if (m->graph_exec) hipGraphExecDestroy(m->graph_exec);
+    if (m->graph) hipGraphDestroy(m->graph);
+    for (void *p : m->allocs) hipFree(p);
+    hipFree(m->p_x); hipFree(m->p_h); hipFree(m->p_n); hipFree(m->p_qkv); hipFree(m->p_qrot);
+    hipFree(m->p_attn); hipFree(m->p_act); hipFree(m->p_logits); hipFree(m->p_ids);
+    delete m;
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg, lumen_llama **out) {
+    if (!ctx || !cfg || !out) LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_create: null argument");
+    *out = nullptr;
+    const int H = cfg->hidden_size, I = cfg->intermediate_size, V = cfg->vocab_size, L = cfg->num_hidden_layers;
+    const int Hq = cfg->num_attention_heads, Hkv = cfg->num_key_value_heads;
+    if (H <= 0 || I <= 0 || V <= 0 || L <= 0 || Hq <= 0 || Hkv <= 0 || cfg->max_seq_len <= 0)
+        LUMEN_FAIL(LUMEN_ERR_SHAPE, "llama_create: non-positive dimension");
+    if (cfg->head_dim == 0 && H % Hq)  // self_attention.rs:69-73
+        LUMEN_FAIL(LUMEN_ERR_SHAPE, "Embed dim must be divisible by n_head (%d %% %d)", H, Hq);
+    if (Hq % Hkv) LUMEN_FAIL(LUMEN_ERR_SHAPE, "n_head %d not a multiple of n_kv_head %d", Hq, Hkv);
+    if (cfg->weight_dtype != LUMEN_DTYPE_F32 && cfg->weight_dtype != LUMEN_DTYPE_BF16)
+        LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_create: weight_dtype %d", cfg->weight_dtype);
+    const int D = cfg->head_dim > 0 ? cfg->head_dim : H / Hq;
+    const int nrep = Hq / Hkv;
+    if (!(D == 16 || D == 32 || D == 64 || D == 128) || !(nrep == 1 || nrep == 2 || nrep == 4 || nrep == 8))
+        LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "head_dim %d / n_rep %d outside the attention kernels (16..128, 1..8)", D, nrep);
+    if (H % 8 || I % 8 || (Hq * D) % 8)
+        LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "hidden %d, intermediate %d and n_head*head_dim %d must be multiples of 8", H, I, Hq * D);
+    if (H > 16384 || I > 16384 || Hq * D > 16384)
+        LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "inner dimensions above 16384 do not fit the GEMV's LDS stage");
+    HIP_TRY(hipSetDevice(ctx->device));
+
+    lumen_llama *m = new lumen_llama();
+    m->ctx = ctx; m->cfg = *cfg; m->D = D; m->qd = Hq * D; m->kvd = Hkv * D; m->qkvd = m->qd + 2 * m->kvd;
+    m->bf16 = cfg->weight_dtype == LUMEN_DTYPE_BF16;
+    m->esz = m->bf16 ? 2 : 4;
+    m->scale = 1.0f / sqrtf((float)D);  // self_attention.rs:89 (sqrt().recip())
+    m->layers.resize(L);
+    int rc = LUMEN_OK;
+#define M_TRY(e) do { rc = (e); if (rc != LUMEN_OK) { lumen_llama_destroy(m); return rc; } } while (0)
+    M_TRY(dmalloc_t(m, &m->embed, (size_t)V * H));
+    if (cfg->tie_embeddings && !m->bf16) {
+        m->lm_head = m->embed;
+    } else {
+        M_TRY(dmalloc(m, &m->lm_head, (size_t)V * H * m->esz));
+        m->lm_head_owned = true;
+    }
+    M_TRY(dmalloc_t(m, &m->final_norm, (size_t)H));
+    M_TRY(fill_ones(m, m->final_norm, H));  // RMSNorm::new, rms_norm.rs:14-20
+    for (int l = 0; l < L; ++l) {
+        LayerW &w = m->layers[l];
+        M_TRY(dmalloc(m, &w.wqkv, (size_t)m->qkvd * H * m->esz));
+        M_TRY(dmalloc(m, &w.wo, (size_t)H * m->qd * m->esz));
+        M_TRY(dmalloc(m, &w.wgu, (size_t)2 * I * H * m->esz));
+        M_TRY(dmalloc(m, &w.wdown, (size_t)H * I * m->esz));
+        M_TRY(dmalloc_t(m, &w.in_norm, (size_t)H));
+        M_TRY(dmalloc_t(m, &w.post_norm, (size_t)H));
+        M_TRY(fill_ones(m, w.in_norm, H));
+        M_TRY(fill_ones(m, w.post_norm, H));
+        if (cfg->qk_norm) {
+            M_TRY(dmalloc_t(m, &w.q_norm, (size_t)D));
+            M_TRY(dmalloc_t(m, &w.k_norm, (size_t)D));
+            M_TRY(fill_ones(m, w.q_norm, D));
+            M_TRY(fill_ones(m, w.k_norm, D));
+        }
+    }
+    // one RoPE table for all layers (the reference builds an identical one per layer, self_attention.rs:78)
+    {
+        std::vector<float> c, s;
+        rope_tables_host(c, s, D, cfg->max_seq_len, cfg->rope_theta);
+        M_TRY(dmalloc_t(m, &m->cos_dev, c.size()));
+        M_TRY(dmalloc_t(m, &m->sin_dev, s.size()));
+        M_TRY(lumen_upload(ctx, m->cos_dev, c.data(), c.size() * sizeof(float)));
+        M_TRY(lumen_upload(ctx, m->sin_dev, s.data(), s.size() * sizeof(float)));
+    }
+    // init_kv_caches(1), llama.rs:161-169: zero-filled [1,Hkv,max_seq,D] per layer
+    m->cache_stride = (size_t)Hkv * cfg->max_seq_len * D;
+    M_TRY(dmalloc_t(m, &m->k_slab, m->cache_stride * L));
+    M_TRY(dmalloc_t(m, &m->v_slab, m->cache_stride * L));
+    if (hipMemsetAsync(m->k_slab, 0, m->cache_stride * L * sizeof(float), ctx->stream) != hipSuccess ||
+        hipMemsetAsync(m->v_slab, 0, m->cache_stride * L * sizeof(float), ctx->stream) != hipSuccess) {
+        lumen_llama_destroy(m);
+        LUMEN_FAIL(LUMEN_ERR_HIP, "llama_create: clearing the KV slab failed");
+    }
+    M_TRY(dmalloc_t(m, &m->x, (size_t)H));
+    M_TRY(dmalloc_t(m, &m->h, (size_t)H));
+    M_TRY(dmalloc_t(m, &m->qkv, (size_t)m->qkvd));
+    M_TRY(dmalloc_t(m, &m->attn, (size_t)m->qd));
+    M_TRY(dmalloc_t(m, &m->act, (size_t)I));
+    M_TRY(dmalloc_t(m, &m->logits, (size_t)V));
+    M_TRY(dmalloc_t(m, &m->d_tok, 4));
+    M_TRY(dmalloc_t(m, &m->d_pos, 4));
+    m->nsplit = attn_decode_nsplit(cfg->max_seq_len);
+    M_TRY(dmalloc_t(m, &m->part, attn_decode_part_floats(1, Hq, D, m->nsplit)));
+    M_TRY(dmalloc_t(m, &m->counters, (size_t)Hkv));
+    if (hipMemsetAsync(m->counters, 0, sizeof(int) * Hkv, ctx->stream) != hipSuccess ||
+        hipMemsetAsync(m->d_tok, 0, 4 * sizeof(int), ctx->stream) != hipSuccess ||
+        hipMemsetAsync(m->d_pos, 0, 4 * sizeof(int), ctx->stream) != hipSuccess ||
+        hipStreamSynchronize(ctx->stream) != hipSuccess) {
+        lumen_llama_destroy(m);
+        LUMEN_FAIL(LUMEN_ERR_HIP, "llama_create: clearing decode state failed");
+    }
+#undef M_TRY
+    *out = m;
+    return LUMEN_OK;
+}
+
+// ----------------------------------------------------------- parameter upload
+static void f32_to_bf16_host(const float *src, uint16_t *dst, size_t n) {
+    for (size_t i = 0; i < n; ++i) {
+        uint32_t u;
+        memcpy(&u, src + i, 4);
+        if ((u & 0x7fffffffu) > 0x7f800000u) {
+            dst[i] = (uint16_t)((u >> 16) | 0x40);
+        } else {
+            u += 0x7fffu + ((u >> 16) & 1u);
+            dst[i] = (uint16_t)(u >> 16);
+        }
+    }
+}
+
+static void bf16_to_f32_host(const uint16_t *src, float *dst, size_t n) {
+    for (size_t i = 0; i < n; ++i) {
+        const uint32_t u = (uint32_t)src[i] << 16;  // half::bf16::to_f32, src/loader.rs:58
+        memcpy(dst + i, &u, 4);
+    }
+}
+
+// Copies a [rows, cols] host matrix (src dtype) into device memory of dst dtype
+// whose row r lands at dst + (row0 + r*row_step) * cols.
+static int upload_matrix(lumen_llama *m, void *dst, bool dst_bf16, const void *src, int src_dtype, size_t rows,
+                         size_t cols, size_t row0, size_t row_step) {
+    const size_t dsz = dst_bf16 ? 2 : 4;
+    const bool src_bf16 = src_dtype == LUMEN_DTYPE_BF16;
+    const size_t chunk_rows = std::max<size_t>(1, (size_t)(64u << 20) / (cols * 4));
+    std::vector<char> stage;
+    for (size_t r0 = 0; r0 < rows; r0 += chunk_rows) {
+        const size_t nr = std::min(chunk_rows, rows - r0);
+        const void *p;
+        if (src_bf16 == dst_bf16) {
+            p = (const char *)src + r0 * cols * dsz;
+        } else {
+            stage.resize(nr * cols * dsz);
+            if (dst_bf16) f32_to_bf16_host((const float *)src + r0 * cols, (uint16_t *)stage.data(), nr * cols);
+            else bf16_to_f32_host((const uint16_t *)src + r0 * cols, (float *)stage.data(), nr * cols);
+            p = stage.data();
+        }
+        char *d = (char *)dst + (row0 + r0 * row_step) * cols * dsz;
+        HIP_TRY(hipMemcpy2DAsync(d, row_step * cols * dsz, p, cols * dsz, cols * dsz, nr, hipMemcpyHostToDevice,
+                                 m->ctx->stream));
+        HIP_TRY(hipStreamSynchronize(m->ctx->stream));
+    }
+    return LUMEN_OK;
+}
+
+static int want_shape(const char *name, const int64_t *shape, int ndim, int64_t a, int64_t b) {
+    const bool ok = (b < 0) ? (ndim == 1 && shape[0] == a) : (ndim == 2 && shape[0] == a && shape[1] == b);
+    if (!ok) {
+        if (b < 0) LUMEN_FAIL(LUMEN_ERR_SHAPE, "Shape mismatch for %s: expected [%lld]", name, (long long)a);
+        LUMEN_FAIL(LUMEN_ERR_SHAPE, "Shape mismatch for %s: expected [%lld, %lld]", name, (long long)a, (long long)b);
+    }
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_llama_set_param(lumen_llama *m, const char *name, const void *data, int dtype,
+                                     const int64_t *shape, int ndim) {
+    if (!m || !name || !data || !shape) LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_set_param: null argument");
+    if (dtype != LUMEN_DTYPE_F32 && dtype != LUMEN_DTYPE_BF16)  // loader.rs:67
+        LUMEN_FAIL(LUMEN_ERR_INVALID, "Unsupported dtype: %d for %s", dtype, name);
+    const lumen_llama_config &c = m->cfg;
+    const int H = c.hidden_size, I = c.intermediate_size, V = c.vocab_size;
+    const std::string n(name);
+    if (n == "model.embed_tokens.weight") {
+        LUMEN_TRY(want_shape(name, shape, ndim, V, H));
+        LUMEN_TRY(upload_matrix(m, m->embed, false, data, dtype, V, H, 0, 1));
+        if (c.tie_embeddings && m->lm_head_owned) return upload_matrix(m, m->lm_head, m->bf16, data, dtype, V, H, 0, 1);
+        return LUMEN_OK;
+    }
+    if (n == "lm_head.weight") {
+        LUMEN_TRY(want_shape(name, shape, ndim, V, H));
+        if (c.tie_embeddings) LUMEN_FAIL(LUMEN_ERR_INVALID, "lm_head.weight given but embeddings are tied");
+        return upload_matrix(m, m->lm_head, m->bf16, data, dtype, V, H, 0, 1);
+    }
+    if (n == "model.norm.weight") {
+        LUMEN_TRY(want_shape(name, shape, ndim, H, -1));
+        return upload_matrix(m, m->final_norm, false, data, dtype, 1, H, 0, 1);
+    }
+    int layer = -1, consumed = 0;
+    if (sscanf(name, "model.layers.%d.%n", &layer, &consumed) != 1 || consumed == 0 || layer < 0 ||
+        layer >= c.num_hidden_layers)
+        LUMEN_FAIL(LUMEN_ERR_INVALID, "Parameter %s not found in model", name);
+    const std::string rest(name + consumed);
+    LayerW &w = m->layers[layer];
+    if (rest == "self_attn.q_proj.weight") {
+        LUMEN_TRY(want_shape(name, shape, ndim, m->qd, H));
+        return upload_matrix(m, w.wqkv, m->bf16, data, dtype, m->qd, H, 0, 1);
+    }
+    if (rest == "self_attn.k_proj.weight") {
+        LUMEN_TRY(want_shape(name, shape, ndim, m->kvd, H));
+        return upload_matrix(m, w.wqkv, m->bf16, data, dtype, m->kvd, H, m->qd, 1);
+    }
+    if (rest == "self_attn.v_proj.weight") {
+        LUMEN_TRY(want_shape(name, shape, ndim, m->kvd, H));
+        return upload_matrix(m, w.wqkv, m->bf16, data, dtype, m->kvd, H, m->qd + m->kvd, 1);
+    }
+    if (rest == "self_attn.o_proj.weight") {
+        LUMEN_TRY(want_shape(name, shape, ndim, H, m->qd));
+        return upload_matrix(m, w.wo, m->bf16, data, dtype, H, m->qd, 0, 1);
+    }
+    if (rest == "mlp.gate_proj.weight") {  // row i -> fused row 2i
+        LUMEN_TRY(want_shape(name, shape, ndim, I, H));
+        return upload_matrix(m, w.wgu, m->bf16, data, dtype, I, H, 0, 2);
+    }
+    if (rest == "mlp.up_proj.weight") {  // row i -> fused row 2i+1
+        LUMEN_TRY(want_shape(name, shape, ndim, I, H));
+        return upload_matrix(m, w.wgu, m->bf16, data, dtype, I, H, 1, 2);
+    }
+    if (rest == "mlp.down_proj.weight") {
+        LUMEN_TRY(want_shape(name, shape, ndim, H, I));
+        return upload_matrix(m, w.wdown, m->bf16, data, dtype, H, I, 0, 1);
+    }
+    if (rest == "input_layernorm.weight") {
+        LUMEN_TRY(want_shape(name, shape, ndim, H, -1));
+        return upload_matrix(m, w.in_norm, false, data, dtype, 1, H, 0, 1);
+    }
+    if (rest == "post_attention_layernorm.weight") {
+        LUMEN_TRY(want_shape(name, shape, ndim, H, -1));
+        return upload_matrix(m, w.post_norm, false, data, dtype, 1, H, 0, 1);
+    }
+    if (c.qk_norm && rest == "self_attn.q_norm.weight") {
+        LUMEN_TRY(want_shape(name, shape, ndim, m->D, -1));
+        return upload_matrix(m, w.q_norm, false, data, dtype, 1, m->D, 0, 1);
+    }
+    if (c.qk_norm && rest == "self_attn.k_norm.weight") {
+        LUMEN_TRY(want_shape(name, shape, ndim, m->D, -1));
+        return upload_matrix(m, w.k_norm, false, data, dtype, 1, m->D, 0, 1);
+    }
+    LUMEN_FAIL(LUMEN_ERR_INVALID, "Parameter %s not found in model", name);
+}
+
+// ------------------------------------------------------------------- decode
+// One token through all layers; every launch reads the token id and the
+// position from device memory, so the sequence is the same for every token.
+static int enqueue_decode_step(lumen_llama *m) {
+    lumen_ctx *ctx = m->ctx;
+    const lumen_llama_config &c = m->cfg;
+    const int H = c.hidden_size, I = c.intermediate_size, V = c.vocab_size;
+    LUMEN_TRY(launch_embedding(ctx, m->embed, m->d_tok, 1, H, V, m->x));  // llama.rs:191
+    for (int l = 0; l < c.num_hidden_layers; ++l) {
+        const LayerW &w = m->layers[l];
+        GemvArgs g = {};
+        // input_layernorm + q|k|v projections, llama.rs:107, self_attention.rs:106-108
+        g.W = w.wqkv; g.x = m->x; g.y = m->qkv; g.N = m->qkvd; g.K = H; g.w_bf16 = m->bf16;
+        g.pro = PRO_RMSNORM; g.norm_w = w.in_norm; g.eps = c.rms_norm_eps; g.epi = EPI_STORE;
+        LUMEN_TRY(launch_gemv(ctx, g));
+        AttnDecodeArgs a = {};
+        a.q = m->qkv; a.k_new = m->qkv + m->qd; a.v_new = m->qkv + m->qd + m->kvd; a.out = m->attn;
+        a.k_cache = m->k_slab + m->cache_stride * l; a.v_cache = m->v_slab + m->cache_stride * l;
+        a.cos_t = m->cos_dev; a.sin_t = m->sin_dev; a.pos_dev = m->d_pos; a.pos_host = 0;
+        a.b = 1; a.hq = c.num_attention_heads; a.hkv = c.num_key_value_heads; a.d = m->D; a.max_seq = c.max_seq_len;
+        a.scale = m->scale; a.q_norm_w = w.q_norm; a.k_norm_w = w.k_norm; a.norm_eps = c.rms_norm_eps;
+        a.part = m->part; a.counters = m->counters; a.nsplit = m->nsplit;
+        LUMEN_TRY(launch_attn_decode(ctx, a));
+        // o_proj + residual, self_attention.rs:303, llama.rs:110
+        g = {};
+        g.W = w.wo; g.x = m->attn; g.y = m->h; g.N = H; g.K = m->qd; g.w_bf16 = m->bf16;
+        g.pro = PRO_NONE; g.epi = EPI_RESIDUAL; g.residual = m->x;
+        LUMEN_TRY(launch_gemv(ctx, g));
+        // post_attention_layernorm + gate|up + silu*up, llama.rs:113, :60-63
+        g = {};
+        g.W = w.wgu; g.x = m->h; g.y = m->act; g.N = 2 * I; g.K = H; g.w_bf16 = m->bf16;
+        g.pro = PRO_RMSNORM; g.norm_w = w.post_norm; g.eps = c.rms_norm_eps; g.epi = EPI_SWIGLU;
+        LUMEN_TRY(launch_gemv(ctx, g));
+        // down_proj + residual, llama.rs:64, :115
+        g = {};
+        g.W = w.wdown; g.x = m->act; g.y = m->x; g.N = H; g.K = I; g.w_bf16 = m->bf16;
+        g.pro = PRO_NONE; g.epi = EPI_RESIDUAL; g.residual = m->h;
+        LUMEN_TRY(launch_gemv(ctx, g));
+    }
+    // final norm + lm_head, llama.rs:202-205
+    GemvArgs g = {};
+    g.W = m->lm_head; g.x = m->x; g.y = m->logits; g.N = V; g.K = H;
+    g.w_bf16 = (m->lm_head == (void *)m->embed) ? 0 : (int)m->bf16;
+    g.pro = PRO_RMSNORM; g.norm_w = m->final_norm; g.eps = c.rms_norm_eps; g.epi = EPI_STORE;
+    LUMEN_TRY(launch_gemv(ctx, g));
+    // greedy pick becomes the next token id; the position counter advances
+    return launch_argmax(ctx, m->logits, V, m->d_tok, m->d_pos);
+}
+
+static int ensure_decode_graph(lumen_llama *m) {
+    if (m->graph_exec) return LUMEN_OK;
+    hipStream_t s = m->ctx->stream;
+    HIP_TRY(hipStreamSynchronize(s));
+    HIP_TRY(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
+    const int rc = enqueue_decode_step(m);
+    hipGraph_t g = nullptr;
+    const hipError_t e = hipStreamEndCapture(s, &g);
+    if (rc != LUMEN_OK) {
+        if (g) hipGraphDestroy(g);
+        return rc;
+    }
+    if (e != hipSuccess) LUMEN_FAIL(LUMEN_ERR_HIP, "hipStreamEndCapture failed: %s", hipGetErrorString(e));
+    m->graph = g;
+    HIP_TRY(hipGraphInstantiate(&m->graph_exec, m->graph, nullptr, nullptr, 0));
+    return LUMEN_OK;
+}
+
+static int sync_pos_to_device(lumen_llama *m) {
+    HIP_TRY(hipMemcpyAsync(m->d_pos, &m->len, sizeof(int), hipMemcpyHostToDevice, m->ctx->stream));
+    HIP_TRY(hipStreamSynchronize(m->ctx->stream));
+    return LUMEN_OK;
+}
+
+static int check_room(const lumen_llama *m, int add) {
+    if (m->len + add > m->cfg.max_seq_len)  // self_attention.rs:144-149, 341-346
+        LUMEN_FAIL(LUMEN_ERR_KV_OVERFLOW, "KV cache overflow: new_len=%d > max_seq=%d", m->len + add, m->cfg.max_seq_len);
+    return LUMEN_OK;
+}
+
+static int ids_to_int(const lumen_llama *m, const float *ids, int s, std::vector<int> &out) {
+    out.resize(s);
+    for (int t = 0; t < s; ++t) {
+        const float f = ids[t];
+        const long long idx = (f > 0.0f) ? (f >= 9.0e18f ? (long long)9e18 : (long long)f) : 0;  // `as usize`
+        if (idx >= m->cfg.vocab_size)  // embedding.rs:55
+            LUMEN_FAIL(LUMEN_ERR_EMBED_OOB, "Embedding index out of bounds: %lld >= %d", idx, m->cfg.vocab_size);
+        out[t] = (int)idx;
+    }
+    return LUMEN_OK;
+}
+
+// ------------------------------------------------------------------ prefill
+static int ensure_prefill_buffers(lumen_llama *m, int s, bool all_rows) {
+    const lumen_llama_config &c = m->cfg;
+    if (s > m->pf_cap) {
+        HIP_TRY(hipStreamSynchronize(m->ctx->stream));
+        hipFree(m->p_x); hipFree(m->p_h); hipFree(m->p_n); hipFree(m->p_qkv); hipFree(m->p_qrot);
+        hipFree(m->p_attn); hipFree(m->p_act); hipFree(m->p_ids);
+        m->p_x = m->p_h = m->p_n = m->p_qkv = m->p_qrot = m->p_attn = m->p_act = nullptr;
+        m->p_ids = nullptr;
+        m->pf_cap = 0;
+        const size_t S = (size_t)s;
+        HIP_TRY(hipMalloc((void **)&m->p_x, S * c.hidden_size * 4));
+        HIP_TRY(hipMalloc((void **)&m->p_h, S * c.hidden_size * 4));
+        HIP_TRY(hipMalloc((void **)&m->p_n, S * c.hidden_size * 4));
+        HIP_TRY(hipMalloc((void **)&m->p_qkv, S * m->qkvd * 4));
+        HIP_TRY(hipMalloc((void **)&m->p_qrot, S * m->qd * 4));
+        HIP_TRY(hipMalloc((void **)&m->p_attn, S * m->qd * 4));
+        HIP_TRY(hipMalloc((void **)&m->p_act, S * c.intermediate_size * 4));
+        HIP_TRY(hipMalloc((void **)&m->p_ids, S * sizeof(int)));
+        m->pf_cap = s;
+    }
+    if (all_rows && s > m->pf_logit_cap) {
+        HIP_TRY(hipStreamSynchronize(m->ctx->stream));
+        hipFree(m->p_logits);
+        m->p_logits = nullptr;
+        m->pf_logit_cap = 0;
+        HIP_TRY(hipMalloc((void **)&m->p_logits, (size_t)s * c.vocab_size * 4));
+        m->pf_logit_cap = s;
+    }
+    return LUMEN_OK;
+}
+
+static int run_prefill(lumen_llama *m, const std::vector<int> &ids, float *logits_host, int all_rows) {
+    lumen_ctx *ctx = m->ctx;
+    const lumen_llama_config &c = m->cfg;
+    const int s = (int)ids.size();
+    const int H = c.hidden_size, I = c.intermediate_size, V = c.vocab_size;
+    LUMEN_TRY(ensure_prefill_buffers(m, s, all_rows != 0));
+    HIP_TRY(hipMemcpyAsync(m->p_ids, ids.data(), sizeof(int) * s, hipMemcpyHostToDevice, ctx->stream));
+    LUMEN_TRY(launch_embedding(ctx, m->embed, m->p_ids, s, H, V, m->p_x));
+    for (int l = 0; l < c.num_hidden_layers; ++l) {
+        const LayerW &w = m->layers[l];
+        LUMEN_TRY(launch_rmsnorm(ctx, m->p_x, w.in_norm, m->p_n, s, H, c.rms_norm_eps));
+        GemmArgs g = {};
+        g.A = m->p_n; g.W = w.wqkv; g.C = m->p_qkv; g.M = s; g.N = m->qkvd; g.K = H; g.w_bf16 = m->bf16; g.epi = EPI_STORE;
+        LUMEN_TRY(launch_gemm(ctx, g));
+        AttnPrefillArgs a = {};
+        a.q = m->p_qkv; a.k = m->p_qkv + m->qd; a.v = m->p_qkv + m->qd + m->kvd; a.out = m->p_attn;
+        a.k_cache = m->k_slab + m->cache_stride * l; a.v_cache = m->v_slab + m->cache_stride * l;
+        a.cos_t = m->cos_dev; a.sin_t = m->sin_dev;
+        a.b = 1; a.s = s; a.hq = c.num_attention_heads; a.hkv = c.num_key_value_heads; a.d = m->D;
+        a.max_seq = c.max_seq_len; a.past_len = m->len;
+        a.q_stride = a.k_stride = a.v_stride = m->qkvd;
+        a.scale = m->scale; a.causal = 1; a.q_norm_w = w.q_norm; a.k_norm_w = w.k_norm; a.norm_eps = c.rms_norm_eps;
+        a.q_rot = m->p_qrot;
+        LUMEN_TRY(launch_attn_prefill(ctx, a));
+        g = {};
+        g.A = m->p_attn; g.W = w.wo; g.C = m->p_h; g.M = s; g.N = H; g.K = m->qd; g.w_bf16 = m->bf16;
+        g.epi = EPI_RESIDUAL; g.residual = m->p_x;
+        LUMEN_TRY(launch_gemm(ctx, g));
+        LUMEN_TRY(launch_rmsnorm(ctx, m->p_h, w.post_norm, m->p_n, s, H, c.rms_norm_eps));
+        g = {};
+        g.A = m->p_n; g.W = w.wgu; g.C = m->p_act; g.M = s; g.N = 2 * I; g.K = H; g.w_bf16 = m->bf16; g.epi = EPI_SWIGLU;
+        LUMEN_TRY(launch_gemm(ctx, g));
+        g = {};
+        g.A = m->p_act; g.W = w.wdown; g.C = m->p_x; g.M = s; g.N = H; g.K = I; g.w_bf16 = m->bf16;
+        g.epi = EPI_RESIDUAL; g.residual = m->p_h;
+        LUMEN_TRY(launch_gemm(ctx, g));
+    }
+    const int head_bf16 = (m->lm_head == (void *)m->embed) ? 0 : (int)m->bf16;
+    if (all_rows) {  // what the reference computes, llama.rs:202-205
+        LUMEN_TRY(launch_rmsnorm(ctx, m->p_x, m->final_norm, m->p_n, s, H, c.rms_norm_eps));
+        GemmArgs g = {};
+        g.A = m->p_n; g.W = m->lm_head; g.C = m->p_logits; g.M = s; g.N = V; g.K = H; g.w_bf16 = head_bf16; g.epi = EPI_STORE;
+        LUMEN_TRY(launch_gemm(ctx, g));
+        m->len += s;
+        if (logits_host) LUMEN_TRY(lumen_download(ctx, logits_host, m->p_logits, sizeof(float) * (size_t)s * V));
+    } else {  // what its caller keeps, main.rs:155-163
+        GemvArgs g = {};
+        g.W = m->lm_head; g.x = m->p_x + (size_t)(s - 1) * H; g.y = m->logits; g.N = V; g.K = H; g.w_bf16 = head_bf16;
+        g.pro = PRO_RMSNORM; g.norm_w = m->final_norm; g.eps = c.rms_norm_eps; g.epi = EPI_STORE;
+        LUMEN_TRY(launch_gemv(ctx, g));
+        m->len += s;
+        if (logits_host) LUMEN_TRY(lumen_download(ctx, logits_host, m->logits, sizeof(float) * (size_t)V));
+    }
+    return sync_pos_to_device(m);
+}
+
+extern "C" int lumen_llama_forward(lumen_llama *m, const float *ids_host, int s, float *logits_host, int all_rows) {
+    if (!m || (!ids_host && s > 0)) LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_forward: null argument");
+    if (s <= 0) LUMEN_FAIL(LUMEN_ERR_SHAPE, "llama_forward: empty input");
+    HIP_TRY(hipSetDevice(m->ctx->device));
+    std::vector<int> ids;
+    LUMEN_TRY(ids_to_int(m, ids_host, s, ids));
+    LUMEN_TRY(check_room(m, s));
+    if (s > 1) return run_prefill(m, ids, logits_host, all_rows);
+    // S == 1: the decode path (self_attention.rs:125)
+    LUMEN_TRY(ensure_decode_graph(m));
+    hipStream_t st = m->ctx->stream;
+    HIP_TRY(hipMemcpyAsync(m->d_tok, ids.data(), sizeof(int), hipMemcpyHostToDevice, st));
+    HIP_TRY(hipStreamSynchronize(st));
+    HIP_TRY(hipGraphLaunch(m->graph_exec, st));
+    m->len += 1;
+    if (logits_host) return lumen_download(m->ctx, logits_host, m->logits, sizeof(float) * (size_t)m->cfg.vocab_size);
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_llama_decode_greedy(lumen_llama *m, int first_id, int n, int32_t *ids_out, float *logits_out) {
+    if (!m) LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_decode_greedy: null model");
+    if (n < 0) LUMEN_FAIL(LUMEN_ERR_SHAPE, "llama_decode_greedy: n=%d", n);
+    if (first_id < 0 || first_id >= m->cfg.vocab_size)
+        LUMEN_FAIL(LUMEN_ERR_EMBED_OOB, "Embedding index out of bounds: %d >= %d", first_id, m->cfg.vocab_size);
+    if (n == 0) return LUMEN_OK;
+    HIP_TRY(hipSetDevice(m->ctx->device));
+    LUMEN_TRY(check_room(m, n));
+    LUMEN_TRY(ensure_decode_graph(m));
+    hipStream_t st = m->ctx->stream;
+    const size_t V = (size_t)m->cfg.vocab_size;
+    HIP_TRY(hipMemcpyAsync(m->d_tok, &first_id, sizeof(int), hipMemcpyHostToDevice, st));
+    HIP_TRY(hipStreamSynchronize(st));
+    int *ids_dev = nullptr;
+    if (ids_out) HIP_TRY(hipMalloc((void **)&ids_dev, sizeof(int) * (size_t)n));
+    int rc = LUMEN_OK;
+    for (int t = 0; t < n && rc == LUMEN_OK; ++t) {
+        hipError_t e = hipGraphLaunch(m->graph_exec, st);
+        if (e == hipSuccess && ids_dev)
+            e = hipMemcpyAsync(ids_dev + t, m->d_tok, sizeof(int), hipMemcpyDeviceToDevice, st);
+        if (e == hipSuccess && logits_out)
+            e = hipMemcpyAsync(logits_out + (size_t)t * V, m->logits, sizeof(float) * V, hipMemcpyDeviceToHost, st);
+        if (e != hipSuccess) {
+            lumen_set_error("decode step %d failed: %s", t, hipGetErrorString(e));
+            rc = LUMEN_ERR_HIP;
+        } else {
+            m->len += 1;
+        }
+    }
+    hipError_t e = hipStreamSynchronize(st);
+    if (rc == LUMEN_OK && e == hipSuccess && ids_dev)
+        e = hipMemcpy(ids_out, ids_dev, sizeof(int) * (size_t)n, hipMemcpyDeviceToHost);
+    hipFree(ids_dev);
+    if (rc == LUMEN_OK && e != hipSuccess) LUMEN_FAIL(LUMEN_ERR_HIP, "decode_greedy: %s", hipGetErrorString(e));
+    return rc;
+}
+
+extern "C" int lumen_llama_reset(lumen_llama *m) {
+    if (!m) LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_reset: null model");
+    m->len = 0;  // KVCacheInner::reset, self_attention.rs:41-43: data stays
+    return sync_pos_to_device(m);
+}
+
+extern "C" int lumen_llama_kv_len(const lumen_llama *m, int *len_out) {
+    if (!m || !len_out) LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_kv_len: null argument");
+    *len_out = m->len;
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_llama_cache_download(lumen_llama *m, int layer, float *k_host, float *v_host) {
+    if (!m || !k_host || !v_host) LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_cache_download: null argument");
+    if (layer < 0 || layer >= m->cfg.num_hidden_layers)  // llama.rs:182-188 analogue
+        LUMEN_FAIL(LUMEN_ERR_CACHE_COUNT, "KV cache index %d outside [0,%d)", layer, m->cfg.num_hidden_layers);
+    const size_t bytes = m->cache_stride * sizeof(float);
+    LUMEN_TRY(lumen_download(m->ctx, k_host, m->k_slab + m->cache_stride * layer, bytes));
+    return lumen_download(m->ctx, v_host, m->v_slab + m->cache_stride * layer, bytes);
+}
+
+extern "C" int lumen_llama_decode_bytes(const lumen_llama *m, int len, double *bytes_out) {
+    if (!m || !bytes_out) LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_decode_bytes: null argument");
+    const lumen_llama_config &c = m->cfg;
+    const double H = c.hidden_size, I = c.intermediate_size, V = c.vocab_size, L = c.num_hidden_layers;
+    const double per_layer = ((double)m->qkvd * H + H * m->qd + 3.0 * H * I) * (double)m->esz;
+    const double head = V * H * ((m->lm_head == (void *)m->embed) ? 4.0 : (double)m->esz);
+    const double norms = (2.0 * L + 1.0) * H * 4.0 + (c.qk_norm ? 2.0 * L * m->D * 4.0 : 0.0);
+    const double kv = L * 2.0 * c.num_key_value_heads * m->D * 4.0 * (double)len;
+    *bytes_out = L * per_layer + head + norms + kv;
+    return LUMEN_OK;
+}

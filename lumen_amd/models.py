@@ -1,0 +1,209 @@
+"""LlamaModel of the reference (src/models/llama.rs) on the GPU.
+
+LlamaModel drives the fused model-level entry points (one HIP-graph replay
+per decoded token).  LayeredLlamaModel composes the same network from the
+layer classes, one C-ABI call per reference operator, exactly as
+LlamaDecoderLayer::forward_infer does; it exists so that the operator-level
+drop-ins are exercised end to end.
+"""
+import ctypes as C
+from dataclasses import dataclass
+
+import numpy as np
+
+from . import _lib, synth
+from ._lib import ERR_CACHE_COUNT, LumenError, check, lib
+from .autograd import Tensor, default_ctx
+from .layers import Embedding, KVCacheInner, Linear, RMSNorm, SelfAttention, SiLU
+
+
+@dataclass
+class LlamaConfig:
+    """src/models/llama.rs:11-37 plus the fields the other benchmark shapes need."""
+    vocab_size: int = 32000
+    hidden_size: int = 2048
+    intermediate_size: int = 5632
+    num_hidden_layers: int = 22
+    num_attention_heads: int = 32
+    num_key_value_heads: int = 4
+    rms_norm_eps: float = 1e-5
+    max_seq_len: int = 2048
+    rope_theta: float = 10000.0
+    head_dim: int = 0
+    qk_norm: bool = False
+    tie_embeddings: bool = False
+    weight_dtype: str = "f32"
+
+    @staticmethod
+    def from_dict(d):
+        return LlamaConfig(**{k: v for k, v in d.items()})
+
+    def as_dict(self):
+        return dict(self.__dict__)
+
+
+class LlamaModel:
+    """llama.rs:129-280.  Caches live inside the model (init_kv_caches(1) happens at construction);
+    init_kv_caches / reset_kv_caches keep the reference's call shape."""
+
+    def __init__(self, config, ctx=None):
+        if isinstance(config, dict):
+            config = LlamaConfig.from_dict(config)
+        self.config = config
+        self.ctx = ctx or default_ctx()
+        c = _lib.LlamaConfigStruct(
+            config.vocab_size, config.hidden_size, config.intermediate_size, config.num_hidden_layers,
+            config.num_attention_heads, config.num_key_value_heads, config.rms_norm_eps, config.max_seq_len,
+            config.rope_theta, config.head_dim or 0, int(config.qk_norm), int(config.tie_embeddings),
+            _lib.DTYPE_BF16 if config.weight_dtype == "bf16" else _lib.DTYPE_F32)
+        h = C.c_void_p()
+        check(lib.lumen_llama_create(self.ctx.handle, C.byref(c), C.byref(h)))
+        self.handle = h
+
+    def __del__(self):
+        h, self.handle = getattr(self, "handle", None), None
+        if h:
+            lib.lumen_llama_destroy(h)
+
+    # -- weights ------------------------------------------------------------
+    def set_param(self, name, array):
+        """One tensor by HF name (llama.rs:218-279); f32 arrays or bf16 bits as uint16 (loader.rs:32-68)."""
+        a = np.ascontiguousarray(array)
+        dtype = _lib.DTYPE_BF16 if a.dtype == np.uint16 else _lib.DTYPE_F32
+        if dtype == _lib.DTYPE_F32 and a.dtype != np.float32:
+            a = a.astype(np.float32)
+        shape = (C.c_int64 * a.ndim)(*a.shape)
+        check(lib.lumen_llama_set_param(self.handle, name.encode(), a.ctypes.data, dtype, shape, a.ndim))
+
+    def load_params(self, named):
+        for name, a in (named.items() if hasattr(named, "items") else named):
+            self.set_param(name, a)
+
+    def named_parameter_shapes(self):
+        return synth.param_shapes(self.config.as_dict())
+
+    # -- caches ---------------------------------------------------------------
+    def init_kv_caches(self, batch_size=1):  # llama.rs:161-169
+        if batch_size != 1:
+            raise LumenError(_lib.ERR_UNSUPPORTED, "batch-1 path only")
+        self.reset_kv_caches()
+        return [("model-owned", i) for i in range(self.config.num_hidden_layers)]
+
+    def reset_kv_caches(self, caches=None):  # llama.rs:172-176
+        check(lib.lumen_llama_reset(self.handle))
+
+    @property
+    def kv_len(self):
+        n = C.c_int()
+        check(lib.lumen_llama_kv_len(self.handle, C.byref(n)))
+        return n.value
+
+    def cache(self, layer):
+        cfg = self.config
+        d = cfg.head_dim or cfg.hidden_size // cfg.num_attention_heads
+        shape = (1, cfg.num_key_value_heads, cfg.max_seq_len, d)
+        k, v = np.empty(shape, np.float32), np.empty(shape, np.float32)
+        check(lib.lumen_llama_cache_download(self.handle, layer, k.ctypes.data, v.ctypes.data))
+        return k, v
+
+    # -- forward ----------------------------------------------------------------
+    def forward(self, input_ids, caches=None, _pos=0, all_rows=True):
+        """llama.rs:181-206.  input_ids: token ids (any numeric dtype; they travel as f32 like
+        main.rs:143-152).  Returns host logits [S, V] (all_rows) or [V] (last position only)."""
+        if caches is not None and len(caches) != self.config.num_hidden_layers:  # llama.rs:182-188
+            raise LumenError(ERR_CACHE_COUNT, "KV cache count mismatch: got %d, expected %d"
+                             % (len(caches), self.config.num_hidden_layers))
+        ids = np.ascontiguousarray(input_ids, np.float32).reshape(-1)
+        s = ids.size
+        out = np.empty((s, self.config.vocab_size) if all_rows else (self.config.vocab_size,), np.float32)
+        check(lib.lumen_llama_forward(self.handle, ids.ctypes.data, s, out.ctypes.data, int(all_rows)))
+        return out
+
+    def decode_greedy(self, first_id, n, want_logits=False):
+        """The generation loop of main.rs:340-378 with greedy picks, entirely on the GPU."""
+        ids = np.empty(n, np.int32)
+        logits = np.empty((n, self.config.vocab_size), np.float32) if want_logits else None
+        check(lib.lumen_llama_decode_greedy(self.handle, int(first_id), n, ids.ctypes.data,
+                                            logits.ctypes.data if want_logits else None))
+        return (ids, logits) if want_logits else ids
+
+    def decode_bytes(self, length):
+        b = C.c_double()
+        check(lib.lumen_llama_decode_bytes(self.handle, int(length), C.byref(b)))
+        return b.value
+
+
+class LlamaMLP:
+    """llama.rs:41-66: down(silu(gate(x)) * up(x)) as five separate operator calls."""
+
+    def __init__(self, gate_w, up_w, down_w):
+        self.gate_proj, self.up_proj, self.down_proj = Linear(gate_w), Linear(up_w), Linear(down_w)
+        self.act = SiLU()
+
+    def forward(self, x):
+        gate = self.gate_proj.forward(x)
+        gate_act = self.act.forward(gate)
+        up = self.up_proj.forward(x)
+        fused = gate_act * up
+        return self.down_proj.forward(fused)
+
+
+class LlamaDecoderLayer:
+    """llama.rs:79-116 (forward_infer)."""
+
+    def __init__(self, cfg, params, prefix, ctx):
+        self.self_attn = SelfAttention(cfg.hidden_size, cfg.num_attention_heads, cfg.num_key_value_heads,
+                                       cfg.max_seq_len, cfg.rope_theta, True, ctx)
+        for attr, name in (("w_q", "q_proj"), ("w_k", "k_proj"), ("w_v", "v_proj"), ("w_o", "o_proj")):
+            setattr(self.self_attn, attr, Linear(Tensor.from_array_no_grad(params[prefix + "self_attn.%s.weight" % name], ctx)))
+        t = lambda n: Tensor.from_array_no_grad(params[prefix + n], ctx)
+        self.mlp = LlamaMLP(t("mlp.gate_proj.weight"), t("mlp.up_proj.weight"), t("mlp.down_proj.weight"))
+        self.input_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps, params[prefix + "input_layernorm.weight"], ctx)
+        self.post_attention_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps,
+                                                params[prefix + "post_attention_layernorm.weight"], ctx)
+
+    def forward_infer(self, x, cache):
+        norm_x = self.input_layernorm.forward(x)
+        attn_out, cache_out = self.self_attn.forward(norm_x, cache)
+        h = x + attn_out
+        norm_h = self.post_attention_layernorm.forward(h)
+        mlp_out = self.mlp.forward(norm_h)
+        return h + mlp_out, cache_out
+
+
+class LayeredLlamaModel:
+    """LlamaModel::forward (llama.rs:181-206) composed operator by operator."""
+
+    def __init__(self, config, params, ctx=None):
+        if isinstance(config, dict):
+            config = LlamaConfig.from_dict(config)
+        if config.head_dim or config.qk_norm or config.tie_embeddings or config.weight_dtype != "f32":
+            raise LumenError(_lib.ERR_UNSUPPORTED, "the layered model covers the reference's Llama shape only")
+        self.config = config
+        self.ctx = ctx or default_ctx()
+        self.embed_tokens = Embedding(Tensor.from_array_no_grad(params["model.embed_tokens.weight"], self.ctx))
+        self.layers = [LlamaDecoderLayer(config, params, "model.layers.%d." % i, self.ctx)
+                       for i in range(config.num_hidden_layers)]
+        self.norm = RMSNorm(config.hidden_size, config.rms_norm_eps, params["model.norm.weight"], self.ctx)
+        self.lm_head = Linear(Tensor.from_array_no_grad(params["lm_head.weight"], self.ctx))
+
+    def init_kv_caches(self, batch_size=1):
+        c = self.config
+        d = c.hidden_size // c.num_attention_heads
+        return [KVCacheInner(batch_size, c.num_key_value_heads, c.max_seq_len, d, self.ctx)
+                for _ in range(c.num_hidden_layers)]
+
+    def reset_kv_caches(self, caches):
+        for c in caches:
+            c.reset()
+
+    def forward(self, input_ids, caches, _pos=0):
+        if len(caches) != len(self.layers):
+            raise LumenError(ERR_CACHE_COUNT, "KV cache count mismatch: got %d, expected %d"
+                             % (len(caches), len(self.layers)))
+        ids = np.ascontiguousarray(input_ids, np.float32).reshape(1, -1)
+        x = self.embed_tokens.forward(ids)
+        for i, layer in enumerate(self.layers):
+            x, caches[i] = layer.forward_infer(x, caches[i])
+        x = self.norm.forward(x)
+        return self.lm_head.forward(x)

@@ -1,0 +1,145 @@
+"""GPU parity: static KV cache, decode attention and prefill attention against the CPU oracle.
+
+Cache rows (RoPE(k), v) must be bit-exact; attention outputs within 2e-5 of max|ref| (the
+online-softmax merge order differs from the reference's sequential scan).
+"""
+import math
+
+import numpy as np
+import pytest
+
+from lumen_amd import _lib
+from lumen_amd.kv_cache import LlamaKVCache
+from lumen_amd.layers import KVCacheInner, RotaryEmbedding
+from lumen_amd.models import LlamaConfig
+from lumen_amd._lib import check, lib
+from lumen_amd.autograd import Tensor
+from oracle import lumen_oracle as lo
+from tests.gpu_util import dev, f32, max_rel
+
+pytestmark = pytest.mark.gpu
+RNG = np.random.default_rng(7)
+TOL = 2e-5
+
+
+def gpu_decode(cache, rope, q, k, v, h, scale):
+    out = Tensor.empty((q.shape[0], 1, h, q.shape[-1]))
+    check(lib.lumen_attn_decode_f32(cache.handle, rope.handle, dev(q).ptr, dev(k).ptr, dev(v).ptr, out.ptr, h, scale, 1))
+    return out.data()
+
+
+def gpu_prefill(cache, rope, q, k, v, scale):
+    b, s, h, d = q.shape
+    out = Tensor.empty((b, s, h, d))
+    check(lib.lumen_attn_prefill_f32(cache.handle, rope.handle, dev(q).ptr, dev(k).ptr, dev(v).ptr, out.ptr, s, h, scale, 1))
+    return out.data()
+
+
+@pytest.mark.parametrize("h,h_kv,d,max_seq,prefill,steps", [
+    (32, 4, 64, 2048, 0, 40), (32, 4, 64, 2048, 300, 6), (16, 8, 128, 512, 100, 5), (32, 32, 128, 256, 61, 4),
+    (8, 2, 16, 64, 0, 64), (8, 1, 32, 4096, 4000, 3), (2, 2, 64, 32, 1, 3)])
+def test_decode_steps_match_oracle(h, h_kv, d, max_seq, prefill, steps):
+    scale = 1.0 / math.sqrt(d)
+    rope = RotaryEmbedding(d, max_seq, 10000.0)
+    cos, sin = lo.rope_table(d, max_seq, 10000.0)
+    g, o = KVCacheInner(1, h_kv, max_seq, d), lo.KVCache(1, h_kv, max_seq, d)
+    if prefill:
+        q = f32(RNG.normal(0, 1, (1, prefill, h, d)))
+        k = f32(RNG.normal(0, 1, (1, prefill, h_kv, d)))
+        v = f32(RNG.normal(0, 1, (1, prefill, h_kv, d)))
+        got = gpu_prefill(g, rope, q, k, v, scale)
+        rc, ref = lo.attn_prefill(o, q, k, v, cos, sin, scale)
+        assert rc == lo.LO_OK and max_rel(got, ref) <= TOL
+    for t in range(steps):
+        q = f32(RNG.normal(0, 1, (1, h, d)))
+        k = f32(RNG.normal(0, 1, (1, h_kv, d)))
+        v = f32(RNG.normal(0, 1, (1, h_kv, d)))
+        got = gpu_decode(g, rope, q, k, v, h, scale)
+        rc, ref = lo.attn_decode(o, q, k, v, cos, sin, scale)
+        assert rc == lo.LO_OK
+        assert max_rel(got, ref) <= TOL, (t, max_rel(got, ref))
+        assert g.len == o.len == prefill + t + 1
+    n = prefill + steps
+    assert np.array_equal(g.k[:, :, :n], o.k[:, :, :n]) and np.array_equal(g.v[:, :, :n], o.v[:, :, :n])
+    assert not g.k[:, :, n:].any() and not g.v[:, :, n:].any()  # untouched rows stay zero
+
+
+def test_decode_degenerate_and_gqa_mapping():
+    h, h_kv, d, max_seq = 8, 2, 64, 128
+    rope = RotaryEmbedding(d, max_seq, 10000.0)
+    g = KVCacheInner(1, h_kv, max_seq, d)
+    q = f32(RNG.normal(0, 1, (1, h, d)))
+    k = f32(RNG.normal(0, 1, (1, h_kv, d)))
+    v = f32(RNG.normal(0, 1, (1, h_kv, d)))
+    out = gpu_decode(g, rope, q, k, v, h, 0.125)
+    for hq in range(h):  # L = 1: out = v of the head's KV group
+        assert np.array_equal(out[0, 0, hq], v[0, hq // 4])
+    g.reset()
+    vs = []
+    for t in range(70):  # zero queries: uniform weights -> mean of V per KV group
+        v = f32(np.stack([np.full(d, 10.0 * (grp + 1) + t) for grp in range(h_kv)])[None])
+        vs.append(v[0])
+        out = gpu_decode(g, rope, np.zeros((1, h, d), np.float32), f32(RNG.normal(0, 1, (1, h_kv, d))), v, h, 0.125)
+    mean = np.mean(vs, 0)
+    for hq in range(h):
+        assert np.allclose(out[0, 0, hq], mean[hq // 4], rtol=1e-5)
+
+
+def test_cache_state_machine_overflow_and_reset():
+    h, h_kv, d, max_seq = 2, 1, 16, 6
+    rope = RotaryEmbedding(d, max_seq, 10000.0)
+    g = KVCacheInner(1, h_kv, max_seq, d)
+    assert g.len == 0 and not g.k.any() and not g.v.any()
+    r = lambda *s: f32(RNG.normal(0, 1, s))
+    gpu_prefill(g, rope, r(1, 4, h, d), r(1, 4, h_kv, d), r(1, 4, h_kv, d), 0.25)
+    assert g.len == 4
+    gpu_decode(g, rope, r(1, h, d), r(1, h_kv, d), r(1, h_kv, d), h, 0.25)
+    assert g.len == 5
+    with pytest.raises(_lib.LumenError) as e:
+        gpu_prefill(g, rope, r(1, 2, h, d), r(1, 2, h_kv, d), r(1, 2, h_kv, d), 0.25)
+    assert e.value.status == _lib.ERR_ROPE_RANGE and g.len == 5
+    gpu_decode(g, rope, r(1, h, d), r(1, h_kv, d), r(1, h_kv, d), h, 0.25)
+    with pytest.raises(_lib.LumenError) as e:
+        gpu_decode(g, rope, r(1, h, d), r(1, h_kv, d), r(1, h_kv, d), h, 0.25)
+    assert e.value.status == _lib.ERR_KV_OVERFLOW and g.len == 6
+    stale = g.k
+    g.reset()
+    assert g.len == 0 and np.array_equal(g.k, stale)
+    q, k, v = r(1, h, d), r(1, h_kv, d), r(1, h_kv, d)
+    a = gpu_decode(g, rope, q, k, v, h, 0.25)
+    b = gpu_decode(KVCacheInner(1, h_kv, max_seq, d), rope, q, k, v, h, 0.25)
+    assert np.array_equal(a, b)  # stale rows beyond len are never read
+
+
+@pytest.mark.parametrize("h,h_kv,d,s,past", [(32, 4, 64, 128, 0), (16, 8, 128, 50, 17), (4, 4, 32, 3, 9), (8, 2, 16, 33, 31)])
+def test_prefill_with_and_without_past(h, h_kv, d, s, past):
+    max_seq = past + s + 3
+    scale = 1.0 / math.sqrt(d)
+    rope = RotaryEmbedding(d, max_seq, 10000.0)
+    cos, sin = lo.rope_table(d, max_seq, 10000.0)
+    g, o = KVCacheInner(1, h_kv, max_seq, d), lo.KVCache(1, h_kv, max_seq, d)
+    for n in ([past, s] if past else [s]):
+        q = f32(RNG.normal(0, 1, (1, n, h, d)))
+        k = f32(RNG.normal(0, 1, (1, n, h_kv, d)))
+        v = f32(RNG.normal(0, 1, (1, n, h_kv, d)))
+        got = gpu_prefill(g, rope, q, k, v, scale)
+        rc, ref = lo.attn_prefill(o, q, k, v, cos, sin, scale)
+        assert rc == lo.LO_OK and max_rel(got, ref) <= TOL
+    assert g.len == o.len == past + s
+    assert np.array_equal(g.k, o.k) and np.array_equal(g.v, o.v)
+
+
+def test_legacy_llama_kv_cache_update_and_view():
+    cfg = LlamaConfig(hidden_size=64, num_attention_heads=4, num_key_value_heads=2, max_seq_len=10)
+    c = LlamaKVCache(cfg)
+    k = f32(RNG.normal(0, 1, (1, 2, 3, 16)))
+    v = f32(RNG.normal(0, 1, (1, 2, 3, 16)))
+    c.update(dev(k), dev(v), 4)
+    assert np.array_equal(c.k_cache[:, :, 4:7], k) and np.array_equal(c.v_cache[:, :, 4:7], v)
+    assert not c.k_cache[:, :, :4].any() and not c.k_cache[:, :, 7:].any()
+    kv, vv = c.get_view(6)
+    assert kv.shape == (1, 2, 6, 16)
+    assert np.array_equal(kv.data(), c.k_cache[:, :, :6]) and np.array_equal(vv.data(), c.v_cache[:, :, :6])
+    with pytest.raises(_lib.LumenError) as e:
+        c.update(dev(k), dev(v), 8)  # kv_cache.rs:33-36
+    assert e.value.status == _lib.ERR_KV_OVERFLOW

@@ -1,0 +1,188 @@
+"""GPU parity: whole-model forward (prefill, teacher-forced decode, greedy generation) against the
+CPU oracle on the same seeded weights and token ids.
+
+Tolerance (stated by the benchmark): per-step logits max|d|/max|ref| <= 1e-4 for f32 weights,
+<= 2e-2 for bf16-stored weights (the oracle runs on the same bf16 values widened to f32); greedy
+picks identical unless the oracle's top-2 logits are closer than the tolerance (an argmax tie).
+"""
+import numpy as np
+import pytest
+
+from lumen_amd import _lib, synth
+from lumen_amd.models import LayeredLlamaModel, LlamaModel
+from oracle import lumen_oracle as lo
+from tests.gpu_util import max_rel
+
+pytestmark = pytest.mark.gpu
+
+TINY = dict(vocab_size=300, hidden_size=128, intermediate_size=352, num_hidden_layers=3, num_attention_heads=8,
+            num_key_value_heads=2, rms_norm_eps=1e-5, max_seq_len=96, rope_theta=10000.0)
+TINY_MHA = dict(TINY, num_key_value_heads=8, hidden_size=256, num_attention_heads=8)
+TINY_QWEN = dict(vocab_size=411, hidden_size=96, intermediate_size=160, num_hidden_layers=2, num_attention_heads=4,
+                 num_key_value_heads=2, rms_norm_eps=1e-6, max_seq_len=80, rope_theta=1.0e6, head_dim=64,
+                 qk_norm=True, tie_embeddings=True)
+SMALL = dict(vocab_size=2000, hidden_size=512, intermediate_size=1408, num_hidden_layers=4, num_attention_heads=8,
+             num_key_value_heads=2, rms_norm_eps=1e-5, max_seq_len=256, rope_theta=10000.0)
+
+
+def build(cfg, seed, std=0.1, gains_one=False, bf16=False):
+    params = synth.make_params(cfg, seed=seed, std=std, gains_one=gains_one)
+    gcfg = dict(cfg)
+    if bf16:
+        gcfg["weight_dtype"] = "bf16"
+        bits = {n: synth.bf16_round(a) for n, a in params.items() if a.ndim == 2}
+        params = {n: (synth.bf16_widen(bits[n]) if n in bits else a) for n, a in params.items()}
+    gpu = LlamaModel(gcfg)
+    for n, a in params.items():
+        gpu.set_param(n, bits[n] if bf16 and n in bits and n != "model.embed_tokens.weight" else a)
+    return gpu, lo.Llama(cfg, params), params
+
+
+def check_argmax(got_logits, ref_logits, tol):
+    ref_pick = lo.argmax(ref_logits)
+    got_pick = int(np.argmax(got_logits))
+    if got_pick != ref_pick:  # only a near-tie may differ
+        top2 = np.sort(ref_logits)[-2:]
+        assert top2[1] - top2[0] <= 2 * tol * np.abs(ref_logits).max(), (got_pick, ref_pick)
+
+
+@pytest.mark.parametrize("cfg,tol,bf16", [(TINY, 1e-4, False), (TINY_MHA, 1e-4, False), (TINY_QWEN, 1e-4, False),
+                                          (SMALL, 1e-4, False), (TINY, 2e-2, True), (TINY_QWEN, 2e-2, True)],
+                         ids=["gqa", "mha", "qwen3", "small", "gqa-bf16", "qwen3-bf16"])
+def test_prefill_then_teacher_forced_decode(cfg, tol, bf16):
+    gpu, ora, _ = build(cfg, seed=11, bf16=bf16)
+    n_prompt, n_dec = 19, 24
+    ids = synth.make_tokens(n_prompt + n_dec, cfg["vocab_size"], seed=11)
+    got = gpu.forward(ids[:n_prompt], all_rows=True)
+    rc, ref = ora.forward(ids[:n_prompt])
+    assert rc == lo.LO_OK and got.shape == ref.shape
+    assert max_rel(got, ref) <= tol
+    assert gpu.kv_len == ora.kv_len == n_prompt
+    for t in range(n_prompt, n_prompt + n_dec):
+        g = gpu.forward(ids[t:t + 1], all_rows=False)
+        rc, r = ora.forward(ids[t:t + 1])
+        assert rc == lo.LO_OK
+        assert max_rel(g, r[0]) <= tol, (t, max_rel(g, r[0]))
+        check_argmax(g, r[0], tol)
+    assert gpu.kv_len == ora.kv_len == n_prompt + n_dec
+    if not bf16:
+        for layer in range(cfg["num_hidden_layers"]):
+            k, v = gpu.cache(layer)
+            n = n_prompt + n_dec
+            assert max_rel(k[:, :, :n], ora.cache_k(layer)[:, :, :n]) <= tol
+            assert max_rel(v[:, :, :n], ora.cache_v(layer)[:, :, :n]) <= tol
+
+
+def test_last_row_only_prefill_equals_all_rows_and_incremental_prefill():
+    gpu, ora, _ = build(TINY, seed=12)
+    ids = synth.make_tokens(30, TINY["vocab_size"], seed=12)
+    full = gpu.forward(ids, all_rows=True)
+    gpu.reset_kv_caches()
+    assert gpu.kv_len == 0
+    last = gpu.forward(ids[:9], all_rows=False)
+    assert max_rel(last, full[8]) <= 1e-5
+    rest = gpu.forward(ids[9:], all_rows=True)  # prefill into a live cache (main.rs:333-335)
+    assert max_rel(rest, full[9:]) <= 1e-5
+    rc, ref = ora.forward(ids)
+    assert max_rel(full, ref) <= 1e-4
+
+
+def test_greedy_generation_on_device_matches_oracle_loop():
+    gpu, ora, _ = build(SMALL, seed=13)
+    prompt = synth.make_tokens(12, SMALL["vocab_size"], seed=13)
+    n = 40
+    g_last = gpu.forward(prompt, all_rows=False)
+    rc, r = ora.forward(prompt)
+    first = lo.argmax(r[-1])
+    assert int(np.argmax(g_last)) == first
+    ids, logits = gpu.decode_greedy(first, n, want_logits=True)
+    assert gpu.kv_len == 12 + n
+    tok = first
+    for t in range(n):
+        rc, r = ora.forward(np.array([tok]))
+        assert max_rel(logits[t], r[0]) <= 1e-4, t
+        nxt = lo.argmax(r[0])
+        if ids[t] != nxt:
+            check_argmax(logits[t], r[0], 1e-4)
+            pytest.skip("argmax near-tie at step %d: sequences legitimately diverge" % t)
+        tok = nxt
+    # the same picks again without logits, after a reset, in one call
+    gpu.reset_kv_caches()
+    gpu.forward(prompt, all_rows=False)
+    assert np.array_equal(gpu.decode_greedy(first, n), ids)
+
+
+def test_layered_operator_path_matches_fused_path_and_oracle():
+    params = synth.make_params(TINY, seed=14, std=0.1, gains_one=False)
+    layered = LayeredLlamaModel(TINY, params)
+    ora = lo.Llama(TINY, params)
+    fused = LlamaModel(TINY)
+    fused.load_params(params)
+    ids = synth.make_tokens(20, TINY["vocab_size"], seed=14)
+    caches = layered.init_kv_caches(1)
+    a = layered.forward(ids[:15], caches).data()[0]
+    rc, r = ora.forward(ids[:15])
+    assert max_rel(a, r) <= 1e-4
+    assert max_rel(fused.forward(ids[:15]), r) <= 1e-4
+    for t in range(15, 20):
+        a = layered.forward(ids[t:t + 1], caches).data()[0, 0]
+        rc, r = ora.forward(ids[t:t + 1])
+        assert max_rel(a, r[0]) <= 1e-4
+        assert max_rel(fused.forward(ids[t:t + 1], all_rows=False), r[0]) <= 1e-4
+    assert caches[0].len == 20
+    with pytest.raises(_lib.LumenError) as e:
+        layered.forward(ids[:1], caches[:-1])  # llama.rs:182-188
+    assert e.value.status == _lib.ERR_CACHE_COUNT
+
+
+def test_status_codes_for_overflow_oob_and_bad_params():
+    gpu, ora, params = build(TINY, seed=15)
+    ids = synth.make_tokens(TINY["max_seq_len"], TINY["vocab_size"], seed=15)
+    gpu.forward(ids[:-1], all_rows=False)
+    gpu.forward(ids[-1:], all_rows=False)
+    assert gpu.kv_len == TINY["max_seq_len"]
+    for call in (lambda: gpu.forward(ids[:1]), lambda: gpu.decode_greedy(1, 1)):
+        with pytest.raises(_lib.LumenError) as e:
+            call()
+        assert e.value.status == _lib.ERR_KV_OVERFLOW
+    gpu.reset_kv_caches()
+    with pytest.raises(_lib.LumenError) as e:
+        gpu.forward(np.array([TINY["vocab_size"]]))
+    assert e.value.status == _lib.ERR_EMBED_OOB and gpu.kv_len == 0
+    with pytest.raises(_lib.LumenError) as e:
+        gpu.set_param("model.layers.0.mlp.up_proj.weight", np.zeros((3, 3), np.float32))
+    assert e.value.status == _lib.ERR_SHAPE
+    with pytest.raises(_lib.LumenError) as e:
+        gpu.set_param("model.layers.99.mlp.up_proj.weight", np.zeros((3, 3), np.float32))
+    assert e.value.status == _lib.ERR_INVALID
+    with pytest.raises(_lib.LumenError) as e:
+        gpu.forward(ids[:2], caches=[0])
+    assert e.value.status == _lib.ERR_CACHE_COUNT
+
+
+@pytest.mark.slow
+def test_tinyllama_1b_shape_prefill_128_decode_teacher_forced():
+    """The headline configuration at full size: 22 layers, hidden 2048, 32/4 heads, vocab 32000,
+    128 random prompt ids then teacher-forced decode; per-step logits within 1e-4."""
+    cfg = synth.TINYLLAMA_1B
+    gpu = LlamaModel(cfg)
+    params = {}
+    for name, a in synth.iter_params(cfg, seed=0):
+        gpu.set_param(name, a)
+        params[name] = a
+    ora = lo.Llama(cfg, params)
+    ids = synth.make_tokens(128 + 16, cfg["vocab_size"], seed=0)
+    got = gpu.forward(ids[:128], all_rows=False)
+    rc, ref = ora.forward(ids[:128])
+    assert rc == lo.LO_OK
+    assert max_rel(got, ref[-1]) <= 1e-4
+    worst = 0.0
+    for t in range(128, 144):
+        g = gpu.forward(ids[t:t + 1], all_rows=False)
+        rc, r = ora.forward(ids[t:t + 1])
+        worst = max(worst, max_rel(g, r[0]))
+        check_argmax(g, r[0], 1e-4)
+    assert worst <= 1e-4, worst
+    # on-device greedy loop reproduces itself and advances the cache
+    a = gpu.decode_greedy(int(ids[0]), 8)
+    assert gpu.kv_len == 144 + 8 and a.shape == (8,)

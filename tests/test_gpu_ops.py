@@ -1,0 +1,145 @@
+"""GPU parity: GEMV / GEMM / RMSNorm / elementwise / embedding / argmax / RoPE against the CPU oracle.
+
+Tolerances: GEMV and GEMM max|d|/max|ref| <= 1e-5 (the GEMV microbenchmark's stated bound);
+RoPE, add, mul and gathers bit-exact; SiLU / RMSNorm within a few f32 ulp.
+"""
+import numpy as np
+import pytest
+
+from lumen_amd import _lib, ops
+from lumen_amd.autograd import Tensor
+from lumen_amd.layers import Embedding, Linear, RMSNorm, RotaryEmbedding, SiLU
+from oracle import lumen_oracle as lo
+from tests.gpu_util import dev, f32, max_rel
+
+pytestmark = pytest.mark.gpu
+RNG = np.random.default_rng(99)
+
+MICROBENCH = [(2048, 2048), (2048, 256), (2048, 5632), (5632, 2048), (2048, 32000), (4096, 11008), (11008, 4096)]
+
+
+@pytest.mark.parametrize("K,N", MICROBENCH)
+def test_gemv_microbench_shapes(K, N):
+    rng = np.random.default_rng(K * 100003 + N)
+    W = f32(rng.standard_normal((N, K), dtype=np.float32) * 0.02)  # logical (K, N), stored [N, K]
+    x = f32(rng.standard_normal(K, dtype=np.float32))
+    y = ops.matmul(dev(x.reshape(1, 1, K)), dev(W)).data().reshape(-1)
+    ref = lo.gemv(W, x)
+    assert max_rel(y, ref) <= 1e-5
+    ref64 = W.astype(np.float64) @ x.astype(np.float64)
+    assert max_rel(y, ref64) <= 1e-5
+
+
+@pytest.mark.parametrize("N,K", [(1, 4), (3, 8), (5, 260), (7, 1000), (64, 12), (33, 37), (2, 1), (130, 513), (9, 20000)])
+def test_gemv_ragged_shapes(N, K):
+    W = f32(RNG.normal(0, 1, (N, K)))
+    x = f32(RNG.normal(0, 1, K))
+    y = Linear(dev(W)).forward(dev(x.reshape(1, K))).data().reshape(-1)
+    assert max_rel(y, lo.gemv(W, x)) <= 1e-5
+
+
+def test_gemv_known_answers():
+    K = 512
+    x = f32(RNG.normal(0, 1, K))
+    assert np.array_equal(ops.matmul(dev(x[None]), dev(np.eye(K, dtype=np.float32))).data()[0], x)
+    e = np.zeros(K, np.float32)
+    e[77] = 1.0
+    W = f32(RNG.normal(0, 1, (40, K)))
+    assert np.array_equal(ops.matmul(dev(e[None]), dev(W)).data()[0], W[:, 77])
+
+
+@pytest.mark.parametrize("N,K", [(256, 2048), (100, 520), (11, 8), (6, 1003)])
+def test_gemv_bf16_weights(N, K):
+    W = f32(RNG.normal(0, 0.02, (N, K)))
+    bits = lo.f32_to_bf16(W)
+    x = f32(RNG.normal(0, 1, K))
+    y = ops.matmul(dev(x[None]), dev(bits)).data()[0]
+    ref = lo.gemv(lo.bf16_to_f32(bits), x)  # the reference's side: same bf16 values widened (loader.rs:58)
+    assert max_rel(y, ref) <= 1e-5
+
+
+def test_matmul_shape_errors_and_empty():
+    a = dev(np.zeros((1, 7), np.float32))
+    with pytest.raises(_lib.LumenError) as e:
+        ops.matmul(a, dev(np.zeros((5, 8), np.float32)))
+    assert e.value.status == _lib.ERR_SHAPE
+    with pytest.raises(_lib.LumenError) as e:
+        ops.matmul(a, dev(np.zeros((2, 2, 2), np.float32)))
+    assert e.value.status == _lib.ERR_SHAPE
+    out = ops.matmul(dev(np.zeros((0, 8), np.float32)), dev(np.zeros((5, 8), np.float32)))
+    assert out.shape == (0, 5)
+
+
+@pytest.mark.parametrize("M,N,K", [(2, 3, 4), (7, 33, 132), (128, 256, 2048), (130, 200, 64), (64, 5632, 512),
+                                   (5, 9, 7), (300, 129, 260), (16, 2560, 2048)])
+def test_gemm_against_oracle(M, N, K):
+    A = f32(RNG.normal(0, 1, (1, M, K)))
+    W = f32(RNG.normal(0, 0.02, (N, K)))
+    C = ops.matmul(dev(A), dev(W)).data()[0]
+    assert C.shape == (M, N)
+    ref = lo.gemm(A[0], W)
+    assert max_rel(C, ref) <= 1e-5
+    assert max_rel(C, A[0].astype(np.float64) @ W.T.astype(np.float64)) <= 1e-5
+
+
+def test_gemm_bf16_weights():
+    M, N, K = 48, 300, 256
+    A = f32(RNG.normal(0, 1, (M, K)))
+    bits = lo.f32_to_bf16(f32(RNG.normal(0, 0.02, (N, K))))
+    C = ops.matmul(dev(A), dev(bits)).data()
+    assert max_rel(C, lo.gemm(A, lo.bf16_to_f32(bits))) <= 1e-5
+
+
+@pytest.mark.parametrize("rows,dim,eps", [(1, 2048, 1e-5), (7, 100, 1e-6), (128, 2048, 1e-5), (3, 1, 1e-5)])
+def test_rmsnorm(rows, dim, eps):
+    x = f32(RNG.normal(0, 2, (rows, dim)))
+    w = f32(RNG.normal(1, 0.2, dim))
+    out = RMSNorm(dim, eps, w).forward(dev(x)).data()
+    assert np.allclose(out, lo.rmsnorm(x, w, eps), rtol=3e-6, atol=1e-7)
+
+
+def test_elementwise_and_swiglu():
+    x = f32(np.concatenate([RNG.normal(0, 3, 5000), [0.0, -100.0, 100.0, -20.0, 20.0]]))
+    y = f32(RNG.normal(0, 1, x.size))
+    assert np.allclose(SiLU().forward(dev(x)).data(), lo.silu(x), rtol=3e-6, atol=1e-30)
+    assert np.array_equal((dev(x) + dev(y)).data(), lo.add(x, y))
+    assert np.array_equal((dev(x) * dev(y)).data(), lo.mul(x, y))
+    assert np.allclose(ops.swiglu(dev(x), dev(y)).data(), lo.mul(lo.silu(x), y), rtol=3e-6, atol=1e-30)
+    with pytest.raises(_lib.LumenError):
+        dev(x) + dev(y[:10])
+    assert (dev(x[:0]) + dev(y[:0])).data().size == 0
+
+
+def test_embedding_and_argmax():
+    W = f32(RNG.normal(0, 1, (50, 24)))
+    emb = Embedding(dev(W))
+    ids = np.array([[3.0, 0.0, 49.0, 3.0, 2.9]], np.float32)
+    assert np.array_equal(emb.forward(ids).data(), lo.embedding(W, ids)[1])
+    with pytest.raises(_lib.LumenError) as e:
+        emb.forward(np.array([50.0], np.float32))
+    assert e.value.status == _lib.ERR_EMBED_OOB
+    v = f32(RNG.normal(0, 1, 32000))
+    v[[123, 20000]] = 9.0
+    assert ops.argmax(dev(v)) == lo.argmax(v) == 123
+    assert ops.argmax(dev(f32([-1.0]))) == 0
+
+
+@pytest.mark.parametrize("dim,max_seq,theta", [(64, 2048, 10000.0), (128, 300, 1.0e6), (16, 32, 10000.0)])
+def test_rope_tables_and_rotation_bit_exact(dim, max_seq, theta):
+    rope = RotaryEmbedding(dim, max_seq, theta)
+    cos, sin = rope.tables()
+    ocos, osin = lo.rope_table(dim, max_seq, theta)
+    assert np.array_equal(cos, ocos) and np.array_equal(sin, osin)
+    x = f32(RNG.normal(0, 1, (1, 3, 5, dim)))
+    off = max_seq - 5
+    assert np.array_equal(rope.forward(dev(x), off).data(), lo.rope_forward(x, ocos, osin, off)[1])
+    with pytest.raises(_lib.LumenError) as e:
+        rope.forward(dev(x), off + 1)
+    assert e.value.status == _lib.ERR_ROPE_RANGE
+    src = f32(RNG.normal(0, 1, dim))
+    dst = Tensor.empty((dim,))
+    rope.rope_1token_copy(dev(src), dst, 7)
+    assert np.array_equal(dst.data(), lo.rope_1token_copy(src, ocos, osin, 7)[1])
+    with pytest.raises(_lib.LumenError) as e:
+        rope.rope_1token_copy(dev(src), dst, max_seq)
+    assert e.value.status == _lib.ERR_ROPE_RANGE
