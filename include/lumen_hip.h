@@ -190,6 +190,12 @@ int lumen_llama_forward(lumen_llama *model, const float *ids_host, int s, float 
  * ids_out_host [n] receives the picks; logits_out_host [n, V] is optional. */
 int lumen_llama_decode_greedy(lumen_llama *model, int first_id, int n, int32_t *ids_out_host,
                               float *logits_out_host);
+/* measurement aid (no reference counterpart): n greedy steps launched kernel by
+ * kernel, every launch bracketed by HIP events on the ctx stream.  Classes:
+ * 0 embedding, 1 norm+q|k|v GEMV, 2 decode attention, 3 o_proj GEMV, 4 norm+gate|up
+ * GEMV, 5 down GEMV, 6 norm+lm_head GEMV, 7 argmax.  ms_sum_out / count_out [n_classes >= 8]. */
+int lumen_llama_decode_profile(lumen_llama *model, int first_id, int n, double *ms_sum_out,
+                               int *count_out, int n_classes);
 int lumen_llama_reset(lumen_llama *model);                      /* reset_kv_caches, llama.rs:172-176 */
 int lumen_llama_kv_len(const lumen_llama *model, int *len_out);
 int lumen_llama_cache_download(lumen_llama *model, int layer, float *k_host, float *v_host);

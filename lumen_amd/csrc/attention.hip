@@ -176,8 +176,11 @@ __device__ __forceinline__ void norm_rope_heads(const float *raw, float *rot, in
             x2 = x2 * inv * g[j + HALF];
         }
         const float c = cs[j], s = sn[j];
-        rot[r * D + j] = __fsub_rn(__fmul_rn(x1, c), __fmul_rn(x2, s));
-        rot[r * D + j + HALF] = __fadd_rn(__fmul_rn(x1, s), __fmul_rn(x2, c));
+        {
+#pragma clang fp contract(off)  // separate multiplies and add, like the reference's compiled code
+            rot[r * D + j] = x1 * c - x2 * s;
+            rot[r * D + j + HALF] = x1 * s + x2 * c;
+        }
     }
 }
 

@@ -189,8 +189,11 @@ __global__ __launch_bounds__(256) void rope_bhsd_kernel(const float *__restrict_
         const float x1 = xr[j], x2 = xr[j + half];
         const float c = cos_t[(size_t)(offset + ss) * d + j];
         const float sv = sin_t[(size_t)(offset + ss) * d + j];
-        out[row * d + j] = __fsub_rn(__fmul_rn(x1, c), __fmul_rn(x2, sv));
-        out[row * d + j + half] = __fadd_rn(__fmul_rn(x2, c), __fmul_rn(x1, sv));
+        {
+#pragma clang fp contract(off)  // separate multiplies and add, like the reference's compiled code
+            out[row * d + j] = x1 * c - x2 * sv;
+            out[row * d + j + half] = x2 * c + x1 * sv;
+        }
     }
 }
 

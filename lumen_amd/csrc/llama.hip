@@ -311,18 +311,47 @@ extern "C" int lumen_llama_set_param(lumen_llama *m, const char *name, const voi
 // ------------------------------------------------------------------- decode
 // One token through all layers; every launch reads the token id and the
 // position from device memory, so the sequence is the same for every token.
-static int enqueue_decode_step(lumen_llama *m) {
+// Kernel classes of a decode step, for per-kernel timing.
+enum { KC_EMBED = 0, KC_QKV, KC_ATTN, KC_OPROJ, KC_GATEUP, KC_DOWN, KC_LMHEAD, KC_ARGMAX, KC_COUNT };
+
+struct StepProbe {  // brackets every launch with a HIP event pair when profiling
+    std::vector<hipEvent_t> ev;
+    std::vector<int> cls;
+    hipStream_t s = nullptr;
+    bool on = false;
+    void before(int c) {
+        if (!on) return;
+        hipEvent_t e0, e1;
+        hipEventCreate(&e0);
+        hipEventCreate(&e1);
+        ev.push_back(e0);
+        ev.push_back(e1);
+        cls.push_back(c);
+        hipEventRecord(e0, s);
+    }
+    void after() {
+        if (on) hipEventRecord(ev.back(), s);
+    }
+};
+
+static int enqueue_decode_step(lumen_llama *m, StepProbe *pr = nullptr) {
+    StepProbe none;
+    if (!pr) pr = &none;
     lumen_ctx *ctx = m->ctx;
     const lumen_llama_config &c = m->cfg;
     const int H = c.hidden_size, I = c.intermediate_size, V = c.vocab_size;
+    pr->before(KC_EMBED);
     LUMEN_TRY(launch_embedding(ctx, m->embed, m->d_tok, 1, H, V, m->x));  // llama.rs:191
+    pr->after();
     for (int l = 0; l < c.num_hidden_layers; ++l) {
         const LayerW &w = m->layers[l];
         GemvArgs g = {};
         // input_layernorm + q|k|v projections, llama.rs:107, self_attention.rs:106-108
         g.W = w.wqkv; g.x = m->x; g.y = m->qkv; g.N = m->qkvd; g.K = H; g.w_bf16 = m->bf16;
         g.pro = PRO_RMSNORM; g.norm_w = w.in_norm; g.eps = c.rms_norm_eps; g.epi = EPI_STORE;
+        pr->before(KC_QKV);
         LUMEN_TRY(launch_gemv(ctx, g));
+        pr->after();
         AttnDecodeArgs a = {};
         a.q = m->qkv; a.k_new = m->qkv + m->qd; a.v_new = m->qkv + m->qd + m->kvd; a.out = m->attn;
         a.k_cache = m->k_slab + m->cache_stride * l; a.v_cache = m->v_slab + m->cache_stride * l;
@@ -330,31 +359,44 @@ static int enqueue_decode_step(lumen_llama *m) {
         a.b = 1; a.hq = c.num_attention_heads; a.hkv = c.num_key_value_heads; a.d = m->D; a.max_seq = c.max_seq_len;
         a.scale = m->scale; a.q_norm_w = w.q_norm; a.k_norm_w = w.k_norm; a.norm_eps = c.rms_norm_eps;
         a.part = m->part; a.counters = m->counters; a.nsplit = m->nsplit;
+        pr->before(KC_ATTN);
         LUMEN_TRY(launch_attn_decode(ctx, a));
+        pr->after();
         // o_proj + residual, self_attention.rs:303, llama.rs:110
         g = {};
         g.W = w.wo; g.x = m->attn; g.y = m->h; g.N = H; g.K = m->qd; g.w_bf16 = m->bf16;
         g.pro = PRO_NONE; g.epi = EPI_RESIDUAL; g.residual = m->x;
+        pr->before(KC_OPROJ);
         LUMEN_TRY(launch_gemv(ctx, g));
+        pr->after();
         // post_attention_layernorm + gate|up + silu*up, llama.rs:113, :60-63
         g = {};
         g.W = w.wgu; g.x = m->h; g.y = m->act; g.N = 2 * I; g.K = H; g.w_bf16 = m->bf16;
         g.pro = PRO_RMSNORM; g.norm_w = w.post_norm; g.eps = c.rms_norm_eps; g.epi = EPI_SWIGLU;
+        pr->before(KC_GATEUP);
         LUMEN_TRY(launch_gemv(ctx, g));
+        pr->after();
         // down_proj + residual, llama.rs:64, :115
         g = {};
         g.W = w.wdown; g.x = m->act; g.y = m->x; g.N = H; g.K = I; g.w_bf16 = m->bf16;
         g.pro = PRO_NONE; g.epi = EPI_RESIDUAL; g.residual = m->h;
+        pr->before(KC_DOWN);
         LUMEN_TRY(launch_gemv(ctx, g));
+        pr->after();
     }
     // final norm + lm_head, llama.rs:202-205
     GemvArgs g = {};
     g.W = m->lm_head; g.x = m->x; g.y = m->logits; g.N = V; g.K = H;
     g.w_bf16 = (m->lm_head == (void *)m->embed) ? 0 : (int)m->bf16;
     g.pro = PRO_RMSNORM; g.norm_w = m->final_norm; g.eps = c.rms_norm_eps; g.epi = EPI_STORE;
+    pr->before(KC_LMHEAD);
     LUMEN_TRY(launch_gemv(ctx, g));
+    pr->after();
     // greedy pick becomes the next token id; the position counter advances
-    return launch_argmax(ctx, m->logits, V, m->d_tok, m->d_pos);
+    pr->before(KC_ARGMAX);
+    const int rc = launch_argmax(ctx, m->logits, V, m->d_tok, m->d_pos);
+    pr->after();
+    return rc;
 }
 
 static int ensure_decode_graph(lumen_llama *m) {
@@ -540,6 +582,48 @@ extern "C" int lumen_llama_decode_greedy(lumen_llama *m, int first_id, int n, in
         e = hipMemcpy(ids_out, ids_dev, sizeof(int) * (size_t)n, hipMemcpyDeviceToHost);
     hipFree(ids_dev);
     if (rc == LUMEN_OK && e != hipSuccess) LUMEN_FAIL(LUMEN_ERR_HIP, "decode_greedy: %s", hipGetErrorString(e));
+    return rc;
+}
+
+// n greedy decode steps launched kernel by kernel (no graph), each launch
+// bracketed by HIP events on the ctx stream: per kernel class the summed
+// event-to-event milliseconds and the launch count.
+extern "C" int lumen_llama_decode_profile(lumen_llama *m, int first_id, int n, double *ms_sum_out, int *count_out,
+                                          int n_classes) {
+    if (!m || !ms_sum_out || !count_out) LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_decode_profile: null argument");
+    if (n_classes < KC_COUNT) LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_decode_profile: need %d classes", (int)KC_COUNT);
+    if (first_id < 0 || first_id >= m->cfg.vocab_size)
+        LUMEN_FAIL(LUMEN_ERR_EMBED_OOB, "Embedding index out of bounds: %d >= %d", first_id, m->cfg.vocab_size);
+    for (int i = 0; i < n_classes; ++i) { ms_sum_out[i] = 0.0; count_out[i] = 0; }
+    if (n <= 0) return LUMEN_OK;
+    HIP_TRY(hipSetDevice(m->ctx->device));
+    LUMEN_TRY(check_room(m, n));
+    hipStream_t st = m->ctx->stream;
+    HIP_TRY(hipMemcpyAsync(m->d_tok, &first_id, sizeof(int), hipMemcpyHostToDevice, st));
+    HIP_TRY(hipStreamSynchronize(st));
+    int rc = LUMEN_OK;
+    for (int t = 0; t < n && rc == LUMEN_OK; ++t) {
+        StepProbe pr;
+        pr.on = true;
+        pr.s = st;
+        rc = enqueue_decode_step(m, &pr);
+        const hipError_t e = hipStreamSynchronize(st);
+        if (rc == LUMEN_OK && e == hipSuccess) {
+            m->len += 1;
+            for (size_t i = 0; i < pr.cls.size(); ++i) {
+                float ms = 0.f;
+                if (hipEventElapsedTime(&ms, pr.ev[2 * i], pr.ev[2 * i + 1]) == hipSuccess) {
+                    ms_sum_out[pr.cls[i]] += ms;
+                    count_out[pr.cls[i]] += 1;
+                }
+            }
+        }
+        for (hipEvent_t ev : pr.ev) hipEventDestroy(ev);
+        if (rc == LUMEN_OK && e != hipSuccess) {
+            lumen_set_error("decode_profile step %d: %s", t, hipGetErrorString(e));
+            rc = LUMEN_ERR_HIP;
+        }
+    }
     return rc;
 }
 

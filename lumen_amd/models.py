@@ -127,6 +127,17 @@ class LlamaModel:
                                             logits.ctypes.data if want_logits else None))
         return (ids, logits) if want_logits else ids
 
+    KERNEL_CLASSES = ("embedding", "norm_qkv_gemv", "attn_decode", "oproj_gemv", "norm_gateup_gemv", "down_gemv",
+                      "norm_lmhead_gemv", "argmax")
+
+    def decode_profile(self, first_id, n):
+        """n greedy steps with every launch bracketed by HIP events: {class: (ms_sum, launches)}."""
+        k = len(self.KERNEL_CLASSES)
+        ms = (C.c_double * k)()
+        cnt = (C.c_int * k)()
+        check(lib.lumen_llama_decode_profile(self.handle, int(first_id), int(n), ms, cnt, k))
+        return {name: (ms[i], cnt[i]) for i, name in enumerate(self.KERNEL_CLASSES)}
+
     def decode_bytes(self, length):
         b = C.c_double()
         check(lib.lumen_llama_decode_bytes(self.handle, int(length), C.byref(b)))

@@ -24,14 +24,16 @@ TOL = 2e-5
 
 def gpu_decode(cache, rope, q, k, v, h, scale):
     out = Tensor.empty((q.shape[0], 1, h, q.shape[-1]))
-    check(lib.lumen_attn_decode_f32(cache.handle, rope.handle, dev(q).ptr, dev(k).ptr, dev(v).ptr, out.ptr, h, scale, 1))
+    qd, kd, vd = dev(q), dev(k), dev(v)  # keep the device buffers alive across the call
+    check(lib.lumen_attn_decode_f32(cache.handle, rope.handle, qd.ptr, kd.ptr, vd.ptr, out.ptr, h, scale, 1))
     return out.data()
 
 
 def gpu_prefill(cache, rope, q, k, v, scale):
     b, s, h, d = q.shape
     out = Tensor.empty((b, s, h, d))
-    check(lib.lumen_attn_prefill_f32(cache.handle, rope.handle, dev(q).ptr, dev(k).ptr, dev(v).ptr, out.ptr, s, h, scale, 1))
+    qd, kd, vd = dev(q), dev(k), dev(v)
+    check(lib.lumen_attn_prefill_f32(cache.handle, rope.handle, qd.ptr, kd.ptr, vd.ptr, out.ptr, s, h, scale, 1))
     return out.data()
 
 

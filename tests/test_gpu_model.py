@@ -9,6 +9,7 @@ import numpy as np
 import pytest
 
 from lumen_amd import _lib, synth
+from lumen_amd.autograd import no_grad
 from lumen_amd.models import LayeredLlamaModel, LlamaModel
 from oracle import lumen_oracle as lo
 from tests.gpu_util import max_rel
@@ -120,6 +121,13 @@ def test_layered_operator_path_matches_fused_path_and_oracle():
     fused.load_params(params)
     ids = synth.make_tokens(20, TINY["vocab_size"], seed=14)
     caches = layered.init_kv_caches(1)
+    with pytest.raises(NotImplementedError):  # outside no_grad the reference takes its train path
+        layered.forward(ids[:15], caches)
+    with no_grad():  # main.rs:255
+        _layered_checks(layered, fused, ora, ids, caches)
+
+
+def _layered_checks(layered, fused, ora, ids, caches):
     a = layered.forward(ids[:15], caches).data()[0]
     rc, r = ora.forward(ids[:15])
     assert max_rel(a, r) <= 1e-4
