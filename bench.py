@@ -32,6 +32,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--prompt", type=int, default=128)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--mode", choices=["graph", "eager"], default="graph",
+                    help="how decode steps are issued: a HIP graph replay per token (default) or kernel by kernel "
+                         "(for rocprofv3 --kernel-trace, which cannot follow graph replays here)")
     ap.add_argument("--cpu-tokens", type=int, default=48)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -50,6 +53,7 @@ def main():
 
     t0 = time.time()
     model = LlamaModel(cfg)
+    model.set_decode_mode(args.mode)
     keep_host = not args.no_cpu_baseline
     params = {}
     for name, a in synth.iter_params(cfg, seed=0):
@@ -112,7 +116,7 @@ def main():
                           "roofline_tokens_per_s": round(HBM_PEAK_GBS * 1e9 / step_bytes, 1)},
         "kernels": kernels,
         "prefill": {"tokens": args.prompt, "ms": round(prefill_ms, 3), "tokens_per_s": round(args.prompt / prefill_ms * 1e3, 1)},
-        "wall_s_timed_region": round(wall, 4), "setup_s": round(t_setup, 1),
+        "decode_mode": args.mode, "wall_s_timed_region": round(wall, 4), "setup_s": round(t_setup, 1),
     }
 
     if not args.no_cpu_baseline:

@@ -196,6 +196,16 @@ int lumen_llama_decode_greedy(lumen_llama *model, int first_id, int n, int32_t *
  * GEMV, 5 down GEMV, 6 norm+lm_head GEMV, 7 argmax.  ms_sum_out / count_out [n_classes >= 8]. */
 int lumen_llama_decode_profile(lumen_llama *model, int first_id, int n, double *ms_sum_out,
                                int *count_out, int n_classes);
+/* how S == 1 steps are issued (no reference counterpart; the results are the same):
+ * PERSISTENT (default when head_dim is 64 or 128): one cooperative kernel runs all
+ * layers of all requested steps, weights of the next stage streaming across each
+ * grid barrier; GRAPH: one captured HIP graph replay per token (5 kernels per layer);
+ * EAGER: the same kernels launched one by one (for kernel tracing tools). */
+#define LUMEN_DECODE_EAGER 0
+#define LUMEN_DECODE_GRAPH 1
+#define LUMEN_DECODE_PERSISTENT 2
+int lumen_llama_set_decode_mode(lumen_llama *model, int mode);
+int lumen_llama_get_decode_mode(const lumen_llama *model, int *mode_out);
 int lumen_llama_reset(lumen_llama *model);                      /* reset_kv_caches, llama.rs:172-176 */
 int lumen_llama_kv_len(const lumen_llama *model, int *len_out);
 int lumen_llama_cache_download(lumen_llama *model, int layer, float *k_host, float *v_host);

@@ -12,6 +12,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "liblumen_hip.so")
 OK, ERR_SHAPE, ERR_KV_OVERFLOW, ERR_ROPE_RANGE, ERR_EMBED_OOB, ERR_CACHE_COUNT, ERR_INVALID, ERR_HIP, \
     ERR_NO_DEVICE, ERR_UNSUPPORTED = range(10)
 DTYPE_F32, DTYPE_BF16 = 0, 1
+DECODE_EAGER, DECODE_GRAPH, DECODE_PERSISTENT = 0, 1, 2
 
 STATUS_NAMES = {OK: "OK", ERR_SHAPE: "SHAPE", ERR_KV_OVERFLOW: "KV_OVERFLOW", ERR_ROPE_RANGE: "ROPE_RANGE",
                 ERR_EMBED_OOB: "EMBED_OOB", ERR_CACHE_COUNT: "CACHE_COUNT", ERR_INVALID: "INVALID",
@@ -83,6 +84,8 @@ SIGNATURES = {
     "lumen_llama_forward": (_i, [_vp, _vp, _i, _vp, _i]),
     "lumen_llama_decode_greedy": (_i, [_vp, _i, _i, _vp, _vp]),
     "lumen_llama_decode_profile": (_i, [_vp, _i, _i, C.POINTER(C.c_double), C.POINTER(_i), _i]),
+    "lumen_llama_set_decode_mode": (_i, [_vp, _i]),
+    "lumen_llama_get_decode_mode": (_i, [_vp, C.POINTER(_i)]),
     "lumen_llama_reset": (_i, [_vp]),
     "lumen_llama_kv_len": (_i, [_vp, C.POINTER(_i)]),
     "lumen_llama_cache_download": (_i, [_vp, _i, _vp, _vp]),

@@ -13,182 +13,14 @@
 //    append to the cache, then one workgroup per (query position, KV group)
 //    runs the same row loop over the causal prefix.
 #include "internal.h"
+#include "attn_device.h"
 
-#include <cmath>
-
-typedef float v4f __attribute__((ext_vector_type(4)));
-
-#define ATT_THREADS 256
 #define ATT_WAVES 4
-
-template <int NREP>
-struct AttnState {
-    float m[NREP], l[NREP];
-    v4f acc[NREP];
-};
-
-template <int NREP>
-__device__ __forceinline__ void state_init(AttnState<NREP> &st) {
-#pragma unroll
-    for (int r = 0; r < NREP; ++r) {
-        st.m[r] = -INFINITY;
-        st.l[r] = 0.f;
-        st.acc[r] = (v4f){0.f, 0.f, 0.f, 0.f};
-    }
-}
-
-// One K/V row piece per lane: score for each of the NREP heads, online-softmax update.
-template <int D, int NREP>
-__device__ __forceinline__ void attn_step(AttnState<NREP> &st, const v4f (&q)[NREP], const v4f kv, const v4f vv,
-                                          bool valid, float scale) {
-    constexpr int LPR = D / 4;
-#pragma unroll
-    for (int r = 0; r < NREP; ++r) {
-        float s = q[r].x * kv.x;
-        s = fmaf(q[r].y, kv.y, s);
-        s = fmaf(q[r].z, kv.z, s);
-        s = fmaf(q[r].w, kv.w, s);
-#pragma unroll
-        for (int off = LPR / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
-        s = valid ? s * scale : -INFINITY;
-        const float m_new = fmaxf(st.m[r], s);
-        if (m_new > -INFINITY) {
-            const float alpha = expf(st.m[r] - m_new);  // exp(-inf) = 0 on the first row
-            const float p = expf(s - m_new);
-            st.l[r] = fmaf(st.l[r], alpha, p);
-            st.acc[r].x = fmaf(st.acc[r].x, alpha, p * vv.x);
-            st.acc[r].y = fmaf(st.acc[r].y, alpha, p * vv.y);
-            st.acc[r].z = fmaf(st.acc[r].z, alpha, p * vv.z);
-            st.acc[r].w = fmaf(st.acc[r].w, alpha, p * vv.w);
-            st.m[r] = m_new;
-        }
-    }
-}
-
-// Rows [p0, p1) of one KV head (Kb/Vb point at row 0), spread over the
-// workgroup's 4 wavefronts x (64/LPR) lane groups.
-template <int D, int NREP>
-__device__ __forceinline__ void attn_rows(AttnState<NREP> &st, const v4f (&q)[NREP], const float *__restrict__ Kb,
-                                          const float *__restrict__ Vb, int p0, int p1, float scale) {
-    constexpr int LPR = D / 4;
-    constexpr int RPW = 64 / LPR;
-    constexpr int RPI = ATT_WAVES * RPW;  // rows per workgroup iteration
-    constexpr int U = 4;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int slot = lane / LPR, c = lane % LPR;
-    const int off = wave * RPW + slot;
-    for (int base = p0; base < p1; base += RPI * U) {  // trip count is uniform over the workgroup
-        v4f kv[U], vv[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int j = base + u * RPI + off;
-            kv[u] = (v4f){0.f, 0.f, 0.f, 0.f};
-            vv[u] = (v4f){0.f, 0.f, 0.f, 0.f};
-            if (j < p1) {
-                kv[u] = *(const v4f *)(Kb + (size_t)j * D + c * 4);
-                vv[u] = *(const v4f *)(Vb + (size_t)j * D + c * 4);
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            // uniform test: every lane of the wavefront takes the step (it shuffles), rows past p1 are masked
-            if (base + u * RPI < p1) attn_step<D, NREP>(st, q, kv[u], vv[u], base + u * RPI + off < p1, scale);
-        }
-    }
-}
-
-// Merge the lane-group states of each wavefront and publish one state per
-// wavefront in LDS (sm, sl [ATT_WAVES][NREP]; sacc [ATT_WAVES][NREP][D]).
-// Ends with a workgroup barrier; wave_fold() then combines the wavefronts.
-template <int D, int NREP>
-__device__ __forceinline__ void block_merge(AttnState<NREP> &st, float *sm, float *sl, float *sacc) {
-    constexpr int LPR = D / 4;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int slot = lane / LPR, c = lane % LPR;
-#pragma unroll
-    for (int r = 0; r < NREP; ++r) {
-#pragma unroll
-        for (int off = LPR; off < 64; off <<= 1) {
-            const float mo = __shfl_xor(st.m[r], off, 64);
-            const float lo = __shfl_xor(st.l[r], off, 64);
-            v4f ao;
-            ao.x = __shfl_xor(st.acc[r].x, off, 64);
-            ao.y = __shfl_xor(st.acc[r].y, off, 64);
-            ao.z = __shfl_xor(st.acc[r].z, off, 64);
-            ao.w = __shfl_xor(st.acc[r].w, off, 64);
-            const float mn = fmaxf(st.m[r], mo);
-            const float a = (mn > -INFINITY) ? expf(st.m[r] - mn) : 0.f;
-            const float b = (mn > -INFINITY) ? expf(mo - mn) : 0.f;
-            st.l[r] = st.l[r] * a + lo * b;
-            st.acc[r].x = st.acc[r].x * a + ao.x * b;
-            st.acc[r].y = st.acc[r].y * a + ao.y * b;
-            st.acc[r].z = st.acc[r].z * a + ao.z * b;
-            st.acc[r].w = st.acc[r].w * a + ao.w * b;
-            st.m[r] = mn;
-        }
-        if (slot == 0) {
-            if (c == 0) {
-                sm[wave * NREP + r] = st.m[r];
-                sl[wave * NREP + r] = st.l[r];
-            }
-            *(v4f *)(sacc + ((size_t)(wave * NREP + r)) * D + c * 4) = st.acc[r];
-        }
-    }
-    __syncthreads();
-}
-
-// (max, sum, ctx) of head r, dim dd over the wavefront states in LDS
-template <int D, int NREP>
-__device__ __forceinline__ void wave_fold(const float *sm, const float *sl, const float *sacc, int r, int dd,
-                                          float &mm, float &ls, float &cx) {
-    mm = -INFINITY;
-#pragma unroll
-    for (int w = 0; w < ATT_WAVES; ++w) mm = fmaxf(mm, sm[w * NREP + r]);
-    ls = 0.f;
-    cx = 0.f;
-    if (mm > -INFINITY) {
-#pragma unroll
-        for (int w = 0; w < ATT_WAVES; ++w) {
-            const float ex = expf(sm[w * NREP + r] - mm);
-            ls = fmaf(sl[w * NREP + r], ex, ls);
-            cx = fmaf(sacc[((size_t)(w * NREP + r)) * D + dd], ex, cx);
-        }
-    }
-}
-
-// Optional per-head RMSNorm (gain g) then half-split RoPE of NH contiguous
-// heads held raw in LDS `raw` ([NH][D]) into `rot`.  cs/sn: table rows at the
-// token's position.  q: (x1*c - x2*s, x1*s + x2*c), self_attention.rs:220-227;
-// k: same values, encoding.rs:196-203.
-template <int D>
-__device__ __forceinline__ void norm_rope_heads(const float *raw, float *rot, int nh, const float *__restrict__ cs,
-                                                const float *__restrict__ sn, const float *__restrict__ g,
-                                                float eps) {
-    constexpr int HALF = D / 2;
-    for (int p = threadIdx.x; p < nh * HALF; p += ATT_THREADS) {
-        const int r = p / HALF, j = p % HALF;
-        float x1 = raw[r * D + j], x2 = raw[r * D + j + HALF];
-        if (g) {
-            float ss = 0.f;
-            for (int i = 0; i < D; ++i) ss = fmaf(raw[r * D + i], raw[r * D + i], ss);
-            const float inv = 1.0f / sqrtf(ss / (float)D + eps);
-            x1 = x1 * inv * g[j];
-            x2 = x2 * inv * g[j + HALF];
-        }
-        const float c = cs[j], s = sn[j];
-        {
-#pragma clang fp contract(off)  // separate multiplies and add, like the reference's compiled code
-            rot[r * D + j] = x1 * c - x2 * s;
-            rot[r * D + j + HALF] = x1 * s + x2 * c;
-        }
-    }
-}
+#define ATT_THREADS (ATT_WAVES * 64)
 
 template <int D, int NREP>
 __global__ __launch_bounds__(ATT_THREADS) void attn_decode_kernel(AttnDecodeArgs a) {
-    constexpr int LPR = D / 4;
-    constexpr int RPW = 64 / LPR;
-    constexpr int RPI = ATT_WAVES * RPW;
+    typedef AttnGeom<D, ATT_WAVES> G;
     __shared__ __align__(16) float q_raw[NREP * D];
     __shared__ __align__(16) float q_rot[NREP * D];
     __shared__ __align__(16) float k_raw[D];
@@ -199,9 +31,11 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_decode_kernel(AttnDecodeArgs
     __shared__ int s_last;
 
     const int split = blockIdx.x, hk = blockIdx.y, bb = blockIdx.z;
-    const int nsplit = gridDim.x;
     const int pos = a.pos_dev ? *a.pos_dev : a.pos_host;  // == past_len
-    const bool has_new = (split == nsplit - 1);
+    int nact, chunk;
+    decode_slices<D, ATT_WAVES>(pos, gridDim.x, nact, chunk);
+    if (split >= nact) return;
+    const bool has_new = (split == nact - 1);
     const float *cs = a.cos_t + (size_t)pos * D, *sn = a.sin_t + (size_t)pos * D;
     const size_t head_base = ((size_t)bb * a.hkv + hk) * a.max_seq * D;
 
@@ -217,8 +51,8 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_decode_kernel(AttnDecodeArgs
         }
     }
     __syncthreads();
-    norm_rope_heads<D>(q_raw, q_rot, NREP, cs, sn, a.q_norm_w, a.norm_eps);
-    if (has_new) norm_rope_heads<D>(k_raw, k_new, 1, cs, sn, a.k_norm_w, a.norm_eps);
+    norm_rope_heads<D>(q_raw, q_rot, NREP, cs, sn, a.q_norm_w, a.norm_eps, ATT_THREADS);
+    if (has_new) norm_rope_heads<D>(k_raw, k_new, 1, cs, sn, a.k_norm_w, a.norm_eps, ATT_THREADS);
     __syncthreads();
     if (has_new) {
         // self_attention.rs:161-176: rotated k and raw v go to cache row `pos`
@@ -229,39 +63,36 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_decode_kernel(AttnDecodeArgs
     }
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int slot = lane / LPR, c = lane % LPR;
+    const int slot = lane / G::LPR, c = lane % G::LPR;
     v4f q[NREP];
 #pragma unroll
     for (int r = 0; r < NREP; ++r) q[r] = *(const v4f *)(q_rot + r * D + c * 4);
 
     // this slice's share of the cached rows [0, pos)
-    int chunk = (pos + nsplit - 1) / nsplit;
-    chunk = (chunk + RPI - 1) / RPI * RPI;
     const int p0 = min(pos, split * chunk), p1 = min(pos, p0 + chunk);
-
     AttnState<NREP> st;
     state_init<NREP>(st);
-    attn_rows<D, NREP>(st, q, a.k_cache + head_base, a.v_cache + head_base, p0, p1, a.scale);
-    if (has_new) {
+    attn_rows<D, NREP, ATT_WAVES>(st, q, a.k_cache + head_base, a.v_cache + head_base, p0, p1, a.scale);
+    if (has_new && wave == 0) {
         // the new token's row comes from LDS (lane group 0 of wavefront 0)
-        const bool mine = (wave == 0 && slot == 0);
         const v4f kv = *(const v4f *)(k_new + c * 4);
         const v4f vv = *(const v4f *)(v_new + c * 4);
-        if (wave == 0) attn_step<D, NREP>(st, q, kv, vv, mine, a.scale);
+        attn_step<D, NREP>(st, q, kv, vv, slot == 0, a.scale);
     }
 
-    block_merge<D, NREP>(st, sm, sl, sacc);
+    wave_merge_publish<D, NREP>(st, sm, sl, sacc);
+    __syncthreads();
     const int t = threadIdx.x;
     for (int e = t; e < NREP * D; e += ATT_THREADS) {
         const int r = e / D, dd = e % D;
         float mm, ls, cx;
-        wave_fold<D, NREP>(sm, sl, sacc, r, dd, mm, ls, cx);
+        wave_fold<D, NREP, ATT_WAVES>(sm, sl, sacc, r, dd, mm, ls, cx);
         const int hq = hk * NREP + r;
-        if (nsplit == 1) {
+        if (nact == 1) {
             // out = ctx / (l + 1e-9), self_attention.rs:287-290
             a.out[((size_t)bb * a.hq + hq) * D + dd] = cx * (1.0f / (ls + 1e-9f));
         } else {
-            float *pp = a.part + (((size_t)bb * a.hq + hq) * nsplit + split) * (D + 2);
+            float *pp = a.part + (((size_t)bb * a.hq + hq) * gridDim.x + split) * (D + 2);
             pp[dd] = cx;
             if (dd == 0) {
                 pp[D] = mm;
@@ -269,32 +100,31 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_decode_kernel(AttnDecodeArgs
             }
         }
     }
-    if (nsplit == 1) return;
+    if (nact == 1) return;
 
     // last workgroup of this (batch, KV head) to arrive folds the slices in index order
     __threadfence();
     __syncthreads();
     if (t == 0) {
         const int old = atomicAdd(&a.counters[bb * a.hkv + hk], 1);
-        s_last = (old == nsplit - 1);
+        s_last = (old == nact - 1);
     }
     __syncthreads();
     if (!s_last) return;
-    __threadfence();
+    __threadfence();  // acquire: the other slices' partial results are visible from here on
     for (int e = t; e < NREP * D; e += ATT_THREADS) {
         const int r = e / D, dd = e % D;
         const int hq = hk * NREP + r;
-        const float *pp = a.part + (((size_t)bb * a.hq + hq) * nsplit) * (D + 2);
+        const float *pp = a.part + (((size_t)bb * a.hq + hq) * gridDim.x) * (D + 2);
         float mm = -INFINITY;
-        for (int s = 0; s < nsplit; ++s)
-            mm = fmaxf(mm, __hip_atomic_load(pp + (size_t)s * (D + 2) + D, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        for (int s = 0; s < nact; ++s) mm = fmaxf(mm, pp[(size_t)s * (D + 2) + D]);
         float ls = 0.f, cx = 0.f;
-        for (int s = 0; s < nsplit; ++s) {
-            const float ms = __hip_atomic_load(pp + (size_t)s * (D + 2) + D, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int s = 0; s < nact; ++s) {
+            const float ms = pp[(size_t)s * (D + 2) + D];
             if (ms > -INFINITY) {
                 const float ex = expf(ms - mm);
-                ls = fmaf(__hip_atomic_load(pp + (size_t)s * (D + 2) + D + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), ex, ls);
-                cx = fmaf(__hip_atomic_load(pp + (size_t)s * (D + 2) + dd, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), ex, cx);
+                ls = fmaf(pp[(size_t)s * (D + 2) + D + 1], ex, ls);
+                cx = fmaf(pp[(size_t)s * (D + 2) + dd], ex, cx);
             }
         }
         a.out[((size_t)bb * a.hq + hq) * D + dd] = cx * (1.0f / (ls + 1e-9f));
@@ -357,7 +187,7 @@ __global__ __launch_bounds__(ATT_THREADS) void prefill_rope_kernel(AttnPrefillAr
         __syncthreads();
         for (int i = threadIdx.x; i < nh * D; i += ATT_THREADS) raw[i] = qrow[(size_t)h0 * D + i];
         __syncthreads();
-        norm_rope_heads<D>(raw, rot, nh, cs, sn, a.q_norm_w, a.norm_eps);
+        norm_rope_heads<D>(raw, rot, nh, cs, sn, a.q_norm_w, a.norm_eps, ATT_THREADS);
         __syncthreads();
         for (int i = threadIdx.x; i < nh * D; i += ATT_THREADS) qo[(size_t)h0 * D + i] = rot[i];
     }
@@ -366,7 +196,7 @@ __global__ __launch_bounds__(ATT_THREADS) void prefill_rope_kernel(AttnPrefillAr
         __syncthreads();
         for (int i = threadIdx.x; i < nh * D; i += ATT_THREADS) raw[i] = krow[(size_t)h0 * D + i];
         __syncthreads();
-        norm_rope_heads<D>(raw, rot, nh, cs, sn, a.k_norm_w, a.norm_eps);
+        norm_rope_heads<D>(raw, rot, nh, cs, sn, a.k_norm_w, a.norm_eps, ATT_THREADS);
         __syncthreads();
         for (int i = threadIdx.x; i < nh * D; i += ATT_THREADS) {
             const int hk = h0 + i / D, dd = i % D;
@@ -382,7 +212,7 @@ __global__ __launch_bounds__(ATT_THREADS) void prefill_rope_kernel(AttnPrefillAr
 // out [B,S,Hq,D] (BSHD, :534).
 template <int D, int NREP>
 __global__ __launch_bounds__(ATT_THREADS) void attn_prefill_kernel(AttnPrefillArgs a) {
-    constexpr int LPR = D / 4;
+    typedef AttnGeom<D, ATT_WAVES> G;
     __shared__ __align__(16) float sacc[ATT_WAVES * NREP * D];
     __shared__ float sm[ATT_WAVES * NREP], sl[ATT_WAVES * NREP];
     const int i = blockIdx.x, hk = blockIdx.y, bb = blockIdx.z;
@@ -390,20 +220,20 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_prefill_kernel(AttnPrefillAr
     const int q_abs = a.past_len + i;
     const int p1 = a.causal ? min(L, q_abs + 1) : L;
     const size_t head_base = ((size_t)bb * a.hkv + hk) * a.max_seq * D;
-    const int lane = threadIdx.x & 63;
-    const int c = lane % LPR;
+    const int c = (threadIdx.x & 63) % G::LPR;
     const float *qr = a.q_rot + (((size_t)bb * a.s + i) * a.hq + (size_t)hk * NREP) * D;
     v4f q[NREP];
 #pragma unroll
     for (int r = 0; r < NREP; ++r) q[r] = *(const v4f *)(qr + r * D + c * 4);
     AttnState<NREP> st;
     state_init<NREP>(st);
-    attn_rows<D, NREP>(st, q, a.k_cache + head_base, a.v_cache + head_base, 0, p1, a.scale);
-    block_merge<D, NREP>(st, sm, sl, sacc);
+    attn_rows<D, NREP, ATT_WAVES>(st, q, a.k_cache + head_base, a.v_cache + head_base, 0, p1, a.scale);
+    wave_merge_publish<D, NREP>(st, sm, sl, sacc);
+    __syncthreads();
     for (int e = threadIdx.x; e < NREP * D; e += ATT_THREADS) {
         const int r = e / D, dd = e % D;
         float mm, ls, cx;
-        wave_fold<D, NREP>(sm, sl, sacc, r, dd, mm, ls, cx);
+        wave_fold<D, NREP, ATT_WAVES>(sm, sl, sacc, r, dd, mm, ls, cx);
         a.out[(((size_t)bb * a.s + i) * a.hq + hk * NREP + r) * D + dd] = cx * (1.0f / (ls + 1e-9f));
     }
 }

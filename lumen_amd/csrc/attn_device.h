@@ -1,0 +1,200 @@
+// Device-side building blocks of GQA attention over the static KV cache,
+// shared by the stand-alone attention kernels and the persistent decode
+// kernel.  WAVES = wavefronts per workgroup (64 lanes each).
+//
+// Lane mapping: a K/V row of D floats is covered by LPR = D/4 lanes holding
+// 16 bytes each, so one 64-lane load instruction fetches 64/LPR rows.  Every
+// lane group keeps an online-softmax state (m, l, ctx) for all NREP query
+// heads of the KV group: each K/V byte is read once and used NREP times from
+// registers.
+#pragma once
+
+#ifndef LUMEN_CPU_EMU
+#include <hip/hip_runtime.h>
+#endif
+#include <cmath>
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+template <int NREP>
+struct AttnState {
+    float m[NREP], l[NREP];
+    v4f acc[NREP];
+};
+
+template <int NREP>
+__device__ __forceinline__ void state_init(AttnState<NREP> &st) {
+#pragma unroll
+    for (int r = 0; r < NREP; ++r) {
+        st.m[r] = -INFINITY;
+        st.l[r] = 0.f;
+        st.acc[r] = (v4f){0.f, 0.f, 0.f, 0.f};
+    }
+}
+
+// One K/V row piece per lane: score for each of the NREP heads, online-softmax
+// update (the reference's branchy form, self_attention.rs:252-285, computes the
+// same quantities).  Every lane of the wavefront must call it (it shuffles).
+template <int D, int NREP>
+__device__ __forceinline__ void attn_step(AttnState<NREP> &st, const v4f (&q)[NREP], const v4f kv, const v4f vv,
+                                          bool valid, float scale) {
+    constexpr int LPR = D / 4;
+#pragma unroll
+    for (int r = 0; r < NREP; ++r) {
+        float s = q[r].x * kv.x;
+        s = fmaf(q[r].y, kv.y, s);
+        s = fmaf(q[r].z, kv.z, s);
+        s = fmaf(q[r].w, kv.w, s);
+#pragma unroll
+        for (int off = LPR / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+        s = valid ? s * scale : -INFINITY;
+        const float m_new = fmaxf(st.m[r], s);
+        if (m_new > -INFINITY) {
+            const float alpha = expf(st.m[r] - m_new);  // exp(-inf) = 0 on the first row
+            const float p = expf(s - m_new);
+            st.l[r] = fmaf(st.l[r], alpha, p);
+            st.acc[r].x = fmaf(st.acc[r].x, alpha, p * vv.x);
+            st.acc[r].y = fmaf(st.acc[r].y, alpha, p * vv.y);
+            st.acc[r].z = fmaf(st.acc[r].z, alpha, p * vv.z);
+            st.acc[r].w = fmaf(st.acc[r].w, alpha, p * vv.w);
+            st.m[r] = m_new;
+        }
+    }
+}
+
+template <int D, int WAVES>
+struct AttnGeom {
+    static constexpr int LPR = D / 4;            // lanes per row
+    static constexpr int RPW = 64 / LPR;         // rows per wavefront load
+    static constexpr int RPI = WAVES * RPW;      // rows per workgroup iteration
+    static constexpr int U = 4;                  // iterations whose loads are in flight together
+    static constexpr int ROWS_PER_TRIP = RPI * U;
+};
+
+// Rows [p0, p1) of one KV head (Kb/Vb point at row 0) spread over the
+// workgroup's WAVES x (64/LPR) lane groups.
+template <int D, int NREP, int WAVES>
+__device__ __forceinline__ void attn_rows(AttnState<NREP> &st, const v4f (&q)[NREP], const float *__restrict__ Kb,
+                                          const float *__restrict__ Vb, int p0, int p1, float scale) {
+    typedef AttnGeom<D, WAVES> G;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int slot = lane / G::LPR, c = lane % G::LPR;
+    const int off = wave * G::RPW + slot;
+    for (int base = p0; base < p1; base += G::ROWS_PER_TRIP) {  // trip count is uniform over the workgroup
+        v4f kv[G::U], vv[G::U];
+#pragma unroll
+        for (int u = 0; u < G::U; ++u) {
+            const int j = base + u * G::RPI + off;
+            kv[u] = (v4f){0.f, 0.f, 0.f, 0.f};
+            vv[u] = (v4f){0.f, 0.f, 0.f, 0.f};
+            if (j < p1) {
+                kv[u] = *(const v4f *)(Kb + (size_t)j * D + c * 4);
+                vv[u] = *(const v4f *)(Vb + (size_t)j * D + c * 4);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < G::U; ++u) {
+            // uniform test: every lane of the wavefront takes the step (it shuffles), rows past p1 are masked
+            if (base + u * G::RPI < p1) attn_step<D, NREP>(st, q, kv[u], vv[u], base + u * G::RPI + off < p1, scale);
+        }
+    }
+}
+
+// Merge the lane-group states of each wavefront and publish one state per
+// wavefront in LDS (sm, sl [WAVES][NREP]; sacc [WAVES][NREP][D]).  The caller
+// puts a workgroup barrier between this and wave_fold().
+template <int D, int NREP>
+__device__ __forceinline__ void wave_merge_publish(AttnState<NREP> &st, float *sm, float *sl, float *sacc) {
+    constexpr int LPR = D / 4;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int slot = lane / LPR, c = lane % LPR;
+#pragma unroll
+    for (int r = 0; r < NREP; ++r) {
+#pragma unroll
+        for (int off = LPR; off < 64; off <<= 1) {
+            const float mo = __shfl_xor(st.m[r], off, 64);
+            const float lo = __shfl_xor(st.l[r], off, 64);
+            v4f ao;
+            ao.x = __shfl_xor(st.acc[r].x, off, 64);
+            ao.y = __shfl_xor(st.acc[r].y, off, 64);
+            ao.z = __shfl_xor(st.acc[r].z, off, 64);
+            ao.w = __shfl_xor(st.acc[r].w, off, 64);
+            const float mn = fmaxf(st.m[r], mo);
+            const float a = (mn > -INFINITY) ? expf(st.m[r] - mn) : 0.f;
+            const float b = (mn > -INFINITY) ? expf(mo - mn) : 0.f;
+            st.l[r] = st.l[r] * a + lo * b;
+            st.acc[r].x = st.acc[r].x * a + ao.x * b;
+            st.acc[r].y = st.acc[r].y * a + ao.y * b;
+            st.acc[r].z = st.acc[r].z * a + ao.z * b;
+            st.acc[r].w = st.acc[r].w * a + ao.w * b;
+            st.m[r] = mn;
+        }
+        if (slot == 0) {
+            if (c == 0) {
+                sm[wave * NREP + r] = st.m[r];
+                sl[wave * NREP + r] = st.l[r];
+            }
+            *(v4f *)(sacc + ((size_t)(wave * NREP + r)) * D + c * 4) = st.acc[r];
+        }
+    }
+}
+
+// (max, sum, ctx) of head r, dim dd over the wavefront states in LDS
+template <int D, int NREP, int WAVES>
+__device__ __forceinline__ void wave_fold(const float *sm, const float *sl, const float *sacc, int r, int dd,
+                                          float &mm, float &ls, float &cx) {
+    mm = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) mm = fmaxf(mm, sm[w * NREP + r]);
+    ls = 0.f;
+    cx = 0.f;
+    if (mm > -INFINITY) {
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) {
+            const float ex = expf(sm[w * NREP + r] - mm);
+            ls = fmaf(sl[w * NREP + r], ex, ls);
+            cx = fmaf(sacc[((size_t)(w * NREP + r)) * D + dd], ex, cx);
+        }
+    }
+}
+
+// Optional per-head RMSNorm (gain g) then half-split RoPE of nh contiguous
+// heads held raw in LDS `raw` ([nh][D]) into `rot`.  cs/sn: table rows at the
+// token's position.  q: (x1*c - x2*s, x1*s + x2*c), self_attention.rs:220-227;
+// k: same values, encoding.rs:196-203.
+template <int D>
+__device__ __forceinline__ void norm_rope_heads(const float *raw, float *rot, int nh, const float *__restrict__ cs,
+                                                const float *__restrict__ sn, const float *__restrict__ g,
+                                                float eps, int nthreads) {
+    constexpr int HALF = D / 2;
+    for (int p = threadIdx.x; p < nh * HALF; p += nthreads) {
+        const int r = p / HALF, j = p % HALF;
+        float x1 = raw[r * D + j], x2 = raw[r * D + j + HALF];
+        if (g) {
+            float ss = 0.f;
+            for (int i = 0; i < D; ++i) ss = fmaf(raw[r * D + i], raw[r * D + i], ss);
+            const float inv = 1.0f / sqrtf(ss / (float)D + eps);
+            x1 = x1 * inv * g[j];
+            x2 = x2 * inv * g[j + HALF];
+        }
+        const float c = cs[j], s = sn[j];
+        {
+#pragma clang fp contract(off)  // separate multiplies and add, like the reference's compiled code
+            rot[r * D + j] = x1 * c - x2 * s;
+            rot[r * D + j + HALF] = x1 * s + x2 * c;
+        }
+    }
+}
+
+// How the cached rows [0, pos) are cut into slices for one decode step: only
+// as many slices as give each at least one full trip of rows take part, the
+// others return at once.  The new token (row `pos`) belongs to the last
+// active slice.
+template <int D, int WAVES>
+__device__ __forceinline__ void decode_slices(int pos, int nsplit, int &nact, int &chunk) {
+    typedef AttnGeom<D, WAVES> G;
+    nact = (pos + G::ROWS_PER_TRIP - 1) / G::ROWS_PER_TRIP;
+    nact = nact < 1 ? 1 : (nact > nsplit ? nsplit : nact);
+    chunk = (pos + nact - 1) / nact;
+    chunk = (chunk + G::RPI - 1) / G::RPI * G::RPI;
+}

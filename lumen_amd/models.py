@@ -127,6 +127,19 @@ class LlamaModel:
                                             logits.ctypes.data if want_logits else None))
         return (ids, logits) if want_logits else ids
 
+    DECODE_MODES = {"eager": _lib.DECODE_EAGER, "graph": _lib.DECODE_GRAPH, "persistent": _lib.DECODE_PERSISTENT}
+
+    def set_decode_mode(self, mode):
+        """'persistent' (one cooperative kernel for all layers and steps), 'graph' (HIP graph replay
+        per token) or 'eager' (kernel by kernel)."""
+        check(lib.lumen_llama_set_decode_mode(self.handle, self.DECODE_MODES[mode]))
+
+    @property
+    def decode_mode(self):
+        v = C.c_int()
+        check(lib.lumen_llama_get_decode_mode(self.handle, C.byref(v)))
+        return {n: k for k, n in self.DECODE_MODES.items()}[v.value]
+
     KERNEL_CLASSES = ("embedding", "norm_qkv_gemv", "attn_decode", "oproj_gemv", "norm_gateup_gemv", "down_gemv",
                       "norm_lmhead_gemv", "argmax")
 

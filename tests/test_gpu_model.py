@@ -168,6 +168,59 @@ def test_status_codes_for_overflow_oob_and_bad_params():
     assert e.value.status == _lib.ERR_CACHE_COUNT
 
 
+GQA64 = dict(vocab_size=1500, hidden_size=512, intermediate_size=1408, num_hidden_layers=3, num_attention_heads=8,
+             num_key_value_heads=1, rms_norm_eps=1e-5, max_seq_len=512, rope_theta=10000.0)  # head_dim 64, n_rep 8
+MHA128 = dict(vocab_size=700, hidden_size=256, intermediate_size=704, num_hidden_layers=2, num_attention_heads=2,
+              num_key_value_heads=2, rms_norm_eps=1e-5, max_seq_len=300, rope_theta=10000.0)  # head_dim 128, n_rep 1
+
+
+# The persistent decode kernel is switched off in the library: its first run on the GPU ended in a
+# memory fault whose cause is not established, so it must not run on a GPU.  Its logic is covered on
+# the CPU by tests/test_cpu_emu.py (ASan build of the same device code against the oracle).
+MODES = ("graph", "eager")
+
+
+def test_persistent_mode_is_refused_while_switched_off():
+    gpu, _, _ = build(GQA64, seed=20)
+    assert gpu.decode_mode == "graph"
+    with pytest.raises(_lib.LumenError) as e:
+        gpu.set_decode_mode("persistent")
+    assert e.value.status == _lib.ERR_UNSUPPORTED
+
+
+@pytest.mark.parametrize("cfg,bf16,n_prompt", [(GQA64, False, 140), (MHA128, False, 37), (TINY_QWEN, False, 9),
+                                               (GQA64, True, 33)], ids=["gqa64", "mha128", "qwen3", "gqa64-bf16"])
+def test_decode_modes_agree_with_each_other_and_the_oracle(cfg, bf16, n_prompt):
+    """HIP-graph replay and eager launches are two ways to issue the same step."""
+    tol = 2e-2 if bf16 else 1e-4
+    gpu, ora, _ = build(cfg, seed=21, bf16=bf16)
+    ids = synth.make_tokens(n_prompt + 6, cfg["vocab_size"], seed=21)
+    rc, ref_prompt = ora.forward(ids[:n_prompt])
+    refs = [ora.forward(ids[t:t + 1])[1][0] for t in range(n_prompt, n_prompt + 6)]
+    first = lo.argmax(refs[-1])
+    tok, greedy_ref = first, []
+    for _ in range(5):
+        r = ora.forward(np.array([tok]))[1][0]
+        greedy_ref.append(r)
+        tok = lo.argmax(r)
+    results = {}
+    for mode in MODES:
+        gpu.reset_kv_caches()
+        gpu.set_decode_mode(mode)
+        gpu.forward(ids[:n_prompt], all_rows=False)
+        rows = [gpu.forward(ids[t:t + 1], all_rows=False) for t in range(n_prompt, n_prompt + 6)]
+        picks, logits = gpu.decode_greedy(first, 5, want_logits=True)
+        assert gpu.kv_len == n_prompt + 11
+        for g, r in zip(rows, refs):
+            assert max_rel(g, r) <= tol, mode
+        for t in range(5):
+            assert max_rel(logits[t], greedy_ref[t]) <= tol, (mode, t)
+            check_argmax(logits[t], greedy_ref[t], tol)
+        results[mode] = (np.stack(rows), picks, logits)
+    assert np.array_equal(results["graph"][0], results["eager"][0])  # same kernels, same order of operations
+    assert np.array_equal(results["graph"][1], results["eager"][1])
+
+
 @pytest.mark.slow
 def test_tinyllama_1b_shape_prefill_128_decode_teacher_forced():
     """The headline configuration at full size: 22 layers, hidden 2048, 32/4 heads, vocab 32000,
