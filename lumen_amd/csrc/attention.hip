@@ -18,45 +18,61 @@
 #define ATT_WAVES 4
 #define ATT_THREADS (ATT_WAVES * 64)
 
+// WAVES wavefronts per workgroup: 8, i.e. one trip covers 128 rows of D = 64; the step is ALU-bound
+// (scores, exponentials and weighted sums for n_rep heads per row), so slices are kept short and
+// spread over many compute units rather than packed into few large workgroups.
 template <int D, int NREP>
-__global__ __launch_bounds__(ATT_THREADS) void attn_decode_kernel(AttnDecodeArgs a) {
-    typedef AttnGeom<D, ATT_WAVES> G;
+struct DecodeWaves {
+    static constexpr int value = 8;
+};
+
+template <int D, int NREP, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void attn_decode_kernel(AttnDecodeArgs a) {
+    typedef AttnGeom<D, WAVES> G;
+    constexpr int THREADS = WAVES * 64;
     __shared__ __align__(16) float q_raw[NREP * D];
     __shared__ __align__(16) float q_rot[NREP * D];
     __shared__ __align__(16) float k_raw[D];
     __shared__ __align__(16) float k_new[D];
     __shared__ __align__(16) float v_new[D];
-    __shared__ __align__(16) float sacc[ATT_WAVES * NREP * D];
-    __shared__ float sm[ATT_WAVES * NREP], sl[ATT_WAVES * NREP];
+    __shared__ __align__(16) float sacc[WAVES * NREP * D];
+    __shared__ float sm[WAVES * NREP], sl[WAVES * NREP];
     __shared__ int s_last;
 
     const int split = blockIdx.x, hk = blockIdx.y, bb = blockIdx.z;
     const int pos = a.pos_dev ? *a.pos_dev : a.pos_host;  // == past_len
     int nact, chunk;
-    decode_slices<D, ATT_WAVES>(pos, gridDim.x, nact, chunk);
+    decode_slices<D, WAVES>(pos, gridDim.x, nact, chunk);
     if (split >= nact) return;
     const bool has_new = (split == nact - 1);
     const float *cs = a.cos_t + (size_t)pos * D, *sn = a.sin_t + (size_t)pos * D;
     const size_t head_base = ((size_t)bb * a.hkv + hk) * a.max_seq * D;
+    const float *Kb = a.k_cache + head_base, *Vb = a.v_cache + head_base;
+
+    // this slice's share of the cached rows [0, pos); its first trip of K/V rows starts streaming
+    // before anything else: it does not depend on q
+    const int p0 = min(pos, split * chunk), p1 = min(pos, p0 + chunk);
+    v4f kv[G::U], vv[G::U];
+    attn_load_trip<D, WAVES>(Kb, Vb, p0, p1, kv, vv);
 
     // stage raw q heads of this KV group (contiguous: hq = hk*NREP + r) and the new k / v
     const float *q_src = a.q + ((size_t)bb * a.hq + (size_t)hk * NREP) * D;
-    for (int i = threadIdx.x; i < NREP * D; i += ATT_THREADS) q_raw[i] = q_src[i];
+    for (int i = threadIdx.x; i < NREP * D; i += THREADS) q_raw[i] = q_src[i];
     if (has_new) {
         const float *k_src = a.k_new + ((size_t)bb * a.hkv + hk) * D;
         const float *v_src = a.v_new + ((size_t)bb * a.hkv + hk) * D;
-        for (int i = threadIdx.x; i < D; i += ATT_THREADS) {
+        for (int i = threadIdx.x; i < D; i += THREADS) {
             k_raw[i] = k_src[i];
             v_new[i] = v_src[i];
         }
     }
     __syncthreads();
-    norm_rope_heads<D>(q_raw, q_rot, NREP, cs, sn, a.q_norm_w, a.norm_eps, ATT_THREADS);
-    if (has_new) norm_rope_heads<D>(k_raw, k_new, 1, cs, sn, a.k_norm_w, a.norm_eps, ATT_THREADS);
+    norm_rope_heads<D>(q_raw, q_rot, NREP, cs, sn, a.q_norm_w, a.norm_eps, THREADS);
+    if (has_new) norm_rope_heads<D>(k_raw, k_new, 1, cs, sn, a.k_norm_w, a.norm_eps, THREADS);
     __syncthreads();
     if (has_new) {
         // self_attention.rs:161-176: rotated k and raw v go to cache row `pos`
-        for (int i = threadIdx.x; i < D; i += ATT_THREADS) {
+        for (int i = threadIdx.x; i < D; i += THREADS) {
             a.k_cache[head_base + (size_t)pos * D + i] = k_new[i];
             a.v_cache[head_base + (size_t)pos * D + i] = v_new[i];
         }
@@ -65,71 +81,57 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_decode_kernel(AttnDecodeArgs
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int slot = lane / G::LPR, c = lane % G::LPR;
     v4f q[NREP];
-#pragma unroll
-    for (int r = 0; r < NREP; ++r) q[r] = *(const v4f *)(q_rot + r * D + c * 4);
+    load_q_scaled<D, NREP>(q, q_rot, c, a.scale);
 
-    // this slice's share of the cached rows [0, pos)
-    const int p0 = min(pos, split * chunk), p1 = min(pos, p0 + chunk);
     AttnState<NREP> st;
     state_init<NREP>(st);
-    attn_rows<D, NREP, ATT_WAVES>(st, q, a.k_cache + head_base, a.v_cache + head_base, p0, p1, a.scale);
+    if (p0 < p1) attn_compute_trip<D, NREP, WAVES>(st, q, kv, vv, p0, p1);
+    attn_rows<D, NREP, WAVES>(st, q, Kb, Vb, p0 + G::ROWS_PER_TRIP, p1);
     if (has_new && wave == 0) {
         // the new token's row comes from LDS (lane group 0 of wavefront 0)
-        const v4f kv = *(const v4f *)(k_new + c * 4);
-        const v4f vv = *(const v4f *)(v_new + c * 4);
-        attn_step<D, NREP>(st, q, kv, vv, slot == 0, a.scale);
+        const v4f kn = *(const v4f *)(k_new + c * 4);
+        const v4f vn = *(const v4f *)(v_new + c * 4);
+        attn_step<D, NREP>(st, q, kn, vn, slot == 0);
     }
 
     wave_merge_publish<D, NREP>(st, sm, sl, sacc);
     __syncthreads();
     const int t = threadIdx.x;
-    for (int e = t; e < NREP * D; e += ATT_THREADS) {
+    for (int e = t; e < NREP * D; e += THREADS) {
         const int r = e / D, dd = e % D;
         float mm, ls, cx;
-        wave_fold<D, NREP, ATT_WAVES>(sm, sl, sacc, r, dd, mm, ls, cx);
+        wave_fold<D, NREP, WAVES>(sm, sl, sacc, r, dd, mm, ls, cx);
         const int hq = hk * NREP + r;
         if (nact == 1) {
             // out = ctx / (l + 1e-9), self_attention.rs:287-290
             a.out[((size_t)bb * a.hq + hq) * D + dd] = cx * (1.0f / (ls + 1e-9f));
         } else {
             float *pp = a.part + (((size_t)bb * a.hq + hq) * gridDim.x + split) * (D + 2);
-            pp[dd] = cx;
+            part_store(pp + dd, cx);
             if (dd == 0) {
-                pp[D] = mm;
-                pp[D + 1] = ls;
+                part_store(pp + D, mm);
+                part_store(pp + D + 1, ls);
             }
         }
     }
     if (nact == 1) return;
 
-    // last workgroup of this (batch, KV head) to arrive folds the slices in index order
-    __threadfence();
+    // last workgroup of this (batch, KV head) to arrive folds the slices in index order.  The barrier
+    // makes every wavefront wait for its own stores before thread 0 signals.
     __syncthreads();
     if (t == 0) {
-        const int old = atomicAdd(&a.counters[bb * a.hkv + hk], 1);
+        const int old = __hip_atomic_fetch_add(&a.counters[bb * a.hkv + hk], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         s_last = (old == nact - 1);
+        if (s_last) __hip_atomic_store(&a.counters[bb * a.hkv + hk], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
     if (!s_last) return;
-    __threadfence();  // acquire: the other slices' partial results are visible from here on
-    for (int e = t; e < NREP * D; e += ATT_THREADS) {
+    for (int e = t; e < NREP * D; e += THREADS) {
         const int r = e / D, dd = e % D;
         const int hq = hk * NREP + r;
         const float *pp = a.part + (((size_t)bb * a.hq + hq) * gridDim.x) * (D + 2);
-        float mm = -INFINITY;
-        for (int s = 0; s < nact; ++s) mm = fmaxf(mm, pp[(size_t)s * (D + 2) + D]);
-        float ls = 0.f, cx = 0.f;
-        for (int s = 0; s < nact; ++s) {
-            const float ms = pp[(size_t)s * (D + 2) + D];
-            if (ms > -INFINITY) {
-                const float ex = expf(ms - mm);
-                ls = fmaf(pp[(size_t)s * (D + 2) + D + 1], ex, ls);
-                cx = fmaf(pp[(size_t)s * (D + 2) + dd], ex, cx);
-            }
-        }
-        a.out[((size_t)bb * a.hq + hq) * D + dd] = cx * (1.0f / (ls + 1e-9f));
+        a.out[((size_t)bb * a.hq + hq) * D + dd] = fold_slices<D>(pp, nact, dd);
     }
-    if (t == 0) a.counters[bb * a.hkv + hk] = 0;  // ready for the next launch
 }
 
 int attn_decode_nsplit(int max_seq) {
@@ -143,15 +145,19 @@ size_t attn_decode_part_floats(int b, int hq, int d, int nsplit) { return (size_
 
 template <int D>
 static int launch_decode_d(lumen_ctx *ctx, const AttnDecodeArgs &a) {
-    dim3 grid(a.nsplit, a.hkv, a.b), block(ATT_THREADS);
+    dim3 grid(a.nsplit, a.hkv, a.b);
     const int nrep = a.hq / a.hkv;
+#define LAUNCH_DECODE(NR)                                                                                     \
+    hipLaunchKernelGGL((attn_decode_kernel<D, NR, DecodeWaves<D, NR>::value>), grid,                          \
+                       dim3(DecodeWaves<D, NR>::value * 64), 0, ctx->stream, a)
     switch (nrep) {
-        case 1: hipLaunchKernelGGL((attn_decode_kernel<D, 1>), grid, block, 0, ctx->stream, a); break;
-        case 2: hipLaunchKernelGGL((attn_decode_kernel<D, 2>), grid, block, 0, ctx->stream, a); break;
-        case 4: hipLaunchKernelGGL((attn_decode_kernel<D, 4>), grid, block, 0, ctx->stream, a); break;
-        case 8: hipLaunchKernelGGL((attn_decode_kernel<D, 8>), grid, block, 0, ctx->stream, a); break;
+        case 1: LAUNCH_DECODE(1); break;
+        case 2: LAUNCH_DECODE(2); break;
+        case 4: LAUNCH_DECODE(4); break;
+        case 8: LAUNCH_DECODE(8); break;
         default: LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "decode attention: n_rep=%d (supported 1, 2, 4, 8)", nrep);
     }
+#undef LAUNCH_DECODE
     LUMEN_CHECK_LAUNCH();
     return LUMEN_OK;
 }
@@ -223,11 +229,10 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_prefill_kernel(AttnPrefillAr
     const int c = (threadIdx.x & 63) % G::LPR;
     const float *qr = a.q_rot + (((size_t)bb * a.s + i) * a.hq + (size_t)hk * NREP) * D;
     v4f q[NREP];
-#pragma unroll
-    for (int r = 0; r < NREP; ++r) q[r] = *(const v4f *)(qr + r * D + c * 4);
+    load_q_scaled<D, NREP>(q, qr, c, a.scale);
     AttnState<NREP> st;
     state_init<NREP>(st);
-    attn_rows<D, NREP, ATT_WAVES>(st, q, a.k_cache + head_base, a.v_cache + head_base, 0, p1, a.scale);
+    attn_rows<D, NREP, ATT_WAVES>(st, q, a.k_cache + head_base, a.v_cache + head_base, 0, p1);
     wave_merge_publish<D, NREP>(st, sm, sl, sacc);
     __syncthreads();
     for (int e = threadIdx.x; e < NREP * D; e += ATT_THREADS) {

@@ -32,12 +32,36 @@ __device__ __forceinline__ void state_init(AttnState<NREP> &st) {
     }
 }
 
-// One K/V row piece per lane: score for each of the NREP heads, online-softmax
-// update (the reference's branchy form, self_attention.rs:252-285, computes the
-// same quantities).  Every lane of the wavefront must call it (it shuffles).
+// exp2 on the hardware transcendental unit (v_exp_f32, ~1 ulp; exp2(-inf) = 0).  Scores are kept in
+// log2 units (q is pre-multiplied by scale * log2(e)), so softmax needs no other exponential.
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+#define LUMEN_LOG2E 1.4426950408889634f
+
+// Sum over the LPR lanes that share a K/V row; every lane of the group gets the total.  Groups of
+// 16 lanes are one DPP row: four rotate-and-add steps on the VALU, no LDS crossbar traffic.
+template <int LPR>
+__device__ __forceinline__ float group_sum(float v) {
+    if (LPR >= 16) {
+        v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false));  // row_ror:8
+        v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xf, 0xf, false));  // row_ror:4
+        v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xf, 0xf, false));  // row_ror:2
+        v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xf, 0xf, false));  // row_ror:1
+#pragma unroll
+        for (int off = 16; off < LPR; off <<= 1) v += __shfl_xor(v, off, 64);
+    } else {
+#pragma unroll
+        for (int off = LPR / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    }
+    return v;
+}
+
+// One K/V row piece per lane: score for each of the NREP heads, online-softmax update (the
+// reference's branchy form, self_attention.rs:252-285, computes the same quantities).  q holds the
+// rotated query times scale * log2(e).  Every lane of the wavefront must call it (it shuffles).
 template <int D, int NREP>
 __device__ __forceinline__ void attn_step(AttnState<NREP> &st, const v4f (&q)[NREP], const v4f kv, const v4f vv,
-                                          bool valid, float scale) {
+                                          bool valid) {
     constexpr int LPR = D / 4;
 #pragma unroll
     for (int r = 0; r < NREP; ++r) {
@@ -45,13 +69,12 @@ __device__ __forceinline__ void attn_step(AttnState<NREP> &st, const v4f (&q)[NR
         s = fmaf(q[r].y, kv.y, s);
         s = fmaf(q[r].z, kv.z, s);
         s = fmaf(q[r].w, kv.w, s);
-#pragma unroll
-        for (int off = LPR / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
-        s = valid ? s * scale : -INFINITY;
+        s = group_sum<LPR>(s);
+        s = valid ? s : -INFINITY;
         const float m_new = fmaxf(st.m[r], s);
         if (m_new > -INFINITY) {
-            const float alpha = expf(st.m[r] - m_new);  // exp(-inf) = 0 on the first row
-            const float p = expf(s - m_new);
+            const float alpha = fast_exp2(st.m[r] - m_new);  // exp2(-inf) = 0 on the first row
+            const float p = fast_exp2(s - m_new);
             st.l[r] = fmaf(st.l[r], alpha, p);
             st.acc[r].x = fmaf(st.acc[r].x, alpha, p * vv.x);
             st.acc[r].y = fmaf(st.acc[r].y, alpha, p * vv.y);
@@ -67,36 +90,53 @@ struct AttnGeom {
     static constexpr int LPR = D / 4;            // lanes per row
     static constexpr int RPW = 64 / LPR;         // rows per wavefront load
     static constexpr int RPI = WAVES * RPW;      // rows per workgroup iteration
-    static constexpr int U = 4;                  // iterations whose loads are in flight together
+    static constexpr int U = 2;                  // iterations whose loads are in flight together
     static constexpr int ROWS_PER_TRIP = RPI * U;
 };
 
 // Rows [p0, p1) of one KV head (Kb/Vb point at row 0) spread over the
 // workgroup's WAVES x (64/LPR) lane groups.
-template <int D, int NREP, int WAVES>
-__device__ __forceinline__ void attn_rows(AttnState<NREP> &st, const v4f (&q)[NREP], const float *__restrict__ Kb,
-                                          const float *__restrict__ Vb, int p0, int p1, float scale) {
+// One trip = ROWS_PER_TRIP rows starting at `base`: issue all of this lane's K/V loads ...
+template <int D, int WAVES>
+__device__ __forceinline__ void attn_load_trip(const float *__restrict__ Kb, const float *__restrict__ Vb, int base,
+                                               int p1, v4f (&kv)[AttnGeom<D, WAVES>::U],
+                                               v4f (&vv)[AttnGeom<D, WAVES>::U]) {
     typedef AttnGeom<D, WAVES> G;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int slot = lane / G::LPR, c = lane % G::LPR;
-    const int off = wave * G::RPW + slot;
+    const int off = wave * G::RPW + lane / G::LPR, c = lane % G::LPR;
+#pragma unroll
+    for (int u = 0; u < G::U; ++u) {
+        // unconditional loads (straight-line code keeps them all in flight): a row past the slice is
+        // clamped to a row inside the cache and masked out in attn_step (weight exp(-inf) = 0)
+        const int j = max(min(base + u * G::RPI + off, p1 - 1), 0);
+        kv[u] = *(const v4f *)(Kb + (size_t)j * D + c * 4);
+        vv[u] = *(const v4f *)(Vb + (size_t)j * D + c * 4);
+    }
+}
+
+// ... and fold them into the running state.
+template <int D, int NREP, int WAVES>
+__device__ __forceinline__ void attn_compute_trip(AttnState<NREP> &st, const v4f (&q)[NREP],
+                                                  const v4f (&kv)[AttnGeom<D, WAVES>::U],
+                                                  const v4f (&vv)[AttnGeom<D, WAVES>::U], int base, int p1) {
+    typedef AttnGeom<D, WAVES> G;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int off = wave * G::RPW + lane / G::LPR;
+#pragma unroll
+    for (int u = 0; u < G::U; ++u) {
+        // uniform test: every lane of the wavefront takes the step (it shuffles), rows past p1 are masked
+        if (base + u * G::RPI < p1) attn_step<D, NREP>(st, q, kv[u], vv[u], base + u * G::RPI + off < p1);
+    }
+}
+
+template <int D, int NREP, int WAVES>
+__device__ __forceinline__ void attn_rows(AttnState<NREP> &st, const v4f (&q)[NREP], const float *__restrict__ Kb,
+                                          const float *__restrict__ Vb, int p0, int p1) {
+    typedef AttnGeom<D, WAVES> G;
     for (int base = p0; base < p1; base += G::ROWS_PER_TRIP) {  // trip count is uniform over the workgroup
         v4f kv[G::U], vv[G::U];
-#pragma unroll
-        for (int u = 0; u < G::U; ++u) {
-            const int j = base + u * G::RPI + off;
-            kv[u] = (v4f){0.f, 0.f, 0.f, 0.f};
-            vv[u] = (v4f){0.f, 0.f, 0.f, 0.f};
-            if (j < p1) {
-                kv[u] = *(const v4f *)(Kb + (size_t)j * D + c * 4);
-                vv[u] = *(const v4f *)(Vb + (size_t)j * D + c * 4);
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < G::U; ++u) {
-            // uniform test: every lane of the wavefront takes the step (it shuffles), rows past p1 are masked
-            if (base + u * G::RPI < p1) attn_step<D, NREP>(st, q, kv[u], vv[u], base + u * G::RPI + off < p1, scale);
-        }
+        attn_load_trip<D, WAVES>(Kb, Vb, base, p1, kv, vv);
+        attn_compute_trip<D, NREP, WAVES>(st, q, kv, vv, base, p1);
     }
 }
 
@@ -120,8 +160,8 @@ __device__ __forceinline__ void wave_merge_publish(AttnState<NREP> &st, float *s
             ao.z = __shfl_xor(st.acc[r].z, off, 64);
             ao.w = __shfl_xor(st.acc[r].w, off, 64);
             const float mn = fmaxf(st.m[r], mo);
-            const float a = (mn > -INFINITY) ? expf(st.m[r] - mn) : 0.f;
-            const float b = (mn > -INFINITY) ? expf(mo - mn) : 0.f;
+            const float a = (mn > -INFINITY) ? fast_exp2(st.m[r] - mn) : 0.f;
+            const float b = (mn > -INFINITY) ? fast_exp2(mo - mn) : 0.f;
             st.l[r] = st.l[r] * a + lo * b;
             st.acc[r].x = st.acc[r].x * a + ao.x * b;
             st.acc[r].y = st.acc[r].y * a + ao.y * b;
@@ -151,10 +191,21 @@ __device__ __forceinline__ void wave_fold(const float *sm, const float *sl, cons
     if (mm > -INFINITY) {
 #pragma unroll
         for (int w = 0; w < WAVES; ++w) {
-            const float ex = expf(sm[w * NREP + r] - mm);
+            const float ex = fast_exp2(sm[w * NREP + r] - mm);
             ls = fmaf(sl[w * NREP + r], ex, ls);
             cx = fmaf(sacc[((size_t)(w * NREP + r)) * D + dd], ex, cx);
         }
+    }
+}
+
+// This lane's 16-byte piece of each rotated query head, times scale * log2(e)
+template <int D, int NREP>
+__device__ __forceinline__ void load_q_scaled(v4f (&q)[NREP], const float *q_rot, int c, float scale) {
+    const float f = scale * LUMEN_LOG2E;
+#pragma unroll
+    for (int r = 0; r < NREP; ++r) {
+        q[r] = *(const v4f *)(q_rot + r * D + c * 4);
+        q[r].x *= f; q[r].y *= f; q[r].z *= f; q[r].w *= f;
     }
 }
 
@@ -184,6 +235,32 @@ __device__ __forceinline__ void norm_rope_heads(const float *raw, float *rot, in
             rot[r * D + j + HALF] = x1 * s + x2 * c;
         }
     }
+}
+
+// Partial results of a slice travel between workgroups through memory with agent-scope accesses
+// (they bypass the per-XCD L2 and the CU's L1, so neither a cache write-back nor an invalidate is
+// needed around the hand-over; the writer only has to wait for its stores before it signals).
+__device__ __forceinline__ void part_store(float *p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float part_load(const float *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Folds the nact partial states of head-dim element (hq, dd) in slice order: out = ctx / (l + 1e-9),
+// self_attention.rs:287-290.  pp points at the head's first partial; entries are (D + 2) floats apart.
+template <int D>
+__device__ __forceinline__ float fold_slices(const float *pp, int nact, int dd) {
+    float mm = -INFINITY;
+    for (int s = 0; s < nact; ++s) mm = fmaxf(mm, part_load(pp + (size_t)s * (D + 2) + D));
+    float ls = 0.f, cx = 0.f;
+    for (int s = 0; s < nact; ++s) {
+        const float ms = part_load(pp + (size_t)s * (D + 2) + D);
+        const float ex = (ms > -INFINITY) ? fast_exp2(ms - mm) : 0.f;
+        ls = fmaf(part_load(pp + (size_t)s * (D + 2) + D + 1), ex, ls);
+        cx = fmaf(part_load(pp + (size_t)s * (D + 2) + dd), ex, cx);
+    }
+    return cx * (1.0f / (ls + 1e-9f));
 }
 
 // How the cached rows [0, pos) are cut into slices for one decode step: only

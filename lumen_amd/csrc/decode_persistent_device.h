@@ -310,16 +310,15 @@ __device__ __forceinline__ void attn_stage(const PkArgs &a, const PkLayer &L, in
             }
         }
         v4f q[NREP];
-#pragma unroll
-        for (int r = 0; r < NREP; ++r) q[r] = *(const v4f *)(q_rot + r * D + c * 4);
+        load_q_scaled<D, NREP>(q, q_rot, c, a.scale);
         const int p0 = min(pos, split * chunk), p1 = min(pos, p0 + chunk);
         AttnState<NREP> st;
         state_init<NREP>(st);
-        attn_rows<D, NREP, PK_WAVES>(st, q, L.k_cache + head_base, L.v_cache + head_base, p0, p1, a.scale);
+        attn_rows<D, NREP, PK_WAVES>(st, q, L.k_cache + head_base, L.v_cache + head_base, p0, p1);
         if (has_new && wave == 0) {
             const v4f kv = *(const v4f *)(k_new + c * 4);
             const v4f vv = *(const v4f *)(v_new + c * 4);
-            attn_step<D, NREP>(st, q, kv, vv, slot == 0, a.scale);
+            attn_step<D, NREP>(st, q, kv, vv, slot == 0);
         }
         wave_merge_publish<D, NREP>(st, sm, sl, sacc);
         __syncthreads();
@@ -332,46 +331,31 @@ __device__ __forceinline__ void attn_stage(const PkArgs &a, const PkLayer &L, in
                 a.attn[(size_t)hq * D + dd] = cx * (1.0f / (ls + 1e-9f));  // self_attention.rs:287-290
             } else {
                 float *pp = a.part + ((size_t)hq * a.nsplit + split) * (D + 2);
-                pp[dd] = cx;
+                part_store(pp + dd, cx);
                 if (dd == 0) {
-                    pp[D] = mm;
-                    pp[D + 1] = ls;
+                    part_store(pp + D, mm);
+                    part_store(pp + D + 1, ls);
                 }
             }
         }
         if (nact > 1) {
             // last workgroup of this KV head to arrive folds the slices in index order
-            __threadfence();
             __syncthreads();
             if (t == 0) {
-                const int old = atomicAdd(&a.head_counters[hk], 1);
+                const int old = __hip_atomic_fetch_add(&a.head_counters[hk], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 *s_last = (old == nact - 1);
+                if (old == nact - 1) __hip_atomic_store(&a.head_counters[hk], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
             __syncthreads();
             if (*s_last) {
-                __threadfence();
                 for (int e = t; e < NREP * D; e += PK_THREADS) {
                     const int r = e / D, dd = e % D;
                     const int hq = hk * NREP + r;
-                    const float *pp = a.part + ((size_t)hq * a.nsplit) * (D + 2);
-                    float mm = -INFINITY;
-                    for (int s = 0; s < nact; ++s) mm = fmaxf(mm, pp[(size_t)s * (D + 2) + D]);
-                    float ls = 0.f, cx = 0.f;
-                    for (int s = 0; s < nact; ++s) {
-                        const float ms = pp[(size_t)s * (D + 2) + D];
-                        if (ms > -INFINITY) {
-                            const float ex = expf(ms - mm);
-                            ls = fmaf(pp[(size_t)s * (D + 2) + D + 1], ex, ls);
-                            cx = fmaf(pp[(size_t)s * (D + 2) + dd], ex, cx);
-                        }
-                    }
-                    a.attn[(size_t)hq * D + dd] = cx * (1.0f / (ls + 1e-9f));
+                    a.attn[(size_t)hq * D + dd] = fold_slices<D>(a.part + ((size_t)hq * a.nsplit) * (D + 2), nact, dd);
                 }
-                if (t == 0) a.head_counters[hk] = 0;
             }
         }
     }
-
 }
 
 // -------------------------------------------------------------------- kernel

@@ -100,11 +100,10 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(GemvArgs a) {
     constexpr int VEC = BF16 ? 8 : 4;          // elements per 16-byte load
     constexpr int SWEEP = 64 * VEC;            // elements one wavefront covers per load
     constexpr int U = 8 / R;                   // loads in flight per lane per row
+    constexpr int PIECE = SWEEP * U;           // elements of a row one piece covers
     constexpr int ESZ = BF16 ? 2 : 4;
     const int K = a.K, N = a.N;
-    const int kpad = (K + SWEEP - 1) / SWEEP * SWEEP;
-
-    stage_x<PRO>(xs, a.x, a.norm_w, a.eps, K, kpad);
+    const int kpad = (K + PIECE - 1) / PIECE * PIECE;  // xs is zero from K to kpad
 
     const int lane = threadIdx.x & 63;
     const int gw = blockIdx.x * GEMV_WAVES + (threadIdx.x >> 6);
@@ -113,35 +112,39 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(GemvArgs a) {
     const char *Wb = (const char *)a.W;
     const size_t row_bytes = (size_t)K * ESZ;
 
-    for (int u = gw; u < nunits; u += nw) {
-        const char *wp[R];
-        float acc[R];
+    // 8 x 16 bytes per lane of unit u from element k0 on.  Every load is issued unconditionally:
+    // positions past the end of the row are clamped to its last 16 bytes (they meet the zero
+    // padding of xs), a row past N to row N-1 (discarded in the epilogue).
+    auto load_piece = [&](int u, int k0, v4u (&raw)[R][U]) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            int row = u * R + r;
-            if (row >= N) row = N - 1;  // odd N with R == 2: result discarded below
-            wp[r] = Wb + (size_t)row * row_bytes + (size_t)lane * 16;
-            acc[r] = 0.f;
-        }
-        for (int k0 = 0; k0 < K; k0 += SWEEP * U) {
-            v4u raw[R][U];
+            const int row = min(u * R + r, N - 1);
+            const char *rp = Wb + (size_t)row * row_bytes;
 #pragma unroll
             for (int uu = 0; uu < U; ++uu) {
-                const int kk = k0 + uu * SWEEP + lane * VEC;
-#pragma unroll
-                for (int r = 0; r < R; ++r) {
-                    raw[r][uu] = (v4u){0u, 0u, 0u, 0u};
-                    if (kk < K)
-                        raw[r][uu] = __builtin_nontemporal_load((const v4u *)(wp[r] + (size_t)(k0 + uu * SWEEP) * ESZ));
-                }
+                const int kk = min(k0 + uu * SWEEP + lane * VEC, K - VEC);
+                raw[r][uu] = __builtin_nontemporal_load((const v4u *)(rp + (size_t)kk * ESZ));
             }
+        }
+    };
+
+    // the first weights of this wavefront start streaming before x is staged: they do not depend on it
+    v4u raw[R][U];
+    load_piece(min(gw, nunits - 1), 0, raw);
+
+    stage_x<PRO>(xs, a.x, a.norm_w, a.eps, K, kpad);
+
+    for (int u = gw; u < nunits; u += nw) {
+        float acc[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[r] = 0.f;
+        for (int k0 = 0; k0 < K; k0 += PIECE) {
+            if (u != gw || k0 != 0) load_piece(u, k0, raw);
 #pragma unroll
             for (int uu = 0; uu < U; ++uu) {
-                const int kk = k0 + uu * SWEEP + lane * VEC;
-                if (kk < kpad) {
+                const float *xp = xs + k0 + uu * SWEEP + lane * VEC;
 #pragma unroll
-                    for (int r = 0; r < R; ++r) acc[r] += dot16<BF16>(raw[r][uu], xs + kk);
-                }
+                for (int r = 0; r < R; ++r) acc[r] += dot16<BF16>(raw[r][uu], xp);
             }
         }
 #pragma unroll
@@ -211,8 +214,9 @@ static void launch_pro(const GemvArgs &a, dim3 grid, size_t lds, hipStream_t s) 
 int launch_gemv(lumen_ctx *ctx, const GemvArgs &a) {
     if (a.N <= 0 || a.K <= 0) return LUMEN_OK;
     const int vec = a.w_bf16 ? 8 : 4;
-    const int sweep = 64 * vec;
-    const int kpad = (a.K + sweep - 1) / sweep * sweep;
+    const int R = (a.epi == EPI_SWIGLU || a.N >= 8192) ? 2 : 1;
+    const int piece = 64 * vec * (8 / R);  // x is staged zero-padded to whole pieces
+    const int kpad = (a.K + piece - 1) / piece * piece;
     const size_t lds = (size_t)kpad * sizeof(float);
     const bool aligned = (((uintptr_t)a.W | (uintptr_t)a.x) & 15) == 0 &&
                          (a.pro != PRO_RMSNORM || ((uintptr_t)a.norm_w & 15) == 0);
@@ -231,7 +235,6 @@ int launch_gemv(lumen_ctx *ctx, const GemvArgs &a) {
         return LUMEN_OK;
     }
     if (a.epi == EPI_SWIGLU && (a.N & 1)) LUMEN_FAIL(LUMEN_ERR_SHAPE, "SwiGLU epilogue needs an even row count, got %d", a.N);
-    const int R = (a.epi == EPI_SWIGLU || a.N >= 8192) ? 2 : 1;
     const int nunits = (a.N + R - 1) / R;
     int blocks = (nunits + GEMV_WAVES - 1) / GEMV_WAVES;
     const int cap = ctx->num_cus * 4;

@@ -59,11 +59,57 @@ static inline float __uint_as_float(unsigned u) {
     memcpy(&f, &u, 4);
     return f;
 }
+static inline int __float_as_int(float f) {
+    int i;
+    memcpy(&i, &f, 4);
+    return i;
+}
+static inline float __int_as_float(int i) {
+    float f;
+    memcpy(&f, &i, 4);
+    return f;
+}
+static inline float emu_exp2f(float x) { return exp2f(x); }
+#define __builtin_amdgcn_exp2f(x) emu_exp2f(x)
+// DPP row_ror:n (control 0x121..0x12f): lane i of each 16-lane row receives the value of lane (i - n) mod 16
+static inline int emu_update_dpp(int old, int src, int ctrl) {
+    (void)old;
+    const int lane = threadIdx.x & 63;
+    int v = src;
+    if (ctrl >= 0x121 && ctrl <= 0x12f) {
+        const int n = ctrl - 0x120, row = lane & ~15, i = lane & 15;
+        const int from = row + ((i - n) & 15);
+        const int wave = threadIdx.x >> 6;
+        uint32_t *s = emu_block->slots.data() + wave * 64;
+        memcpy(&s[lane], &src, 4);
+        pthread_barrier_wait(&emu_block->wave_bar[wave]);
+        memcpy(&v, &s[from], 4);
+        pthread_barrier_wait(&emu_block->wave_bar[wave]);
+    }
+    return v;
+}
+#define __builtin_amdgcn_update_dpp(old, src, ctrl, rm, bm, bc) emu_update_dpp((old), (src), (ctrl))
 static inline int min(int a, int b) { return a < b ? a : b; }
 static inline int max(int a, int b) { return a > b ? a : b; }
 
-#define __hip_atomic_load(p, order, scope) __atomic_load_n((p), __ATOMIC_SEQ_CST)
-#define __hip_atomic_store(p, v, order, scope) __atomic_store_n((p), (v), __ATOMIC_SEQ_CST)
+template <typename T>
+static inline T emu_atomic_load(const T *p) {
+    static_assert(sizeof(T) == 4, "32-bit atomics only");
+    uint32_t u = __atomic_load_n((const uint32_t *)p, __ATOMIC_SEQ_CST);
+    T v;
+    memcpy(&v, &u, 4);
+    return v;
+}
+template <typename T, typename V>
+static inline void emu_atomic_store(T *p, V val) {
+    static_assert(sizeof(T) == 4, "32-bit atomics only");
+    const T v = (T)val;
+    uint32_t u;
+    memcpy(&u, &v, 4);
+    __atomic_store_n((uint32_t *)p, u, __ATOMIC_SEQ_CST);
+}
+#define __hip_atomic_load(p, order, scope) emu_atomic_load(p)
+#define __hip_atomic_store(p, v, order, scope) emu_atomic_store((p), (v))
 #define __hip_atomic_fetch_add(p, v, order, scope) __atomic_fetch_add((p), (v), __ATOMIC_SEQ_CST)
 static inline int atomicAdd(int *p, int v) { return __atomic_fetch_add(p, v, __ATOMIC_SEQ_CST); }
 static inline void __threadfence() { __atomic_thread_fence(__ATOMIC_SEQ_CST); }
