@@ -26,7 +26,9 @@ struct DecodeWaves {
     static constexpr int value = 8;
 };
 
-template <int D, int NREP, int WAVES>
+// PRE: q arrives rotated and cache row `pos` is already written (both done by the q|k|v GEMV's
+// epilogue), so the kernel is only the row loop over [0, pos] and the merges.
+template <int D, int NREP, int WAVES, bool PRE>
 __global__ __launch_bounds__(WAVES * 64) void attn_decode_kernel(AttnDecodeArgs a) {
     typedef AttnGeom<D, WAVES> G;
     constexpr int THREADS = WAVES * 64;
@@ -40,12 +42,13 @@ __global__ __launch_bounds__(WAVES * 64) void attn_decode_kernel(AttnDecodeArgs 
     __shared__ int s_last;
 
     const int split = blockIdx.x, hk = blockIdx.y, bb = blockIdx.z;
-    const int pos = a.pos_dev ? *a.pos_dev : a.pos_host;  // == past_len
+    const int pos_new = a.pos_dev ? *a.pos_dev : a.pos_host;  // == past_len, the new token's position
+    const int pos = PRE ? pos_new + 1 : pos_new;             // rows that come from the cache
     int nact, chunk;
     decode_slices<D, WAVES>(pos, gridDim.x, nact, chunk);
     if (split >= nact) return;
-    const bool has_new = (split == nact - 1);
-    const float *cs = a.cos_t + (size_t)pos * D, *sn = a.sin_t + (size_t)pos * D;
+    const bool has_new = !PRE && (split == nact - 1);
+    const float *cs = a.cos_t + (size_t)pos_new * D, *sn = a.sin_t + (size_t)pos_new * D;
     const size_t head_base = ((size_t)bb * a.hkv + hk) * a.max_seq * D;
     const float *Kb = a.k_cache + head_base, *Vb = a.v_cache + head_base;
 
@@ -57,6 +60,12 @@ __global__ __launch_bounds__(WAVES * 64) void attn_decode_kernel(AttnDecodeArgs 
 
     // stage raw q heads of this KV group (contiguous: hq = hk*NREP + r) and the new k / v
     const float *q_src = a.q + ((size_t)bb * a.hq + (size_t)hk * NREP) * D;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int slot = lane / G::LPR, c = lane % G::LPR;
+    v4f q[NREP];
+    if (PRE) {
+        load_q_scaled<D, NREP>(q, q_src, c, a.scale);
+    } else {
     for (int i = threadIdx.x; i < NREP * D; i += THREADS) q_raw[i] = q_src[i];
     if (has_new) {
         const float *k_src = a.k_new + ((size_t)bb * a.hkv + hk) * D;
@@ -77,11 +86,8 @@ __global__ __launch_bounds__(WAVES * 64) void attn_decode_kernel(AttnDecodeArgs 
             a.v_cache[head_base + (size_t)pos * D + i] = v_new[i];
         }
     }
-
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int slot = lane / G::LPR, c = lane % G::LPR;
-    v4f q[NREP];
     load_q_scaled<D, NREP>(q, q_rot, c, a.scale);
+    }
 
     AttnState<NREP> st;
     state_init<NREP>(st);
@@ -148,8 +154,14 @@ static int launch_decode_d(lumen_ctx *ctx, const AttnDecodeArgs &a) {
     dim3 grid(a.nsplit, a.hkv, a.b);
     const int nrep = a.hq / a.hkv;
 #define LAUNCH_DECODE(NR)                                                                                     \
-    hipLaunchKernelGGL((attn_decode_kernel<D, NR, DecodeWaves<D, NR>::value>), grid,                          \
-                       dim3(DecodeWaves<D, NR>::value * 64), 0, ctx->stream, a)
+    do {                                                                                                      \
+        if (a.pre_rotated)                                                                                    \
+            hipLaunchKernelGGL((attn_decode_kernel<D, NR, DecodeWaves<D, NR>::value, true>), grid,            \
+                               dim3(DecodeWaves<D, NR>::value * 64), 0, ctx->stream, a);                      \
+        else                                                                                                  \
+            hipLaunchKernelGGL((attn_decode_kernel<D, NR, DecodeWaves<D, NR>::value, false>), grid,           \
+                               dim3(DecodeWaves<D, NR>::value * 64), 0, ctx->stream, a);                      \
+    } while (0)
     switch (nrep) {
         case 1: LAUNCH_DECODE(1); break;
         case 2: LAUNCH_DECODE(2); break;

@@ -251,16 +251,29 @@ __device__ __forceinline__ float part_load(const float *p) {
 // self_attention.rs:287-290.  pp points at the head's first partial; entries are (D + 2) floats apart.
 template <int D>
 __device__ __forceinline__ float fold_slices(const float *pp, int nact, int dd) {
-    float mm = -INFINITY;
-    for (int s = 0; s < nact; ++s) mm = fmaxf(mm, part_load(pp + (size_t)s * (D + 2) + D));
-    float ls = 0.f, cx = 0.f;
-    for (int s = 0; s < nact; ++s) {
-        const float ms = part_load(pp + (size_t)s * (D + 2) + D);
-        const float ex = (ms > -INFINITY) ? fast_exp2(ms - mm) : 0.f;
-        ls = fmaf(part_load(pp + (size_t)s * (D + 2) + D + 1), ex, ls);
-        cx = fmaf(part_load(pp + (size_t)s * (D + 2) + dd), ex, cx);
+    constexpr int B = 8;  // slices fetched together: 3 * B independent loads in flight, one wait
+    float M = -INFINITY, Ls = 0.f, Cx = 0.f;
+    for (int s0 = 0; s0 < nact; s0 += B) {
+        float mv[B], lv[B], cv[B];
+#pragma unroll
+        for (int j = 0; j < B; ++j) {
+            const float *e = pp + (size_t)min(s0 + j, nact - 1) * (D + 2);
+            mv[j] = part_load(e + D);
+            lv[j] = part_load(e + D + 1);
+            cv[j] = part_load(e + dd);
+        }
+#pragma unroll
+        for (int j = 0; j < B; ++j) {
+            if (s0 + j < nact && mv[j] > -INFINITY) {
+                const float mn = fmaxf(M, mv[j]);
+                const float a = fast_exp2(M - mn), b = fast_exp2(mv[j] - mn);
+                Ls = Ls * a + lv[j] * b;
+                Cx = Cx * a + cv[j] * b;
+                M = mn;
+            }
+        }
     }
-    return cx * (1.0f / (ls + 1e-9f));
+    return Cx * (1.0f / (Ls + 1e-9f));
 }
 
 // How the cached rows [0, pos) are cut into slices for one decode step: only

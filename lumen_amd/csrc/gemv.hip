@@ -111,6 +111,13 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(GemvArgs a) {
     const int nunits = (N + R - 1) / R;
     const char *Wb = (const char *)a.W;
     const size_t row_bytes = (size_t)K * ESZ;
+    const int half_d = a.D >> 1;
+
+    // row r of unit u: consecutive rows, or the RoPE pair (j, j + D/2) of one head
+    auto unit_row = [&](int u, int r) {
+        if (EPI == EPI_ROPE_QKV) return (u / half_d) * a.D + (u % half_d) + r * half_d;
+        return u * R + r;
+    };
 
     // 8 x 16 bytes per lane of unit u from element k0 on.  Every load is issued unconditionally:
     // positions past the end of the row are clamped to its last 16 bytes (they meet the zero
@@ -118,7 +125,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(GemvArgs a) {
     auto load_piece = [&](int u, int k0, v4u (&raw)[R][U]) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int row = min(u * R + r, N - 1);
+            const int row = min(unit_row(u, r), N - 1);
             const char *rp = Wb + (size_t)row * row_bytes;
 #pragma unroll
             for (int uu = 0; uu < U; ++uu) {
@@ -132,7 +139,11 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(GemvArgs a) {
     v4u raw[R][U];
     load_piece(min(gw, nunits - 1), 0, raw);
 
-    stage_x<PRO>(xs, a.x, a.norm_w, a.eps, K, kpad);
+    const long sel_off = a.row_sel ? (long)(*a.row_sel) * a.row_stride : 0;
+    stage_x<PRO>(xs, a.x + (a.x_sel ? sel_off : 0), a.norm_w, a.eps, K, kpad);
+    const float *residual = a.residual + (a.residual_sel ? sel_off : 0);
+    float best = -INFINITY;
+    int best_idx = 0x7fffffff;
 
     for (int u = gw; u < nunits; u += nw) {
         float acc[R];
@@ -149,20 +160,121 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(GemvArgs a) {
         }
 #pragma unroll
         for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
+        if (EPI == EPI_ARGMAX) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const int row = u * R + r;
+                if (row < N && (acc[r] > best || (acc[r] == best && row < best_idx))) {
+                    best = acc[r];
+                    best_idx = row;
+                }
+            }
+        }
         if (lane == 0) {
             if (EPI == EPI_SWIGLU) {
                 // rows (2u, 2u+1) hold (gate_u, up_u): silu(gate) * up, src/models/llama.rs:60-63
                 a.y[u] = silu_f(acc[0]) * acc[R - 1];
+            } else if (EPI == EPI_ROPE_QKV) {
+                // half-split rotation at the token's position (src/layers/attention/encoding.rs:196-203,
+                // self_attention.rs:220-227); k and v land in cache row pos (self_attention.rs:161-176)
+                const int head = u / half_d, j = u % half_d;
+                const int pos = *a.pos;
+                const float c = a.cos_t[(size_t)pos * a.D + j], sn = a.sin_t[(size_t)pos * a.D + j];
+                const float x1 = acc[0], x2 = acc[R - 1];
+                float o1, o2;
+                {
+#pragma clang fp contract(off)
+                    o1 = x1 * c - x2 * sn;
+                    o2 = x1 * sn + x2 * c;
+                }
+                if (head < a.hq) {
+                    a.y[head * a.D + j] = o1;
+                    a.y[head * a.D + j + half_d] = o2;
+                } else if (head < a.hq + a.hkv) {
+                    float *dst = a.k_cache + ((size_t)(head - a.hq) * a.max_seq + pos) * a.D;
+                    dst[j] = o1;
+                    dst[j + half_d] = o2;
+                } else {
+                    float *dst = a.v_cache + ((size_t)(head - a.hq - a.hkv) * a.max_seq + pos) * a.D;
+                    dst[j] = x1;
+                    dst[j + half_d] = x2;
+                }
             } else {
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     const int row = u * R + r;
                     if (row < N) {
                         // residual: x + y, src/ops/arithmetic.rs:48-51 via src/models/llama.rs:110,115
-                        a.y[row] = (EPI == EPI_RESIDUAL) ? a.residual[row] + acc[r] : acc[r];
+                        a.y[row] = (EPI == EPI_RESIDUAL) ? residual[row] + acc[r] : acc[r];
                     }
                 }
             }
+        }
+    }
+
+    if (EPI == EPI_ARGMAX) {
+        // greedy pick fused into the lm_head product: per-workgroup candidates go through memory with
+        // agent-scope accesses, the last workgroup to arrive folds them (lowest index wins ties)
+        __shared__ float am_v[GEMV_WAVES];
+        __shared__ int am_i[GEMV_WAVES];
+        __shared__ int am_last;
+        const int wave = threadIdx.x >> 6;
+        if (lane == 0) {
+            am_v[wave] = best;
+            am_i[wave] = best_idx;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            for (int w = 1; w < GEMV_WAVES; ++w)
+                if (am_v[w] > best || (am_v[w] == best && am_i[w] < best_idx)) {
+                    best = am_v[w];
+                    best_idx = am_i[w];
+                }
+            __hip_atomic_store(a.amax_val + blockIdx.x, best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(a.amax_idx + blockIdx.x, best_idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();  // thread 0's stores are complete past this barrier
+        if (threadIdx.x == 0) {
+            const int old = __hip_atomic_fetch_add(a.amax_counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            am_last = (old == (int)gridDim.x - 1);
+            if (am_last) __hip_atomic_store(a.amax_counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+        if (!am_last) return;
+        float bv = -INFINITY;
+        int bi = 0x7fffffff;
+        for (int i = threadIdx.x; i < (int)gridDim.x; i += GEMV_THREADS) {
+            const float v = __hip_atomic_load(a.amax_val + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const int ix = __hip_atomic_load(a.amax_idx + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (v > bv || (v == bv && ix < bi)) {
+                bv = v;
+                bi = ix;
+            }
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const float ov = __shfl_xor(bv, off, 64);
+            const int oi = __shfl_xor(bi, off, 64);
+            if (ov > bv || (ov == bv && oi < bi)) {
+                bv = ov;
+                bi = oi;
+            }
+        }
+        __syncthreads();
+        if (lane == 0) {
+            am_v[wave] = bv;
+            am_i[wave] = bi;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            for (int w = 1; w < GEMV_WAVES; ++w)
+                if (am_v[w] > bv || (am_v[w] == bv && am_i[w] < bi)) {
+                    bv = am_v[w];
+                    bi = am_i[w];
+                }
+            if (bi == 0x7fffffff) bi = 0;  // all NaN: index 0 like a sequential scan
+            *a.tok_out = bi;
+            if (a.pos_inc) *a.pos_inc += 1;
         }
     }
 }
@@ -197,6 +309,12 @@ static void launch_epi(const GemvArgs &a, dim3 grid, size_t lds, hipStream_t s) 
         case EPI_RESIDUAL:
             hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_RESIDUAL>), grid, dim3(GEMV_THREADS), lds, s, a);
             break;
+        case EPI_ARGMAX:
+            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_ARGMAX>), grid, dim3(GEMV_THREADS), lds, s, a);
+            break;
+        case EPI_ROPE_QKV:
+            hipLaunchKernelGGL((gemv_kernel<BF16, 2, PRO, EPI_ROPE_QKV>), grid, dim3(GEMV_THREADS), lds, s, a);
+            break;
         default:
             hipLaunchKernelGGL((gemv_kernel<BF16, 2, PRO, EPI_SWIGLU>), grid, dim3(GEMV_THREADS), lds, s, a);
             break;
@@ -211,10 +329,12 @@ static void launch_pro(const GemvArgs &a, dim3 grid, size_t lds, hipStream_t s) 
         launch_epi<BF16, R, PRO_NONE>(a, grid, lds, s);
 }
 
+int gemv_max_blocks(const lumen_ctx *ctx) { return ctx->num_cus * 4; }
+
 int launch_gemv(lumen_ctx *ctx, const GemvArgs &a) {
     if (a.N <= 0 || a.K <= 0) return LUMEN_OK;
     const int vec = a.w_bf16 ? 8 : 4;
-    const int R = (a.epi == EPI_SWIGLU || a.N >= 8192) ? 2 : 1;
+    const int R = (a.epi == EPI_SWIGLU || a.epi == EPI_ROPE_QKV || a.N >= 8192) ? 2 : 1;
     const int piece = 64 * vec * (8 / R);  // x is staged zero-padded to whole pieces
     const int kpad = (a.K + piece - 1) / piece * piece;
     const size_t lds = (size_t)kpad * sizeof(float);
@@ -222,7 +342,7 @@ int launch_gemv(lumen_ctx *ctx, const GemvArgs &a) {
                          (a.pro != PRO_RMSNORM || ((uintptr_t)a.norm_w & 15) == 0);
     const bool fast = (a.K % vec == 0) && aligned && lds <= 64 * 1024;
     if (!fast) {
-        if (a.pro != PRO_NONE || a.epi != EPI_STORE)
+        if (a.pro != PRO_NONE || a.epi != EPI_STORE || a.row_sel)
             LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "fused GEMV needs K %% %d == 0, 16-byte alignment and K <= %d (K=%d)", vec,
                        16384, a.K);
         int blocks = (a.N + GEMV_WAVES - 1) / GEMV_WAVES;
@@ -234,7 +354,8 @@ int launch_gemv(lumen_ctx *ctx, const GemvArgs &a) {
         LUMEN_CHECK_LAUNCH();
         return LUMEN_OK;
     }
-    if (a.epi == EPI_SWIGLU && (a.N & 1)) LUMEN_FAIL(LUMEN_ERR_SHAPE, "SwiGLU epilogue needs an even row count, got %d", a.N);
+    if ((a.epi == EPI_SWIGLU || a.epi == EPI_ROPE_QKV) && (a.N & 1))
+        LUMEN_FAIL(LUMEN_ERR_SHAPE, "paired-row epilogue needs an even row count, got %d", a.N);
     const int nunits = (a.N + R - 1) / R;
     int blocks = (nunits + GEMV_WAVES - 1) / GEMV_WAVES;
     const int cap = ctx->num_cus * 4;

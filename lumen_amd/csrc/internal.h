@@ -70,7 +70,7 @@ struct lumen_kv_cache {
 // Every launcher validates nothing: callers check shapes first.
 
 enum GemvPro { PRO_NONE = 0, PRO_RMSNORM = 1 };
-enum GemvEpi { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2 };
+enum GemvEpi { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2, EPI_ARGMAX = 3, EPI_ROPE_QKV = 4 };
 
 struct GemvArgs {
     const void *W;        // [N, K] f32 or bf16 bits
@@ -82,8 +82,26 @@ struct GemvArgs {
     const float *norm_w;  // PRO_RMSNORM: gain [K]
     float eps;
     const float *residual;  // EPI_RESIDUAL: [N]
+    // x (and, with residual_sel, the residual) is row *row_sel of a [rows, row_stride] table:
+    // the embedding gather folded into the first layer's GEMVs
+    const int *row_sel;
+    long row_stride;
+    int x_sel, residual_sel;
+    // EPI_ARGMAX: y still receives the N values; the index of the first maximum goes to *tok_out
+    // and *pos_inc is incremented, by the last workgroup to finish
+    float *amax_val;   // [gridDim.x]
+    int *amax_idx;     // [gridDim.x]
+    int *amax_counter; // zero between launches
+    int *tok_out, *pos_inc;
+    // EPI_ROPE_QKV: rows are q|k|v heads of D; a unit is the RoPE pair (j, j + D/2) of one head.
+    // q is rotated into y, k rotated and v as is go to row *pos of the KV cache.
+    const float *cos_t, *sin_t;
+    const int *pos;
+    float *k_cache, *v_cache;  // [hkv, max_seq, D]
+    int hq, hkv, D, max_seq;
 };
 int launch_gemv(lumen_ctx *ctx, const GemvArgs &a);
+int gemv_max_blocks(const lumen_ctx *ctx);
 
 struct GemmArgs {
     const float *A;   // [M, K]
@@ -126,6 +144,7 @@ struct AttnDecodeArgs {
     float *part;        // split scratch
     int *counters;
     int nsplit;
+    int pre_rotated;    // q is already rotated and row pos of the cache already written (fused QKV GEMV)
 };
 int launch_attn_decode(lumen_ctx *ctx, const AttnDecodeArgs &a);
 

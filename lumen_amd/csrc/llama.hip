@@ -49,6 +49,7 @@ struct lumen_llama {
     PkLayer *pk_layers = nullptr;          // device copy of the per-layer pointers
     float *amax_val = nullptr;
     int *amax_idx = nullptr;
+    int *amax_counter = nullptr;
     unsigned *d_bar = nullptr;
     int *d_err = nullptr;
     // prefill buffers (grown on demand, kept)
@@ -191,8 +192,15 @@ extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg,
         }
         M_TRY(dmalloc_t(m, &m->pk_layers, (size_t)L));
         M_TRY(lumen_upload(ctx, m->pk_layers, pl.data(), sizeof(PkLayer) * (size_t)L));
-        M_TRY(dmalloc_t(m, &m->amax_val, (size_t)ctx->num_cus));
-        M_TRY(dmalloc_t(m, &m->amax_idx, (size_t)ctx->num_cus));
+        const size_t nb = (size_t)std::max(gemv_max_blocks(ctx), ctx->num_cus);
+        M_TRY(dmalloc_t(m, &m->amax_val, nb));
+        M_TRY(dmalloc_t(m, &m->amax_idx, nb));
+        M_TRY(dmalloc_t(m, &m->amax_counter, 4));
+        if (hipMemsetAsync(m->amax_counter, 0, 4 * sizeof(int), ctx->stream) != hipSuccess ||
+            hipStreamSynchronize(ctx->stream) != hipSuccess) {
+            lumen_llama_destroy(m);
+            LUMEN_FAIL(LUMEN_ERR_HIP, "llama_create: clearing the arg-max counter failed");
+        }
         M_TRY(dmalloc_t(m, &m->d_bar, 4));
         M_TRY(dmalloc_t(m, &m->d_err, 4));
     }
@@ -367,15 +375,21 @@ static int enqueue_decode_step(lumen_llama *m, StepProbe *pr = nullptr) {
     lumen_ctx *ctx = m->ctx;
     const lumen_llama_config &c = m->cfg;
     const int H = c.hidden_size, I = c.intermediate_size, V = c.vocab_size;
-    pr->before(KC_EMBED);
-    LUMEN_TRY(launch_embedding(ctx, m->embed, m->d_tok, 1, H, V, m->x));  // llama.rs:191
-    pr->after();
+    // Embedding::forward (llama.rs:191) is folded into the first layer: its GEMVs read row *d_tok of
+    // the table directly.  RoPE + KV append ride on the q|k|v product unless q/k need a per-head norm first.
+    const bool fuse_rope = !c.qk_norm;
     for (int l = 0; l < c.num_hidden_layers; ++l) {
         const LayerW &w = m->layers[l];
         GemvArgs g = {};
         // input_layernorm + q|k|v projections, llama.rs:107, self_attention.rs:106-108
         g.W = w.wqkv; g.x = m->x; g.y = m->qkv; g.N = m->qkvd; g.K = H; g.w_bf16 = m->bf16;
         g.pro = PRO_RMSNORM; g.norm_w = w.in_norm; g.eps = c.rms_norm_eps; g.epi = EPI_STORE;
+        if (l == 0) { g.x = m->embed; g.row_sel = m->d_tok; g.row_stride = H; g.x_sel = 1; }
+        if (fuse_rope) {
+            g.epi = EPI_ROPE_QKV; g.cos_t = m->cos_dev; g.sin_t = m->sin_dev; g.pos = m->d_pos;
+            g.k_cache = m->k_slab + m->cache_stride * l; g.v_cache = m->v_slab + m->cache_stride * l;
+            g.hq = c.num_attention_heads; g.hkv = c.num_key_value_heads; g.D = m->D; g.max_seq = c.max_seq_len;
+        }
         pr->before(KC_QKV);
         LUMEN_TRY(launch_gemv(ctx, g));
         pr->after();
@@ -385,7 +399,7 @@ static int enqueue_decode_step(lumen_llama *m, StepProbe *pr = nullptr) {
         a.cos_t = m->cos_dev; a.sin_t = m->sin_dev; a.pos_dev = m->d_pos; a.pos_host = 0;
         a.b = 1; a.hq = c.num_attention_heads; a.hkv = c.num_key_value_heads; a.d = m->D; a.max_seq = c.max_seq_len;
         a.scale = m->scale; a.q_norm_w = w.q_norm; a.k_norm_w = w.k_norm; a.norm_eps = c.rms_norm_eps;
-        a.part = m->part; a.counters = m->counters; a.nsplit = m->nsplit;
+        a.part = m->part; a.counters = m->counters; a.nsplit = m->nsplit; a.pre_rotated = fuse_rope;
         pr->before(KC_ATTN);
         LUMEN_TRY(launch_attn_decode(ctx, a));
         pr->after();
@@ -393,6 +407,7 @@ static int enqueue_decode_step(lumen_llama *m, StepProbe *pr = nullptr) {
         g = {};
         g.W = w.wo; g.x = m->attn; g.y = m->h; g.N = H; g.K = m->qd; g.w_bf16 = m->bf16;
         g.pro = PRO_NONE; g.epi = EPI_RESIDUAL; g.residual = m->x;
+        if (l == 0) { g.residual = m->embed; g.row_sel = m->d_tok; g.row_stride = H; g.residual_sel = 1; }
         pr->before(KC_OPROJ);
         LUMEN_TRY(launch_gemv(ctx, g));
         pr->after();
@@ -415,13 +430,12 @@ static int enqueue_decode_step(lumen_llama *m, StepProbe *pr = nullptr) {
     GemvArgs g = {};
     g.W = m->lm_head; g.x = m->x; g.y = m->logits; g.N = V; g.K = H;
     g.w_bf16 = (m->lm_head == (void *)m->embed) ? 0 : (int)m->bf16;
-    g.pro = PRO_RMSNORM; g.norm_w = m->final_norm; g.eps = c.rms_norm_eps; g.epi = EPI_STORE;
+    g.pro = PRO_RMSNORM; g.norm_w = m->final_norm; g.eps = c.rms_norm_eps;
+    // the greedy pick is folded in: it becomes the next token id and the position counter advances
+    g.epi = EPI_ARGMAX; g.amax_val = m->amax_val; g.amax_idx = m->amax_idx; g.amax_counter = m->amax_counter;
+    g.tok_out = m->d_tok; g.pos_inc = m->d_pos;
     pr->before(KC_LMHEAD);
-    LUMEN_TRY(launch_gemv(ctx, g));
-    pr->after();
-    // greedy pick becomes the next token id; the position counter advances
-    pr->before(KC_ARGMAX);
-    const int rc = launch_argmax(ctx, m->logits, V, m->d_tok, m->d_pos);
+    const int rc = launch_gemv(ctx, g);
     pr->after();
     return rc;
 }
