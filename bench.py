@@ -36,10 +36,18 @@ def main():
                     help="how decode steps are issued: a HIP graph replay per token (default) or kernel by kernel "
                          "(for rocprofv3 --kernel-trace, which cannot follow graph replays here)")
     ap.add_argument("--cpu-tokens", type=int, default=48)
+    ap.add_argument("--workload", choices=["decode", "gemv", "copy"], default="decode",
+                    help="decode: the headline batch-1 decode benchmark; gemv: the isolated M=1 GEMV shapes; "
+                         "copy: a plain 1 GiB copy kernel (calibrates the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs the batch-1 decode path on ONE GPU; --gpus %d is not supported "
                  "(nothing here shards across GPUs)" % args.gpus)
+
+    if args.workload == "gemv":
+        return gemv_microbench(args)
+    if args.workload == "copy":
+        return copy_bench(args)
 
     import numpy as np
 
@@ -107,9 +115,9 @@ def main():
                                "greedy decode, static KV cache max_seq_len %d" % (args.prompt, cfg["max_seq_len"]),
                    "layers": cfg["num_hidden_layers"], "hidden": H, "heads": "32q/4kv", "head_dim": 64,
                    "intermediate": I, "vocab": cfg["vocab_size"], "kv_len_during_timing": [len0, len0 + args.steps]},
-        "roofline": {"bound": "hbm", "kernel": "gemv_kernel<f32,R=2,RMSNORM,SWIGLU> (norm+gate|up GEMV, [11264,2048])",
+        "roofline": {"bound": "hbm", "kernel": "gemv_kernel<false, 2, 1, 2> (RMSNorm + gate|up GEMV [11264,2048] + SwiGLU)",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic(),
                      "bytes_per_launch": gu_bytes, "avg_launch_us": round(gu_avg_ms * 1e3, 3)},
         "step_roofline": {"bytes_per_token": step_bytes, "achieved_GBps": round(step_bytes / (ms_per_step * 1e-3) / 1e9, 1),
                           "frac_of_8TBps": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
@@ -122,6 +130,79 @@ def main():
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, params, prompt, args.cpu_tokens)
     print(json.dumps(out))
+
+
+def measured_traffic():
+    """HBM bytes per launch of the dominant kernel from the committed rocprofv3 --pmc runs
+    (FETCH_SIZE + WRITE_SIZE, calibrated on the copy kernel); counters cannot be read from here."""
+    path = os.path.join(ROOT, "profiles", "decode_gateup_gemv_traffic.json")
+    try:
+        with open(path) as f:
+            t = json.load(f)
+        return round(t["fetch_bytes_per_launch"] + t["write_bytes_per_launch"], 1)
+    except (OSError, KeyError, ValueError):
+        return None
+
+
+def copy_bench(args):
+    """out[i] = in[i] over 2^28 floats: 1 GiB read + 1 GiB written per launch."""
+    import numpy as np
+
+    from lumen_amd._lib import check, lib
+    from lumen_amd.autograd import Tensor, default_ctx
+
+    ctx = default_ctx()
+    n = 1 << 28
+    src, dst = Tensor.empty((n,), np.float32, ctx), Tensor.empty((n,), np.float32, ctx)
+    check(lib.lumen_copy_f32(ctx.handle, dst.ptr, src.ptr, n))  # touch both
+    iters = 10
+    ctx.timer_start()
+    for _ in range(iters):
+        check(lib.lumen_copy_f32(ctx.handle, src.ptr, dst.ptr, n))
+    ms = ctx.timer_stop() / iters
+    print(json.dumps({"metric": "copy GB/s", "bytes_read": 4 * n, "bytes_written": 4 * n, "ms": round(ms, 4),
+                      "GBps_read_plus_write": round(8 * n / ms / 1e6, 1)}))
+
+
+GEMV_SHAPES = [(2048, 2048), (2048, 256), (2048, 5632), (5632, 2048), (2048, 32000), (4096, 11008), (11008, 4096)]
+
+
+def gemv_microbench(args):
+    """Isolated M=1 GEMV, fp32, logical (K, N) stored [N, K] like the reference's Linear weights.
+    Each launch reads a different copy of W (>= 1.2 GB of copies in rotation) so the figure is HBM
+    bandwidth, not L2 / memory-side-cache bandwidth; algorithmic bytes = 4 (K N + K + N)."""
+    import ctypes as C
+
+    import numpy as np
+
+    from lumen_amd._lib import check, lib
+    from lumen_amd.autograd import Tensor, default_ctx
+
+    ctx = default_ctx()
+    rows = []
+    for K, N in GEMV_SHAPES:
+        rng = np.random.default_rng(K * 100003 + N)
+        W = (rng.standard_normal((N, K), dtype=np.float32) * np.float32(0.02))
+        x = rng.standard_normal(K, dtype=np.float32)
+        ncopies = max(2, int(np.ceil(1.2e9 / W.nbytes)))
+        slab = Tensor.empty((ncopies, N, K), np.float32, ctx)
+        for c in range(ncopies):
+            check(lib.lumen_upload(ctx.handle, slab.ptr + c * W.nbytes, W.ctypes.data, W.nbytes))
+        xd, yd = Tensor.from_array_no_grad(x, ctx), Tensor.empty((N,), np.float32, ctx)
+        ms = C.c_float()
+        check(lib.lumen_gemv_bench(ctx.handle, slab.ptr, N * K, ncopies, 0, xd.ptr, yd.ptr, N, K, args.warmup or 8, C.byref(ms)))
+        iters = max(args.steps, 200)
+        check(lib.lumen_gemv_bench(ctx.handle, slab.ptr, N * K, ncopies, 0, xd.ptr, yd.ptr, N, K, iters, C.byref(ms)))
+        ref = W.astype(np.float64) @ x.astype(np.float64)
+        err = float(np.abs(yd.data() - ref).max() / np.abs(ref).max())
+        us = ms.value * 1e3 / iters
+        nbytes = 4.0 * (K * N + K + N)
+        rows.append({"K": K, "N": N, "us": round(us, 3), "GBps": round(nbytes / us / 1e3, 1),
+                     "frac_of_8TBps": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), "max_rel_err": err,
+                     "weight_copies": ncopies})
+        del slab
+    print(json.dumps({"metric": "M=1 GEMV HBM GB/s", "unit": "GB/s", "n_gpus": 1, "dtype": "f32", "data": "synthetic",
+                      "layout": "[N,K] row-major (out,in)", "shapes": rows}))
 
 
 def cpu_baseline(cfg, params, prompt, n_tokens):

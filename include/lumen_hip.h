@@ -89,11 +89,21 @@ int lumen_gemv_bf16w(lumen_ctx *ctx, const uint16_t *W_dev, const float *x_dev, 
 int lumen_gemm_bf16w(lumen_ctx *ctx, const float *A_dev, const uint16_t *W_dev, float *C_dev,
                      int M, int N, int K);
 
+/* measurement aid (no reference counterpart): iters GEMVs back to back on the ctx
+ * stream, launch i using the weight matrix at W_base + (i % ncopies) * stride_elems
+ * elements, so that each launch streams from HBM and not from a cache; ms_out is the
+ * HIP-event time of the whole run. */
+int lumen_gemv_bench(lumen_ctx *ctx, const void *W_base_dev, size_t stride_elems, int ncopies,
+                     int w_bf16, const float *x_dev, float *y_dev, int N, int K, int iters,
+                     float *ms_out);
+
 /* RMSNorm::forward, src/layers/norm/rms_norm.rs:24-62.  x [rows, dim], w [dim] */
 int lumen_rmsnorm_f32(lumen_ctx *ctx, const float *x_dev, const float *w_dev, float *out_dev,
                       int rows, int dim, float eps);
 /* SiLU::forward, src/layers/activation.rs:139-146 */
 int lumen_silu_f32(lumen_ctx *ctx, const float *x_dev, float *out_dev, size_t n);
+/* plain device copy out[i] = x[i] (Tensor::detach / to_owned, src/autograd.rs:262-266) */
+int lumen_copy_f32(lumen_ctx *ctx, const float *x_dev, float *out_dev, size_t n);
 /* Tensor + Tensor and Tensor * Tensor, same shape, src/ops/arithmetic.rs:48-51, 105-108 */
 int lumen_add_f32(lumen_ctx *ctx, const float *a_dev, const float *b_dev, float *out_dev, size_t n);
 int lumen_mul_f32(lumen_ctx *ctx, const float *a_dev, const float *b_dev, float *out_dev, size_t n);

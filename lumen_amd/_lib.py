@@ -54,11 +54,13 @@ SIGNATURES = {
     "lumen_download": (_i, [_vp, _vp, _vp, C.c_size_t]),
     "lumen_matmul_f32": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     "lumen_gemv_f32": (_i, [_vp, _vp, _vp, _vp, _i, _i]),
+    "lumen_gemv_bench": (_i, [_vp, _vp, C.c_size_t, _i, _i, _vp, _vp, _i, _i, _i, C.POINTER(_f)]),
     "lumen_gemm_f32": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i]),
     "lumen_gemv_bf16w": (_i, [_vp, _vp, _vp, _vp, _i, _i]),
     "lumen_gemm_bf16w": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i]),
     "lumen_rmsnorm_f32": (_i, [_vp, _vp, _vp, _vp, _i, _i, _f]),
     "lumen_silu_f32": (_i, [_vp, _vp, _vp, C.c_size_t]),
+    "lumen_copy_f32": (_i, [_vp, _vp, _vp, C.c_size_t]),
     "lumen_add_f32": (_i, [_vp, _vp, _vp, _vp, C.c_size_t]),
     "lumen_mul_f32": (_i, [_vp, _vp, _vp, _vp, C.c_size_t]),
     "lumen_swiglu_f32": (_i, [_vp, _vp, _vp, _vp, C.c_size_t]),

@@ -43,7 +43,7 @@ int launch_rmsnorm(lumen_ctx *ctx, const float *x, const float *w, float *out, i
 }
 
 // -------------------------------------------------------------- elementwise
-enum { OP_SILU, OP_ADD, OP_MUL, OP_SWIGLU };
+enum { OP_SILU, OP_ADD, OP_MUL, OP_SWIGLU, OP_COPY };
 
 template <int OP>
 __global__ __launch_bounds__(256) void ew_kernel(const float *__restrict__ a, const float *__restrict__ b,
@@ -55,6 +55,8 @@ __global__ __launch_bounds__(256) void ew_kernel(const float *__restrict__ a, co
         if (OP == OP_SILU) {
             const float sig = 1.0f / (1.0f + expf(-x));  // src/layers/activation.rs:143-146
             r = x * sig;
+        } else if (OP == OP_COPY) {
+            r = x;
         } else if (OP == OP_ADD) {
             r = x + b[i];
         } else if (OP == OP_MUL) {
@@ -82,6 +84,7 @@ int launch_silu(lumen_ctx *ctx, const float *x, float *out, size_t n) { return l
 int launch_add(lumen_ctx *ctx, const float *a, const float *b, float *out, size_t n) { return launch_ew<OP_ADD>(ctx, a, b, out, n); }
 int launch_mul(lumen_ctx *ctx, const float *a, const float *b, float *out, size_t n) { return launch_ew<OP_MUL>(ctx, a, b, out, n); }
 int launch_swiglu(lumen_ctx *ctx, const float *g, const float *u, float *out, size_t n) { return launch_ew<OP_SWIGLU>(ctx, g, u, out, n); }
+static int launch_copy(lumen_ctx *ctx, const float *x, float *out, size_t n) { return launch_ew<OP_COPY>(ctx, x, x, out, n); }
 
 // ---------------------------------------------------------------- embedding
 // out[t, :] = W[ids[t], :], src/layers/basic/embedding.rs:47-57.  ids were
@@ -229,6 +232,7 @@ extern "C" int lumen_rmsnorm_f32(lumen_ctx *ctx, const float *x, const float *w,
         return fn(ctx, a, b, out, n);                                                             \
     }
 EW_ABI1(lumen_silu_f32, launch_silu)
+EW_ABI1(lumen_copy_f32, launch_copy)
 EW_ABI2(lumen_add_f32, launch_add)
 EW_ABI2(lumen_mul_f32, launch_mul)
 EW_ABI2(lumen_swiglu_f32, launch_swiglu)

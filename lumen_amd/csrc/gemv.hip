@@ -402,3 +402,21 @@ extern "C" int lumen_matmul_f32(lumen_ctx *ctx, const float *A, const float *W, 
     if (M == 1) return lumen_gemv_f32(ctx, W, A, C, N, K_a);  // src/ops/matmul.rs:42
     return lumen_gemm_f32(ctx, A, W, C, M, N, K_a);
 }
+
+// Measurement aid: `iters` GEMVs back to back on the ctx stream, cycling through `ncopies` weight
+// matrices `stride_elems` apart so that every launch streams its weights from HBM rather than from
+// the L2 / memory-side cache; returns the HIP-event time of the whole run.
+extern "C" int lumen_gemv_bench(lumen_ctx *ctx, const void *W_base, size_t stride_elems, int ncopies, int w_bf16,
+                                const float *x, float *y, int N, int K, int iters, float *ms_out) {
+    if (!ctx || !W_base || !x || !y || !ms_out) LUMEN_FAIL(LUMEN_ERR_INVALID, "gemv_bench: null argument");
+    if (ncopies <= 0 || iters <= 0 || N <= 0 || K <= 0) LUMEN_FAIL(LUMEN_ERR_SHAPE, "gemv_bench: non-positive argument");
+    const size_t esz = w_bf16 ? 2 : 4;
+    GemvArgs a = {};
+    a.x = x; a.y = y; a.N = N; a.K = K; a.w_bf16 = w_bf16; a.pro = PRO_NONE; a.epi = EPI_STORE;
+    LUMEN_TRY(lumen_timer_start(ctx));
+    for (int i = 0; i < iters; ++i) {
+        a.W = (const char *)W_base + (size_t)(i % ncopies) * stride_elems * esz;
+        LUMEN_TRY(launch_gemv(ctx, a));
+    }
+    return lumen_timer_stop(ctx, ms_out);
+}
