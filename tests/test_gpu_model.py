@@ -247,3 +247,65 @@ def test_tinyllama_1b_shape_prefill_128_decode_teacher_forced():
     # on-device greedy loop reproduces itself and advances the cache
     a = gpu.decode_greedy(int(ids[0]), 8)
     assert gpu.kv_len == 144 + 8 and a.shape == (8,)
+
+
+def _stream_build(cfg, seed, bf16=False):
+    """Full-width shapes: tensors are generated one at a time and shared by the GPU model and the oracle."""
+    gcfg = dict(cfg, weight_dtype="bf16") if bf16 else dict(cfg)
+    gpu = LlamaModel(gcfg)
+    params = {}
+    for name, a in synth.iter_params(cfg, seed=seed):
+        if bf16 and a.ndim == 2:
+            bits = synth.bf16_round(a)
+            a = synth.bf16_widen(bits)
+            gpu.set_param(name, a if name == "model.embed_tokens.weight" and not cfg.get("tie_embeddings") else bits)
+        else:
+            gpu.set_param(name, a)
+        params[name] = a
+    ocfg = {k: v for k, v in cfg.items() if k != "weight_dtype"}
+    return gpu, lo.Llama(ocfg, params)
+
+
+def _prefill_decode_check(gpu, ora, vocab, n_prompt, n_dec, tol, seed):
+    ids = synth.make_tokens(n_prompt + n_dec, vocab, seed=seed)
+    got = gpu.forward(ids[:n_prompt], all_rows=False)
+    rc, ref = ora.forward(ids[:n_prompt])
+    assert rc == lo.LO_OK
+    assert max_rel(got, ref[-1]) <= tol, max_rel(got, ref[-1])
+    worst = 0.0
+    for t in range(n_prompt, n_prompt + n_dec):
+        g = gpu.forward(ids[t:t + 1], all_rows=False)
+        rc, r = ora.forward(ids[t:t + 1])
+        worst = max(worst, max_rel(g, r[0]))
+        check_argmax(g, r[0], tol)
+    assert worst <= tol, worst
+    assert gpu.kv_len == ora.kv_len == n_prompt + n_dec
+
+
+@pytest.mark.slow
+def test_long_context_tinyllama_shape_3968_prompt():
+    """Config 3 at full width and full context (prompt 3968, decode to the 4096 limit region) on 3 of the
+    22 layers: every kernel shape and the 62-slice attention merge are the real ones."""
+    cfg = dict(synth.TINYLLAMA_1B_LONG, num_hidden_layers=3)
+    gpu, ora = _stream_build(cfg, seed=3)
+    _prefill_decode_check(gpu, ora, cfg["vocab_size"], 3968, 12, 1e-4, seed=3)
+
+
+@pytest.mark.slow
+def test_qwen3_0p6b_shape_prefill_256_decode():
+    """Config 4 shape (head_dim 128 decoupled from hidden 1024, per-head q/k RMSNorm, tied 151936-row
+    embedding, rope_theta 1e6) on 4 of the 28 layers; no reference model exists for it (oracle-extrapolated)."""
+    cfg = dict(synth.QWEN3_0P6B, num_hidden_layers=4)
+    gpu, ora = _stream_build(cfg, seed=4)
+    _prefill_decode_check(gpu, ora, cfg["vocab_size"], 256, 12, 1e-4, seed=4)
+
+
+@pytest.mark.slow
+def test_llama2_7b_shape_bf16_weights_prefill_512_decode():
+    """Config 5 shape (hidden 4096, 32-head MHA, head_dim 128, intermediate 11008, bf16-stored weights,
+    f32 accumulate and f32 KV cache) on 2 of the 32 layers; tolerance 2e-2 against the oracle run on the
+    same bf16 values widened to f32."""
+    cfg = dict(synth.LLAMA2_7B, num_hidden_layers=2)
+    cfg.pop("weight_dtype")
+    gpu, ora = _stream_build(cfg, seed=5, bf16=True)
+    _prefill_decode_check(gpu, ora, cfg["vocab_size"], 512, 8, 2e-2, seed=5)
