@@ -26,6 +26,49 @@ struct DecodeWaves {
     static constexpr int value = 8;
 };
 
+// Short contexts (up to ATTN_SHORT_ROWS cached rows, q already rotated): one query head per
+// workgroup over ALL rows, 8 row loads per lane in flight, so that nothing has to travel between
+// workgroups -- at these lengths the hand-over of partial results through memory (an atomic and
+// a round of agent-scope loads, each a trip to the memory side) costs more than reading the few
+// hundred K/V rows once per query head instead of once per KV head.
+#define ATTN_SHORT_ROWS 512
+template <int D, int WAVES>
+__device__ __forceinline__ void attn_decode_short(const AttnDecodeArgs &a, int hq, int hk, int bb, int pos, float *sm,
+                                                  float *sl, float *sacc) {
+    constexpr int LPR = D / 4, RPW = 64 / LPR, RPI = WAVES * RPW, UB = 8;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int off = wave * RPW + lane / LPR, c = lane % LPR;
+    const size_t head_base = ((size_t)bb * a.hkv + hk) * a.max_seq * D;
+    const float *Kb = a.k_cache + head_base + c * 4, *Vb = a.v_cache + head_base + c * 4;
+    AttnState<1> st;
+    state_init<1>(st);
+    v4f q[1];
+    bool have_q = false;
+    for (int base = 0; base < pos; base += RPI * UB) {
+        v4f kv[UB], vv[UB];
+#pragma unroll
+        for (int u = 0; u < UB; ++u) {  // rows past the end are clamped here and masked in attn_step
+            const int j = min(base + u * RPI + off, pos - 1);
+            kv[u] = *(const v4f *)(Kb + (size_t)j * D);
+            vv[u] = *(const v4f *)(Vb + (size_t)j * D);
+        }
+        if (!have_q) {
+            load_q_scaled<D, 1>(q, a.q + ((size_t)bb * a.hq + hq) * D, c, a.scale);
+            have_q = true;
+        }
+#pragma unroll
+        for (int u = 0; u < UB; ++u)
+            if (base + u * RPI < pos) attn_step<D, 1>(st, q, kv[u], vv[u], base + u * RPI + off < pos);
+    }
+    wave_merge_publish<D, 1>(st, sm, sl, sacc);
+    __syncthreads();
+    for (int dd = threadIdx.x; dd < D; dd += WAVES * 64) {
+        float mm, ls, cx;
+        wave_fold<D, 1, WAVES>(sm, sl, sacc, 0, dd, mm, ls, cx);
+        a.out[((size_t)bb * a.hq + hq) * D + dd] = cx * (1.0f / (ls + 1e-9f));  // self_attention.rs:287-290
+    }
+}
+
 // PRE: q arrives rotated and cache row `pos` is already written (both done by the q|k|v GEMV's
 // epilogue), so the kernel is only the row loop over [0, pos] and the merges.
 template <int D, int NREP, int WAVES, bool PRE>
@@ -44,6 +87,10 @@ __global__ __launch_bounds__(WAVES * 64) void attn_decode_kernel(AttnDecodeArgs 
     const int split = blockIdx.x, hk = blockIdx.y, bb = blockIdx.z;
     const int pos_new = a.pos_dev ? *a.pos_dev : a.pos_host;  // == past_len, the new token's position
     const int pos = PRE ? pos_new + 1 : pos_new;             // rows that come from the cache
+    if (PRE && pos <= ATTN_SHORT_ROWS && (int)gridDim.x >= NREP) {
+        if (split < NREP) attn_decode_short<D, WAVES>(a, hk * NREP + split, hk, bb, pos, sm, sl, sacc);
+        return;
+    }
     int nact, chunk;
     decode_slices<D, WAVES>(pos, gridDim.x, nact, chunk);
     if (split >= nact) return;

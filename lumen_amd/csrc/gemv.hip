@@ -55,19 +55,22 @@ __device__ __forceinline__ float dot16(const v4u raw, const float *xs) {
 }
 
 // Stages x (optionally RMS-normalised: (x * inv_rms) * g, src/layers/norm/rms_norm.rs:45-58)
-// into LDS, zero-padded to kpad.  All threads of the workgroup must call it.
+// into LDS, zero-padded to kpad.  x is read from memory once: the raw values go to LDS while the
+// sum of squares is taken, then every thread scales the elements it staged itself.  All threads
+// of the workgroup must call it.
 template <int PRO>
 __device__ __forceinline__ void stage_x(float *xs, const float *__restrict__ x, const float *__restrict__ g,
                                         float eps, int K, int kpad) {
     __shared__ float red[GEMV_WAVES];
     const int tid = threadIdx.x;
-    float inv = 1.0f;
+    float ss = 0.f;
+    for (int k = tid * 4; k < kpad; k += GEMV_THREADS * 4) {
+        v4f v = {0.f, 0.f, 0.f, 0.f};
+        if (k < K) v = *(const v4f *)(x + k);
+        ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+        *(v4f *)(xs + k) = v;
+    }
     if (PRO == PRO_RMSNORM) {
-        float ss = 0.f;
-        for (int k = tid * 4; k < K; k += GEMV_THREADS * 4) {
-            const v4f v = *(const v4f *)(x + k);
-            ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
-        }
         ss = wave_sum(ss);
         if ((tid & 63) == 0) red[tid >> 6] = ss;
         __syncthreads();
@@ -75,21 +78,16 @@ __device__ __forceinline__ void stage_x(float *xs, const float *__restrict__ x, 
 #pragma unroll
         for (int w = 0; w < GEMV_WAVES; ++w) tot += red[w];
         const float rms = sqrtf(tot / (float)K + eps);
-        inv = 1.0f / rms;
-    }
-    for (int k = tid * 4; k < kpad; k += GEMV_THREADS * 4) {
-        v4f v = {0.f, 0.f, 0.f, 0.f};
-        if (k < K) {
-            v = *(const v4f *)(x + k);
-            if (PRO == PRO_RMSNORM) {
-                const v4f gg = *(const v4f *)(g + k);
-                v.x = v.x * inv * gg.x;
-                v.y = v.y * inv * gg.y;
-                v.z = v.z * inv * gg.z;
-                v.w = v.w * inv * gg.w;
-            }
+        const float inv = 1.0f / rms;
+        for (int k = tid * 4; k < K; k += GEMV_THREADS * 4) {
+            v4f v = *(const v4f *)(xs + k);
+            const v4f gg = *(const v4f *)(g + k);
+            v.x = v.x * inv * gg.x;
+            v.y = v.y * inv * gg.y;
+            v.z = v.z * inv * gg.z;
+            v.w = v.w * inv * gg.w;
+            *(v4f *)(xs + k) = v;
         }
-        *(v4f *)(xs + k) = v;
     }
     __syncthreads();
 }
@@ -135,9 +133,29 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(GemvArgs a) {
         }
     };
 
+    // A wavefront's work is a sequence of pieces: np pieces per unit, units gw, gw + nw, ...  Two
+    // pieces (2 x 8 loads per lane) are kept in flight: while one is multiplied the next one is
+    // already on its way and the one after is requested as soon as its registers are free.
+    const int np = kpad / PIECE;
+    const int my_units = (nunits > gw) ? (nunits - gw + nw - 1) / nw : 0;
+    const int T = my_units * np;
+    int lu = gw, lk = 0;  // unit / element offset of the next piece to load
+    auto advance_load = [&]() {
+        lk += PIECE;
+        if (lk >= kpad) {
+            lk = 0;
+            lu += nw;
+        }
+    };
+
     // the first weights of this wavefront start streaming before x is staged: they do not depend on it
-    v4u raw[R][U];
-    load_piece(min(gw, nunits - 1), 0, raw);
+    v4u rawA[R][U], rawB[R][U];
+    load_piece(min(lu, nunits - 1), lk, rawA);
+    advance_load();
+    if (T > 1) {
+        load_piece(lu, lk, rawB);
+        advance_load();
+    }
 
     const long sel_off = a.row_sel ? (long)(*a.row_sel) * a.row_stride : 0;
     stage_x<PRO>(xs, a.x + (a.x_sel ? sel_off : 0), a.norm_w, a.eps, K, kpad);
@@ -145,69 +163,88 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(GemvArgs a) {
     float best = -INFINITY;
     int best_idx = 0x7fffffff;
 
-    for (int u = gw; u < nunits; u += nw) {
-        float acc[R];
+    float acc[R];
 #pragma unroll
-        for (int r = 0; r < R; ++r) acc[r] = 0.f;
-        for (int k0 = 0; k0 < K; k0 += PIECE) {
-            if (u != gw || k0 != 0) load_piece(u, k0, raw);
+    for (int r = 0; r < R; ++r) acc[r] = 0.f;
+    int u = gw, k0 = 0;  // unit / element offset of the piece being multiplied
+    auto consume = [&](const v4u (&raw)[R][U]) {
 #pragma unroll
-            for (int uu = 0; uu < U; ++uu) {
-                const float *xp = xs + k0 + uu * SWEEP + lane * VEC;
+        for (int uu = 0; uu < U; ++uu) {
+            const float *xp = xs + k0 + uu * SWEEP + lane * VEC;
 #pragma unroll
-                for (int r = 0; r < R; ++r) acc[r] += dot16<BF16>(raw[r][uu], xp);
-            }
+            for (int r = 0; r < R; ++r) acc[r] += dot16<BF16>(raw[r][uu], xp);
         }
+        k0 += PIECE;
+        if (k0 >= kpad) {  // unit complete
 #pragma unroll
-        for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
-        if (EPI == EPI_ARGMAX) {
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const int row = u * R + r;
-                if (row < N && (acc[r] > best || (acc[r] == best && row < best_idx))) {
-                    best = acc[r];
-                    best_idx = row;
-                }
-            }
-        }
-        if (lane == 0) {
-            if (EPI == EPI_SWIGLU) {
-                // rows (2u, 2u+1) hold (gate_u, up_u): silu(gate) * up, src/models/llama.rs:60-63
-                a.y[u] = silu_f(acc[0]) * acc[R - 1];
-            } else if (EPI == EPI_ROPE_QKV) {
-                // half-split rotation at the token's position (src/layers/attention/encoding.rs:196-203,
-                // self_attention.rs:220-227); k and v land in cache row pos (self_attention.rs:161-176)
-                const int head = u / half_d, j = u % half_d;
-                const int pos = *a.pos;
-                const float c = a.cos_t[(size_t)pos * a.D + j], sn = a.sin_t[(size_t)pos * a.D + j];
-                const float x1 = acc[0], x2 = acc[R - 1];
-                float o1, o2;
-                {
-#pragma clang fp contract(off)
-                    o1 = x1 * c - x2 * sn;
-                    o2 = x1 * sn + x2 * c;
-                }
-                if (head < a.hq) {
-                    a.y[head * a.D + j] = o1;
-                    a.y[head * a.D + j + half_d] = o2;
-                } else if (head < a.hq + a.hkv) {
-                    float *dst = a.k_cache + ((size_t)(head - a.hq) * a.max_seq + pos) * a.D;
-                    dst[j] = o1;
-                    dst[j + half_d] = o2;
-                } else {
-                    float *dst = a.v_cache + ((size_t)(head - a.hq - a.hkv) * a.max_seq + pos) * a.D;
-                    dst[j] = x1;
-                    dst[j + half_d] = x2;
-                }
-            } else {
+            for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
+            if (EPI == EPI_ARGMAX) {
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     const int row = u * R + r;
-                    if (row < N) {
-                        // residual: x + y, src/ops/arithmetic.rs:48-51 via src/models/llama.rs:110,115
-                        a.y[row] = (EPI == EPI_RESIDUAL) ? residual[row] + acc[r] : acc[r];
+                    if (row < N && (acc[r] > best || (acc[r] == best && row < best_idx))) {
+                        best = acc[r];
+                        best_idx = row;
                     }
                 }
+            }
+            if (lane == 0) {
+                if (EPI == EPI_SWIGLU) {
+                    // rows (2u, 2u+1) hold (gate_u, up_u): silu(gate) * up, src/models/llama.rs:60-63
+                    a.y[u] = silu_f(acc[0]) * acc[R - 1];
+                } else if (EPI == EPI_ROPE_QKV) {
+                    // half-split rotation at the token's position (src/layers/attention/encoding.rs:196-203,
+                    // self_attention.rs:220-227); k and v land in cache row pos (self_attention.rs:161-176)
+                    const int head = u / half_d, j = u % half_d;
+                    const int pos = *a.pos;
+                    const float c = a.cos_t[(size_t)pos * a.D + j], sn = a.sin_t[(size_t)pos * a.D + j];
+                    const float x1 = acc[0], x2 = acc[R - 1];
+                    float o1, o2;
+                    {
+#pragma clang fp contract(off)
+                        o1 = x1 * c - x2 * sn;
+                        o2 = x1 * sn + x2 * c;
+                    }
+                    if (head < a.hq) {
+                        a.y[head * a.D + j] = o1;
+                        a.y[head * a.D + j + half_d] = o2;
+                    } else if (head < a.hq + a.hkv) {
+                        float *dst = a.k_cache + ((size_t)(head - a.hq) * a.max_seq + pos) * a.D;
+                        dst[j] = o1;
+                        dst[j + half_d] = o2;
+                    } else {
+                        float *dst = a.v_cache + ((size_t)(head - a.hq - a.hkv) * a.max_seq + pos) * a.D;
+                        dst[j] = x1;
+                        dst[j + half_d] = x2;
+                    }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        const int row = u * R + r;
+                        if (row < N) {
+                            // residual: x + y, src/ops/arithmetic.rs:48-51 via src/models/llama.rs:110,115
+                            a.y[row] = (EPI == EPI_RESIDUAL) ? residual[row] + acc[r] : acc[r];
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc[r] = 0.f;
+            k0 = 0;
+            u += nw;
+        }
+    };
+    for (int t = 0; t < T; t += 2) {
+        consume(rawA);
+        if (t + 2 < T) {
+            load_piece(lu, lk, rawA);
+            advance_load();
+        }
+        if (t + 1 < T) {
+            consume(rawB);
+            if (t + 3 < T) {
+                load_piece(lu, lk, rawB);
+                advance_load();
             }
         }
     }
