@@ -47,6 +47,7 @@ extern "C" int lumen_ctx_destroy(lumen_ctx *ctx) {
     hipSetDevice(ctx->device);
     hipStreamSynchronize(ctx->stream);
     hipFree(ctx->d_scratch_int);
+    if (ctx->gemm_ws) hipFree(ctx->gemm_ws);
     hipEventDestroy(ctx->ev0);
     hipEventDestroy(ctx->ev1);
     hipStreamDestroy(ctx->own_stream);

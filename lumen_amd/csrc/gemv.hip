@@ -158,8 +158,25 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(GemvArgs a) {
     }
 
     const long sel_off = a.row_sel ? (long)(*a.row_sel) * a.row_stride : 0;
-    stage_x<PRO>(xs, a.x + (a.x_sel ? sel_off : 0), a.norm_w, a.eps, K, kpad);
     const float *residual = a.residual + (a.residual_sel ? sel_off : 0);
+    // What a unit's epilogue needs from memory is requested a unit ahead -- the first one here,
+    // before x is staged -- so that no load sits between the last multiply and the store:
+    // cos / sin of the unit's RoPE pair, or the residual of its rows.
+    const int pos = (EPI == EPI_ROPE_QKV) ? *a.pos : 0;
+    float pre0 = 0.f, pre1 = 0.f;
+    auto preload = [&](int un) {
+        if (EPI == EPI_ROPE_QKV && un < nunits) {
+            const int j = un % half_d;
+            pre0 = a.cos_t[(size_t)pos * a.D + j];
+            pre1 = a.sin_t[(size_t)pos * a.D + j];
+        }
+        if (EPI == EPI_RESIDUAL) {
+            if (un * R < N) pre0 = residual[un * R];
+            if (R == 2 && un * R + 1 < N) pre1 = residual[un * R + 1];
+        }
+    };
+    preload(gw);
+    stage_x<PRO>(xs, a.x + (a.x_sel ? sel_off : 0), a.norm_w, a.eps, K, kpad);
     float best = -INFINITY;
     int best_idx = 0x7fffffff;
 
@@ -196,8 +213,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(GemvArgs a) {
                     // half-split rotation at the token's position (src/layers/attention/encoding.rs:196-203,
                     // self_attention.rs:220-227); k and v land in cache row pos (self_attention.rs:161-176)
                     const int head = u / half_d, j = u % half_d;
-                    const int pos = *a.pos;
-                    const float c = a.cos_t[(size_t)pos * a.D + j], sn = a.sin_t[(size_t)pos * a.D + j];
+                    const float c = pre0, sn = pre1;
                     const float x1 = acc[0], x2 = acc[R - 1];
                     float o1, o2;
                     {
@@ -223,7 +239,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(GemvArgs a) {
                         const int row = u * R + r;
                         if (row < N) {
                             // residual: x + y, src/ops/arithmetic.rs:48-51 via src/models/llama.rs:110,115
-                            a.y[row] = (EPI == EPI_RESIDUAL) ? residual[row] + acc[r] : acc[r];
+                            a.y[row] = (EPI == EPI_RESIDUAL) ? (r == 0 ? pre0 : pre1) + acc[r] : acc[r];
                         }
                     }
                 }
@@ -232,6 +248,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(GemvArgs a) {
             for (int r = 0; r < R; ++r) acc[r] = 0.f;
             k0 = 0;
             u += nw;
+            preload(u);
         }
     };
     for (int t = 0; t < T; t += 2) {

@@ -44,6 +44,8 @@ struct lumen_ctx {
     hipStream_t stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     int *d_scratch_int = nullptr;  // small device scratch (argmax result etc.)
+    float *gemm_ws = nullptr;      // split-K workspace of the prefill GEMM, grown on demand
+    size_t gemm_ws_bytes = 0;
 };
 
 struct lumen_rope {
@@ -111,6 +113,7 @@ struct GemmArgs {
     int w_bf16;
     int epi;
     const float *residual;  // [M, N]
+    float *part;            // split-K partial tiles [splits, M, N] (set by the launcher)
 };
 int launch_gemm(lumen_ctx *ctx, const GemmArgs &a);
 
