@@ -23,6 +23,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+MFMA_FP32_PEAK_TF = 157.3  # MI355X dense fp32 matrix peak, TFLOP/s
 
 
 def main():
@@ -71,11 +72,16 @@ def main():
     prompt = synth.make_tokens(args.prompt, cfg["vocab_size"], seed=0)
     t_setup = time.time() - t0
 
-    # prefill (untimed here; reported separately)
+    # prefill (outside the timed decode region; reported separately).  The first pass sizes the
+    # prompt buffers and the GEMM workspace; the second, from a reset cache, is the one timed.
     ctx = model.ctx
-    ctx.timer_start()
-    last = model.forward(prompt, all_rows=False)
-    prefill_ms = ctx.timer_stop()
+    prefill_all_ms = []
+    for _ in range(3):  # the third pass is the steady one (the first two still see allocator / loader warm-up)
+        model.reset_kv_caches()
+        ctx.timer_start()
+        last = model.forward(prompt, all_rows=False)
+        prefill_all_ms.append(ctx.timer_stop())
+    prefill_ms = prefill_all_ms[-1]
     first = int(np.argmax(last))
 
     # warmup, then EXACTLY --steps decoded tokens between two events on the library's stream
@@ -123,13 +129,28 @@ def main():
                           "frac_of_8TBps": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                           "roofline_tokens_per_s": round(HBM_PEAK_GBS * 1e9 / step_bytes, 1)},
         "kernels": kernels,
-        "prefill": {"tokens": args.prompt, "ms": round(prefill_ms, 3), "tokens_per_s": round(args.prompt / prefill_ms * 1e3, 1)},
+        "prefill": dict(prefill_report(cfg, args.prompt, prefill_ms), passes_ms=[round(x, 3) for x in prefill_all_ms]),
         "decode_mode": args.mode, "wall_s_timed_region": round(wall, 4), "setup_s": round(t_setup, 1),
     }
 
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, params, prompt, args.cpu_tokens)
     print(json.dumps(out))
+
+
+def prefill_report(cfg, S, ms):
+    """Prompt pass: tokens/s and the share of the fp32 matrix-core peak its GEMM flops amount to
+    (all projections on S rows, lm_head on the last row only, causal attention counted once)."""
+    H, I, V, L = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"], cfg["num_hidden_layers"]
+    hq, hkv = cfg["num_attention_heads"], cfg["num_key_value_heads"]
+    D = cfg.get("head_dim") or H // hq
+    per_layer = hq * D * H + 2 * hkv * D * H + H * hq * D + 3 * H * I
+    gemm_flops = 2.0 * S * L * per_layer + 2.0 * V * H
+    attn_flops = 4.0 * L * hq * D * S * S / 2.0
+    tf = (gemm_flops + attn_flops) / (ms * 1e-3) / 1e12
+    return {"tokens": S, "ms": round(ms, 3), "tokens_per_s": round(S / ms * 1e3, 1),
+            "gemm_flops": gemm_flops, "attention_flops": attn_flops, "achieved_TFLOPs": round(tf, 2),
+            "mfma_fp32_peak_TFLOPs": MFMA_FP32_PEAK_TF, "frac_of_mfma_fp32_peak": round(tf / MFMA_FP32_PEAK_TF, 4)}
 
 
 def measured_traffic():
