@@ -306,6 +306,7 @@ template <int D>
 static int launch_prefill_d(lumen_ctx *ctx, const AttnPrefillArgs &a) {
     hipLaunchKernelGGL(prefill_rope_kernel<D>, dim3(a.s, a.b), dim3(ATT_THREADS), 0, ctx->stream, a);
     LUMEN_CHECK_LAUNCH();
+    if (attn_prefill_mfma_supported(a)) return launch_attn_prefill_mfma(ctx, a);  // head_dim 64 / 128: matrix cores
     dim3 grid(a.s, a.hkv, a.b), block(ATT_THREADS);
     const int nrep = a.hq / a.hkv;
     switch (nrep) {

@@ -167,6 +167,9 @@ struct AttnPrefillArgs {
     float *q_rot;    // scratch [B, S, Hq, D]
 };
 int launch_attn_prefill(lumen_ctx *ctx, const AttnPrefillArgs &a);
+// the scores / softmax / context part on the matrix cores (q_rot and the cache rows already written)
+bool attn_prefill_mfma_supported(const AttnPrefillArgs &a);
+int launch_attn_prefill_mfma(lumen_ctx *ctx, const AttnPrefillArgs &a);
 
 int attn_decode_nsplit(int max_seq);
 size_t attn_decode_part_floats(int b, int hq, int d, int nsplit);

@@ -1,0 +1,205 @@
+// Causal GQA attention for a prompt (S > 1) on the matrix cores:
+// self_attention.rs:308-419 with gqa_attention_no_repeat_bshd_view (:519-641)
+// and softmax_inplace_view (:643-678) -- scores = Q K^T * scale, mask
+// j > past_len + i, softmax with divisor (sum + 1e-9), ctx = P V, output BSHD.
+//
+// The reference materialises the S x L score matrix per head; here a
+// workgroup keeps 128 (position, query head) rows of one KV group in
+// registers and walks the cached keys in tiles of 32 with an online softmax,
+// so scores never leave the compute unit and every K/V tile read from the
+// cache serves all n_rep heads of the group and 128 / n_rep positions at once.
+//
+// Per wavefront (32 rows) and key tile:
+//   S  = Q K^T        D/2 v_mfma_f32_32x32x2_f32, Q fragments in registers, K from LDS
+//   row max           across the 32 lanes that hold a row's 32 keys (DPP + one shuffle)
+//   P  = exp2(S - m)  scores are kept in log2 units (Q is pre-multiplied by scale * log2 e);
+//                     the row sums stay per lane and are folded across lanes once at the end
+//   O  = alpha O + P V   P goes through a per-wavefront LDS patch to become an A operand
+// fp32 operands and accumulation throughout.
+#include "internal.h"
+#include "attn_device.h"
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+#define FA_ROWS 128  // (position, head) rows per workgroup
+#define FA_KEYS 32   // keys per tile
+#define FA_THREADS 256
+
+// max over the 32 lanes of a half-wavefront; every lane gets the result
+__device__ __forceinline__ float half_max(float v) {
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false)));  // row_ror:8
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xf, 0xf, false)));  // row_ror:4
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xf, 0xf, false)));  // row_ror:2
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xf, 0xf, false)));  // row_ror:1
+    return fmaxf(v, __shfl_xor(v, 16, 64));
+}
+
+__device__ __forceinline__ float half_sum(float v) {
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false));
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xf, 0xf, false));
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xf, 0xf, false));
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xf, 0xf, false));
+    return v + __shfl_xor(v, 16, 64);
+}
+
+// q_rot [B,S,Hq,D] rotated queries; K (rotated) and V already in the cache up to past_len + S.
+template <int D, int NREP>
+__global__ __launch_bounds__(FA_THREADS) void attn_prefill_mfma_kernel(AttnPrefillArgs a) {
+    constexpr int BQ = FA_ROWS / NREP;       // positions per workgroup
+    constexpr int DT = D / 32;               // 32-wide output tiles per row
+    constexpr int PIECES = D * FA_KEYS / 4 / FA_THREADS;  // 16-byte pieces of a K (or V) tile per thread
+    constexpr int LDK = D + 1;
+    __shared__ float Ks[FA_KEYS][LDK];
+    __shared__ __align__(16) float Vs[FA_KEYS][D];
+    __shared__ float Ps[FA_THREADS / 64][32][33];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int c = lane & 31, half = lane >> 5;
+    // workgroups are dealt in index order: the blocks of late positions (most keys) go first
+    const int q0 = (int)(gridDim.x - 1 - blockIdx.x) * BQ, hk = blockIdx.y, bb = blockIdx.z;
+    const int L = a.past_len + a.s;
+    const size_t head_base = ((size_t)bb * a.hkv + hk) * a.max_seq * D;
+    const float *Kc = a.k_cache + head_base, *Vc = a.v_cache + head_base;
+
+    // accumulator register r of lane l belongs to row 8*(r/4) + 4*(l/32) + r%4 of the wavefront's 32
+    auto row_of = [&](int r) { return 8 * (r >> 2) + 4 * half + (r & 3); };
+
+    // Q fragments: lane l feeds row l%32, element 2*kk + l/32 of the dot product
+    const int my_row = wave * 32 + c;                 // row this lane feeds as an A operand
+    const int my_i = min(q0 + my_row / NREP, a.s - 1);  // clamped: rows past S are computed and dropped
+    const float *qrow = a.q_rot + (((size_t)bb * a.s + my_i) * a.hq + (size_t)hk * NREP + my_row % NREP) * D;
+    const float qf_scale = a.scale * LUMEN_LOG2E;
+    float qf[D / 2];
+#pragma unroll
+    for (int kk = 0; kk < D / 2; ++kk) qf[kk] = qrow[2 * kk + half] * qf_scale;
+
+    // keys this workgroup needs: up to the last position's own key
+    const int q_last = min(q0 + BQ, a.s) - 1;
+    const int kmax = a.causal ? min(L, a.past_len + q_last + 1) : L;
+    // last key the rows of this wavefront may see (uniform per wavefront)
+    const int wave_i_last = min(q0 + (wave * 32 + 31) / NREP, a.s - 1);
+    const int wave_kmax = a.causal ? min(L, a.past_len + wave_i_last + 1) : L;
+
+    v16f O[DT];
+    float m_run[16], l_run[16];
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) O[t][r] = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        m_run[r] = -INFINITY;
+        l_run[r] = 0.f;
+    }
+    // position (absolute) of the row behind each accumulator register
+    int pos_r[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) pos_r[r] = a.past_len + q0 + (wave * 32 + row_of(r)) / NREP;
+
+    v4f kreg[PIECES], vreg[PIECES];
+    auto fetch = [&](int j0) {
+#pragma unroll
+        for (int p = 0; p < PIECES; ++p) {
+            const int idx = tid + p * FA_THREADS;
+            const int key = idx / (D / 4), k4 = (idx % (D / 4)) * 4;
+            const int j = min(j0 + key, L - 1);  // keys past L are masked below
+            kreg[p] = *(const v4f *)(Kc + (size_t)j * D + k4);
+            vreg[p] = *(const v4f *)(Vc + (size_t)j * D + k4);
+        }
+    };
+
+    if (kmax > 0) fetch(0);
+    for (int j0 = 0; j0 < kmax; j0 += FA_KEYS) {
+#pragma unroll
+        for (int p = 0; p < PIECES; ++p) {
+            const int idx = tid + p * FA_THREADS;
+            const int key = idx / (D / 4), k4 = (idx % (D / 4)) * 4;
+            Ks[key][k4 + 0] = kreg[p].x; Ks[key][k4 + 1] = kreg[p].y; Ks[key][k4 + 2] = kreg[p].z; Ks[key][k4 + 3] = kreg[p].w;
+            *(v4f *)&Vs[key][k4] = vreg[p];
+        }
+        __syncthreads();
+        if (j0 + FA_KEYS < kmax) fetch(j0 + FA_KEYS);  // in flight during the matrix instructions below
+
+        if (j0 < wave_kmax) {  // uniform per wavefront: tiles wholly above the causal diagonal are skipped
+            v16f S;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) S[r] = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < D / 2; ++kk)
+                S = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[kk], Ks[c][2 * kk + half], S, 0, 0, 0);
+
+            const int j = j0 + c;  // this lane's key
+            float alpha[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const bool valid = j < L && (!a.causal || j <= pos_r[r]);
+                const float s = valid ? S[r] : -INFINITY;
+                const float m_new = fmaxf(m_run[r], half_max(s));
+                float p = 0.f;
+                alpha[r] = 1.0f;
+                if (m_new > -INFINITY) {
+                    alpha[r] = fast_exp2(m_run[r] - m_new);  // exp2(-inf) = 0 on the row's first live tile
+                    p = fast_exp2(s - m_new);
+                }
+                l_run[r] = fmaf(l_run[r], alpha[r], p);
+                m_run[r] = m_new;
+                Ps[wave][row_of(r)][c] = p;
+            }
+#pragma unroll
+            for (int t = 0; t < DT; ++t)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) O[t][r] *= alpha[r];
+            __builtin_amdgcn_wave_barrier();  // P: written above by this wavefront, read below in another lane order
+#pragma unroll
+            for (int kk = 0; kk < FA_KEYS / 2; ++kk) {
+                const float pf = Ps[wave][c][2 * kk + half];
+#pragma unroll
+                for (int t = 0; t < DT; ++t)
+                    O[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(pf, Vs[2 * kk + half][32 * t + c], O[t], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+
+    // out = ctx / (sum + 1e-9), self_attention.rs:670-676; [B,S,Hq,D]
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const float inv = 1.0f / (half_sum(l_run[r]) + 1e-9f);
+        const int row = wave * 32 + row_of(r);
+        const int i = q0 + row / NREP;
+        if (i < a.s) {
+            float *o = a.out + (((size_t)bb * a.s + i) * a.hq + (size_t)hk * NREP + row % NREP) * D;
+#pragma unroll
+            for (int t = 0; t < DT; ++t) o[32 * t + c] = O[t][r] * inv;
+        }
+    }
+}
+
+template <int D>
+static int launch_fa_d(lumen_ctx *ctx, const AttnPrefillArgs &a) {
+    const int nrep = a.hq / a.hkv;
+    dim3 block(FA_THREADS);
+#define LAUNCH_FA(NR)                                                                                  \
+    hipLaunchKernelGGL((attn_prefill_mfma_kernel<D, NR>), dim3((a.s + FA_ROWS / NR - 1) / (FA_ROWS / NR), a.hkv, a.b), \
+                       block, 0, ctx->stream, a)
+    switch (nrep) {
+        case 1: LAUNCH_FA(1); break;
+        case 2: LAUNCH_FA(2); break;
+        case 4: LAUNCH_FA(4); break;
+        case 8: LAUNCH_FA(8); break;
+        default: LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "prefill attention: n_rep=%d (supported 1, 2, 4, 8)", nrep);
+    }
+#undef LAUNCH_FA
+    LUMEN_CHECK_LAUNCH();
+    return LUMEN_OK;
+}
+
+// Worth it from a few hundred positions on: below that the tile loop of the few workgroups is
+// longer than the row loop of one workgroup per position.
+bool attn_prefill_mfma_supported(const AttnPrefillArgs &a) { return (a.d == 64 || a.d == 128) && a.s >= 192; }
+
+int launch_attn_prefill_mfma(lumen_ctx *ctx, const AttnPrefillArgs &a) {
+    if (a.d == 64) return launch_fa_d<64>(ctx, a);
+    if (a.d == 128) return launch_fa_d<128>(ctx, a);
+    LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "matrix-core prefill attention: head_dim=%d (supported 64, 128)", a.d);
+}

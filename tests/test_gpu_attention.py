@@ -113,7 +113,11 @@ def test_cache_state_machine_overflow_and_reset():
     assert np.array_equal(a, b)  # stale rows beyond len are never read
 
 
-@pytest.mark.parametrize("h,h_kv,d,s,past", [(32, 4, 64, 128, 0), (16, 8, 128, 50, 17), (4, 4, 32, 3, 9), (8, 2, 16, 33, 31)])
+# prompts of 192 positions and more with head_dim 64 / 128 take the matrix-core kernel (n_rep 8, 2, 1, 4 here;
+# lengths that are no multiple of the tile sizes, with and without rows already in the cache)
+@pytest.mark.parametrize("h,h_kv,d,s,past", [(32, 4, 64, 128, 0), (16, 8, 128, 50, 17), (4, 4, 32, 3, 9), (8, 2, 16, 33, 31),
+                                             (16, 2, 64, 331, 0), (8, 4, 128, 200, 45), (4, 4, 64, 193, 230),
+                                             (8, 2, 64, 257, 63)])
 def test_prefill_with_and_without_past(h, h_kv, d, s, past):
     max_seq = past + s + 3
     scale = 1.0 / math.sqrt(d)
