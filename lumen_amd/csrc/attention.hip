@@ -88,7 +88,12 @@ __global__ __launch_bounds__(WAVES * 64) void attn_decode_kernel(AttnDecodeArgs 
     const int pos_new = a.pos_dev ? *a.pos_dev : a.pos_host;  // == past_len, the new token's position
     const int pos = PRE ? pos_new + 1 : pos_new;             // rows that come from the cache
     if (PRE && pos <= ATTN_SHORT_ROWS && (int)gridDim.x >= NREP) {
-        if (split < NREP) attn_decode_short<D, WAVES>(a, hk * NREP + split, hk, bb, pos, sm, sl, sacc);
+        // Workgroups are dealt round-robin over the 8 XCDs, each with an L2 of its own.  With 32 or
+        // more workgroups per KV head the heads of a group are placed 8 apart, four to an XCD, so
+        // that a group's K/V rows are fetched into two L2s instead of eight.
+        int r = split;
+        if (NREP == 8 && gridDim.x >= 32 && (gridDim.x & 7) == 0) r = (split & 7) < 2 && split < 32 ? (split >> 3) + 4 * (split & 7) : NREP;
+        if (r < NREP) attn_decode_short<D, WAVES>(a, hk * NREP + r, hk, bb, pos, sm, sl, sacc);
         return;
     }
     int nact, chunk;
