@@ -190,6 +190,17 @@ int lumen_llama_destroy(lumen_llama *model);
  * match -> LUMEN_ERR_SHAPE; unknown name -> LUMEN_ERR_INVALID. */
 int lumen_llama_set_param(lumen_llama *model, const char *name, const void *data_host,
                           int dtype, const int64_t *shape, int ndim);
+/* ModelLoader::load_llama_weights, src/loader.rs:10-80: maps a .safetensors file and
+ * sets every parameter of the model that the file holds (F32 or BF16, :32-66);
+ * a parameter the file lacks is counted in *n_missing_out and left as it is (the
+ * reference's warning, :69-74); another dtype -> LUMEN_ERR_INVALID (:67); an element
+ * count that differs from the parameter's -> LUMEN_ERR_SHAPE (:44-46).  Counters may be NULL. */
+int lumen_llama_load_safetensors(lumen_llama *model, const char *path, int *n_loaded_out, int *n_missing_out);
+/* the header lookup behind it (SafeTensors::deserialize + tensor(name), loader.rs:18, :24), host only:
+ * dtype (LUMEN_DTYPE_* or -1 for any other), shape (ndim_inout: room in, dimensions out) and the
+ * byte range of one tensor relative to the end of the header; not in the file -> LUMEN_ERR_INVALID. */
+int lumen_safetensors_find(const char *path, const char *name, int *dtype_out, int64_t *shape_out,
+                           int *ndim_inout, uint64_t *begin_out, uint64_t *end_out);
 /* LlamaModel::forward, llama.rs:181-206: ids_host [S] as f32 (main.rs:143-152);
  * S == 1 takes the decode path, S > 1 prefill (appending to the live cache).
  * logits_host receives [S, V] when all_rows != 0 (what the reference computes)

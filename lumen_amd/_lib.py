@@ -83,6 +83,9 @@ SIGNATURES = {
     "lumen_llama_create": (_i, [_vp, C.POINTER(LlamaConfigStruct), _pp]),
     "lumen_llama_destroy": (_i, [_vp]),
     "lumen_llama_set_param": (_i, [_vp, C.c_char_p, _vp, _i, C.POINTER(C.c_int64), _i]),
+    "lumen_llama_load_safetensors": (_i, [_vp, C.c_char_p, C.POINTER(_i), C.POINTER(_i)]),
+    "lumen_safetensors_find": (_i, [C.c_char_p, C.c_char_p, C.POINTER(_i), C.POINTER(C.c_int64), C.POINTER(_i),
+                                    C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "lumen_llama_forward": (_i, [_vp, _vp, _i, _vp, _i]),
     "lumen_llama_decode_greedy": (_i, [_vp, _i, _i, _vp, _vp]),
     "lumen_llama_decode_profile": (_i, [_vp, _i, _i, C.POINTER(C.c_double), C.POINTER(_i), _i]),

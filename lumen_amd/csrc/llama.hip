@@ -343,6 +343,39 @@ extern "C" int lumen_llama_set_param(lumen_llama *m, const char *name, const voi
     LUMEN_FAIL(LUMEN_ERR_INVALID, "Parameter %s not found in model", name);
 }
 
+// Names and shapes of the model's parameters, LlamaModel::named_parameters (llama.rs:218-279),
+// plus the per-head q/k norm gains of the Qwen3 extension; no lm_head when it is tied.
+int lumen_llama_param_list(const lumen_llama *m, std::vector<std::string> &names,
+                           std::vector<std::vector<int64_t>> &shapes) {
+    if (!m) LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_param_list: null model");
+    const lumen_llama_config &c = m->cfg;
+    const int64_t H = c.hidden_size, I = c.intermediate_size, V = c.vocab_size;
+    auto add = [&](const std::string &n, std::vector<int64_t> sh) {
+        names.push_back(n);
+        shapes.push_back(sh);
+    };
+    add("model.embed_tokens.weight", {V, H});
+    for (int l = 0; l < c.num_hidden_layers; ++l) {
+        const std::string p = "model.layers." + std::to_string(l) + ".";
+        add(p + "self_attn.q_proj.weight", {m->qd, H});
+        add(p + "self_attn.k_proj.weight", {m->kvd, H});
+        add(p + "self_attn.v_proj.weight", {m->kvd, H});
+        add(p + "self_attn.o_proj.weight", {H, m->qd});
+        add(p + "mlp.gate_proj.weight", {I, H});
+        add(p + "mlp.up_proj.weight", {I, H});
+        add(p + "mlp.down_proj.weight", {H, I});
+        add(p + "input_layernorm.weight", {H});
+        add(p + "post_attention_layernorm.weight", {H});
+        if (c.qk_norm) {
+            add(p + "self_attn.q_norm.weight", {m->D});
+            add(p + "self_attn.k_norm.weight", {m->D});
+        }
+    }
+    add("model.norm.weight", {H});
+    if (!c.tie_embeddings) add("lm_head.weight", {V, H});
+    return LUMEN_OK;
+}
+
 // ------------------------------------------------------------------- decode
 // One token through all layers; every launch reads the token id and the
 // position from device memory, so the sequence is the same for every token.

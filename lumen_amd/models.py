@@ -75,6 +75,12 @@ class LlamaModel:
         shape = (C.c_int64 * a.ndim)(*a.shape)
         check(lib.lumen_llama_set_param(self.handle, name.encode(), a.ctypes.data, dtype, shape, a.ndim))
 
+    def load_safetensors(self, path):
+        """ModelLoader::load_llama_weights (loader.rs:10-80): returns (tensors set, parameters the file lacks)."""
+        loaded, missing = C.c_int(), C.c_int()
+        check(lib.lumen_llama_load_safetensors(self.handle, str(path).encode(), C.byref(loaded), C.byref(missing)))
+        return loaded.value, missing.value
+
     def load_params(self, named):
         for name, a in (named.items() if hasattr(named, "items") else named):
             self.set_param(name, a)
