@@ -211,6 +211,30 @@ int lumen_llama_forward(lumen_llama *model, const float *ids_host, int s, float 
  * ids_out_host [n] receives the picks; logits_out_host [n, V] is optional. */
 int lumen_llama_decode_greedy(lumen_llama *model, int first_id, int n, int32_t *ids_out_host,
                               float *logits_out_host);
+/* sample_top_p, src/main.rs:74-137 (host code there and here): repetition penalty over the
+ * recent tokens, temperature, softmax, nucleus of mass top_p, inverse-CDF pick.  The uniform
+ * draw r in [0,1) is an argument; the reference takes it from an unseeded generator (:69-72). */
+int lumen_sample_top_p_f32(const float *logits_host, int n, float temperature, float top_p,
+                           float repetition_penalty, const int32_t *recent_tokens, int n_recent,
+                           float r, int32_t *index_out);
+/* the seeded stand-in for rand01 (main.rs:69-72): splitmix64, 24 random bits -> [0,1) */
+float lumen_rand01(uint64_t *state);
+typedef struct lumen_sampling {
+    float temperature, top_p, repetition_penalty; /* main.rs:223-225: 0.8, 0.9, 1.05 there */
+    int recent_window;                            /* tokens the penalty looks back over, :226 (96) */
+    int max_gen;                                  /* tokens per turn at most, :227 (200) */
+    uint64_t seed;                                /* start of the lumen_rand01 stream of this turn */
+} lumen_sampling;
+/* one turn of the chat loop, src/main.rs:325-378, without the tokenizer: prefill the turn's new
+ * tokens into the live cache, then sample / feed back until a stop id, max_gen, out_cap or the end
+ * of the cache (len + 2 >= max_seq).  history = tokens already in the cache (the penalty window
+ * reaches into them).  len + n_new + 8 >= max_seq -> LUMEN_ERR_KV_OVERFLOW: the caller resets and
+ * starts a first turn, as the reference does at :266-270.  Stops on generated text (:364-366)
+ * need the tokenizer and stay with the caller. */
+int lumen_llama_generate_turn(lumen_llama *model, const int32_t *new_tokens, int n_new,
+                              const int32_t *history, int n_history, const lumen_sampling *sampling,
+                              const int32_t *stop_ids, int n_stop, int32_t *out_ids, int out_cap, int *n_out);
+int lumen_llama_get_config(const lumen_llama *model, lumen_llama_config *cfg_out);
 /* measurement aid (no reference counterpart): n greedy steps launched kernel by
  * kernel, every launch bracketed by HIP events on the ctx stream.  Classes:
  * 0 embedding, 1 norm+q|k|v GEMV, 2 decode attention, 3 o_proj GEMV, 4 norm+gate|up

@@ -27,6 +27,11 @@ class LumenError(RuntimeError):
         self.status = status
 
 
+class SamplingStruct(C.Structure):  # lumen_sampling
+    _fields_ = [("temperature", C.c_float), ("top_p", C.c_float), ("repetition_penalty", C.c_float),
+                ("recent_window", C.c_int), ("max_gen", C.c_int), ("seed", C.c_uint64)]
+
+
 class LlamaConfigStruct(C.Structure):
     _fields_ = [("vocab_size", C.c_int), ("hidden_size", C.c_int), ("intermediate_size", C.c_int),
                 ("num_hidden_layers", C.c_int), ("num_attention_heads", C.c_int),
@@ -84,6 +89,10 @@ SIGNATURES = {
     "lumen_llama_destroy": (_i, [_vp]),
     "lumen_llama_set_param": (_i, [_vp, C.c_char_p, _vp, _i, C.POINTER(C.c_int64), _i]),
     "lumen_llama_load_safetensors": (_i, [_vp, C.c_char_p, C.POINTER(_i), C.POINTER(_i)]),
+    "lumen_sample_top_p_f32": (_i, [_vp, _i, _f, _f, _f, _vp, _i, _f, C.POINTER(C.c_int32)]),
+    "lumen_rand01": (_f, [C.POINTER(C.c_uint64)]),
+    "lumen_llama_generate_turn": (_i, [_vp, _vp, _i, _vp, _i, _vp, _vp, _i, _vp, _i, C.POINTER(_i)]),
+    "lumen_llama_get_config": (_i, [_vp, _vp]),
     "lumen_safetensors_find": (_i, [C.c_char_p, C.c_char_p, C.POINTER(_i), C.POINTER(C.c_int64), C.POINTER(_i),
                                     C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "lumen_llama_forward": (_i, [_vp, _vp, _i, _vp, _i]),

@@ -791,6 +791,12 @@ extern "C" int lumen_llama_reset(lumen_llama *m) {
     return sync_pos_to_device(m);
 }
 
+extern "C" int lumen_llama_get_config(const lumen_llama *m, lumen_llama_config *cfg_out) {
+    if (!m || !cfg_out) LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_get_config: null argument");
+    *cfg_out = m->cfg;
+    return LUMEN_OK;
+}
+
 extern "C" int lumen_llama_kv_len(const lumen_llama *m, int *len_out) {
     if (!m || !len_out) LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_kv_len: null argument");
     *len_out = m->len;

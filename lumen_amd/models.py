@@ -81,6 +81,21 @@ class LlamaModel:
         check(lib.lumen_llama_load_safetensors(self.handle, str(path).encode(), C.byref(loaded), C.byref(missing)))
         return loaded.value, missing.value
 
+    def generate_turn(self, new_tokens, history=(), temperature=0.8, top_p=0.9, repetition_penalty=1.05,
+                      recent_window=96, max_gen=200, seed=0, stop_ids=()):
+        """One turn of the chat loop (main.rs:325-378; defaults = its parameters, :223-227): prefill
+        new_tokens, then sample until a stop id / max_gen / the end of the cache.  Returns the new ids."""
+        new = np.ascontiguousarray(new_tokens, np.int32)
+        hist = np.ascontiguousarray(history, np.int32)
+        stops = np.ascontiguousarray(stop_ids, np.int32)
+        sp = _lib.SamplingStruct(temperature, top_p, repetition_penalty, recent_window, max_gen, seed)
+        out = np.zeros(max(max_gen, 1), np.int32)
+        n = C.c_int()
+        check(lib.lumen_llama_generate_turn(self.handle, new.ctypes.data, new.size, hist.ctypes.data, hist.size,
+                                            C.byref(sp), stops.ctypes.data, stops.size, out.ctypes.data, out.size,
+                                            C.byref(n)))
+        return out[:n.value].copy()
+
     def load_params(self, named):
         for name, a in (named.items() if hasattr(named, "items") else named):
             self.set_param(name, a)

@@ -1,4 +1,6 @@
 """Operator functions of the reference's src/ops on the GPU."""
+import ctypes as C
+
 import numpy as np
 
 from ._lib import ERR_SHAPE, LumenError, check, lib
@@ -67,3 +69,19 @@ def argmax(t):
     idx = C.c_int()
     check(lib.lumen_argmax_f32(t.ctx.handle, t.ptr, t.size, C.byref(idx)))
     return idx.value
+
+
+def sample_top_p(logits, temperature, top_p, repetition_penalty, recent_tokens, r):
+    """sample_top_p, src/main.rs:74-137, on host logits with the uniform draw r given."""
+    x = np.ascontiguousarray(logits, np.float32)
+    rec = np.ascontiguousarray(recent_tokens, np.int32)
+    out = C.c_int32()
+    check(lib.lumen_sample_top_p_f32(x.ctypes.data, x.size, float(temperature), float(top_p), float(repetition_penalty),
+                                     rec.ctypes.data, rec.size, float(r), C.byref(out)))
+    return out.value
+
+
+def rand01_stream(seed, n):
+    """The first n draws of the seeded generator behind lumen_llama_generate_turn."""
+    state = C.c_uint64(seed)
+    return np.array([lib.lumen_rand01(C.byref(state)) for _ in range(n)], np.float32)

@@ -221,6 +221,77 @@ int lo_argmax_f32(const float *x, int n) {
     return best;
 }
 
+/* sample_top_p, src/main.rs:74-137, with the uniform draw r passed in (the
+ * reference takes it from an unseeded generator, :69-72).  Steps as written
+ * there: logits of the recent tokens divided by the penalty (also negative
+ * ones, :84-89), division by max(temperature, 1e-5), softmax with divisor
+ * (sum + 1e-9) in f32 (:100-110), indices sorted by probability descending --
+ * a stable sort, equal probabilities stay in index order (:113-114) --
+ * nucleus = shortest prefix whose running f32 sum reaches
+ * clamp(top_p, 0, 1).max(1e-6) (:116-126), then the first index whose running
+ * sum of p / cumulative reaches r, else the nucleus' last (:129-137).
+ * Returns -1 when n <= 0. */
+int lo_sample_top_p(const float *logits, int n, float temperature, float top_p, float repetition_penalty,
+                    const int *recent, int n_recent, float r) {
+    if (n <= 0) return -1;
+    float *adj = (float *)malloc(sizeof(float) * (size_t)n);
+    int *idx = (int *)malloc(sizeof(int) * (size_t)n);
+    int *tmp = (int *)malloc(sizeof(int) * (size_t)n);
+    memcpy(adj, logits, sizeof(float) * (size_t)n);
+    if (repetition_penalty > 1.0f)
+        for (int i = 0; i < n_recent; ++i)
+            if (recent[i] >= 0 && recent[i] < n) adj[recent[i]] /= repetition_penalty;
+    const float temp = temperature > 1e-5f ? temperature : 1e-5f;
+    for (int i = 0; i < n; ++i) adj[i] /= temp;
+    float maxv = -INFINITY;
+    for (int i = 0; i < n; ++i)
+        if (adj[i] > maxv) maxv = adj[i];
+    float sum = 0.f;
+    for (int i = 0; i < n; ++i) {
+        adj[i] = expf(adj[i] - maxv);
+        sum += adj[i];
+    }
+    const float inv = 1.0f / (sum + 1e-9f);
+    for (int i = 0; i < n; ++i) adj[i] *= inv;
+    /* bottom-up merge sort, descending by probability, stable */
+    for (int i = 0; i < n; ++i) idx[i] = i;
+    for (int w = 1; w < n; w *= 2) {
+        for (int lo = 0; lo < n; lo += 2 * w) {
+            int mid = lo + w < n ? lo + w : n, hi = lo + 2 * w < n ? lo + 2 * w : n;
+            int a = lo, b = mid, o = lo;
+            while (a < mid && b < hi) tmp[o++] = (adj[idx[b]] > adj[idx[a]]) ? idx[b++] : idx[a++];
+            while (a < mid) tmp[o++] = idx[a++];
+            while (b < hi) tmp[o++] = idx[b++];
+        }
+        int *sw = idx;
+        idx = tmp;
+        tmp = sw;
+    }
+    float target = top_p < 0.f ? 0.f : (top_p > 1.f ? 1.f : top_p);
+    if (target < 1e-6f) target = 1e-6f;
+    float cumulative = 0.f;
+    int cut = 0;
+    for (int k = 0; k < n; ++k) {
+        cumulative += adj[idx[k]];
+        cut = k + 1;
+        if (cumulative >= target) break;
+    }
+    if (cut < 1) cut = 1;
+    float acc = 0.f;
+    int pick = idx[cut - 1];
+    for (int k = 0; k < cut; ++k) {
+        acc += adj[idx[k]] / cumulative;
+        if (r <= acc) {
+            pick = idx[k];
+            break;
+        }
+    }
+    free(adj);
+    free(idx);
+    free(tmp);
+    return pick;
+}
+
 /* ------------------------------------------------------------------------
  * KVCacheInner.  src/layers/attention/self_attention.rs:24-44
  * ---------------------------------------------------------------------- */

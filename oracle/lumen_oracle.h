@@ -70,6 +70,9 @@ int lo_embedding_f32(const float *W, const float *ids, int n_ids, int vocab, int
 void lo_bf16_to_f32(const uint16_t *src, float *dst, long n);
 void lo_f32_to_bf16_rne(const float *src, uint16_t *dst, long n);
 int lo_argmax_f32(const float *x, int n);
+/* sample_top_p, src/main.rs:74-137, with the uniform draw r supplied by the caller */
+int lo_sample_top_p(const float *logits, int n, float temperature, float top_p, float repetition_penalty,
+                    const int *recent, int n_recent, float r);
 
 /* static KV cache: k, v are [B, H_kv, max_seq, D] (self_attention.rs:24-44) */
 typedef struct {

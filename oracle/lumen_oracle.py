@@ -80,6 +80,7 @@ _sig("lo_embedding_f32", C.c_int, _f, _f, C.c_int, C.c_int, C.c_int, _f)
 _sig("lo_bf16_to_f32", None, _u16, _f, C.c_long)
 _sig("lo_f32_to_bf16_rne", None, _f, _u16, C.c_long)
 _sig("lo_argmax_f32", C.c_int, _f, C.c_int)
+_sig("lo_sample_top_p", C.c_int, _f, C.c_int, C.c_float, C.c_float, C.c_float, C.POINTER(C.c_int), C.c_int, C.c_float)
 _sig("lo_kv_cache_new", C.POINTER(KVCacheStruct), C.c_int, C.c_int, C.c_int, C.c_int)
 _sig("lo_kv_cache_reset", None, C.POINTER(KVCacheStruct))
 _sig("lo_kv_cache_free", None, C.POINTER(KVCacheStruct))
@@ -202,6 +203,14 @@ def f32_to_bf16(x):
 
 def argmax(x):
     return _lib.lo_argmax_f32(_p(x), x.size)
+
+
+def sample_top_p(logits, temperature, top_p, repetition_penalty, recent, r):
+    """sample_top_p of src/main.rs:74-137 with the uniform draw r given."""
+    logits = np.ascontiguousarray(logits, np.float32)
+    rec = np.ascontiguousarray(recent, np.int32)
+    return _lib.lo_sample_top_p(_p(logits), logits.size, float(temperature), float(top_p), float(repetition_penalty),
+                                rec.ctypes.data_as(C.POINTER(C.c_int)), rec.size, float(r))
 
 
 class KVCache:
