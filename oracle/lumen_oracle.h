@@ -23,6 +23,10 @@
  *     pinned by fp64 closed forms, algebraic invariants, brute force and
  *     torch / HF-transformers (config-only, random-init) cross-checks in
  *     tests/test_oracle_*.py.
+ *   lo_sample_top_p: pinned in tests/test_sampler.py by the definition of
+ *     nucleus sampling (share of a swept draw per token = renormalised fp64
+ *     softmax over the shortest prefix reaching top_p, ties in index order,
+ *     penalty and temperature special cases).
  *   lo_gemm_f32 and the two GEMMs inside lo_attn_prefill_f32: the reference
  *     calls matrixmultiply::sgemm (transitive dependency of ndarray 0.15,
  *     version not locked, source not in the reference tree); its accumulation
