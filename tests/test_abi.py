@@ -55,3 +55,17 @@ def test_product_never_imports_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".hpp", ".cpp")) or f == "Makefile":
                 text = open(os.path.join(dirpath, f), errors="replace").read()
                 assert "oracle" not in text.lower(), os.path.join(dirpath, f)
+
+
+def test_rust_binding_is_in_step_with_the_header():
+    """include/lumen_hip_ffi.rs is generated from the header; it must be regenerated when the header changes
+    and has to name every symbol the Python binding names."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    rc = subprocess.run([sys.executable, os.path.join(root, "include", "gen_rust_ffi.py"), "--check"]).returncode
+    assert rc == 0, "run python include/gen_rust_ffi.py"
+    from lumen_amd import _lib
+    text = open(os.path.join(root, "include", "lumen_hip_ffi.rs")).read()
+    for name in _lib.SIGNATURES:
+        assert "pub fn %s(" % name in text, name
