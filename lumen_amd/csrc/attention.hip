@@ -184,12 +184,9 @@ __global__ __launch_bounds__(WAVES * 64) void attn_decode_kernel(AttnDecodeArgs 
     }
     __syncthreads();
     if (!s_last) return;
-    for (int e = t; e < NREP * D; e += THREADS) {
-        const int r = e / D, dd = e % D;
-        const int hq = hk * NREP + r;
-        const float *pp = a.part + (((size_t)bb * a.hq + hq) * gridDim.x) * (D + 2);
-        a.out[((size_t)bb * a.hq + hq) * D + dd] = fold_slices<D>(pp, nact, dd);
-    }
+    // sacc is free again: slice weights [NREP][64] and the NREP reciprocals behind them
+    fold_slices_block<D, NREP, WAVES>(a.part + (((size_t)bb * a.hq + (size_t)hk * NREP) * gridDim.x) * (D + 2), gridDim.x, nact,
+                                      sacc, sacc + NREP * 64, a.out + ((size_t)bb * a.hq + (size_t)hk * NREP) * D);
 }
 
 int attn_decode_nsplit(int max_seq) {

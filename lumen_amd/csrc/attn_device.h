@@ -276,6 +276,62 @@ __device__ __forceinline__ float fold_slices(const float *pp, int nact, int dd) 
     return Cx * (1.0f / (Ls + 1e-9f));
 }
 
+// The same fold for a whole KV group by one workgroup, with one trip to memory instead of one per
+// batch of slices: every thread first requests the context partials of its own output element
+// (up to 32 slices, held in registers), then wavefront r reads the (max, sum) pairs of head r --
+// lane s takes slice s -- and leaves the slice weights exp2(m_s - M) and 1 / (sum + 1e-9) in LDS;
+// after the barrier the partials are already there.  More than 32 slices take a second trip.
+// part_group: partials of the group's first head; heads are nsplit * (D + 2) floats apart.
+// w_lds [NREP][64], linv_lds [NREP].  All threads of the workgroup call it; nsplit <= 64.
+template <int D, int NREP, int WAVES>
+__device__ __forceinline__ void fold_slices_block(const float *part_group, int nsplit, int nact, float *w_lds,
+                                                  float *linv_lds, float *out_group) {
+    constexpr int THREADS = WAVES * 64, B = 32;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const size_t head_stride = (size_t)nsplit * (D + 2);
+    // context partials of the first output element of this thread
+    float cv[B];
+    {
+        const int r = (t / D) % NREP, dd = t % D;  // t < NREP * D, or a harmless in-range duplicate
+        const float *pp = part_group + r * head_stride;
+#pragma unroll
+        for (int j = 0; j < B; ++j) cv[j] = part_load(pp + (size_t)min(j, nact - 1) * (D + 2) + dd);
+    }
+    for (int r = wave; r < NREP; r += WAVES) {
+        const float *pp = part_group + r * head_stride + (size_t)min(lane, nact - 1) * (D + 2);
+        float m = part_load(pp + D), l = part_load(pp + D + 1);
+        if (lane >= nact) {
+            m = -INFINITY;
+            l = 0.f;
+        }
+        float M = m;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off, 64));
+        const float w = (m > -INFINITY) ? fast_exp2(m - M) : 0.f;
+        float L = l * w;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) L += __shfl_xor(L, off, 64);
+        w_lds[r * 64 + lane] = w;
+        if (lane == 0) linv_lds[r] = 1.0f / (L + 1e-9f);
+    }
+    __syncthreads();
+    for (int e = t; e < NREP * D; e += THREADS) {
+        const int r = e / D, dd = e % D;
+        const float *pp = part_group + r * head_stride;
+        float acc = 0.f;
+        for (int s0 = 0; s0 < nact; s0 += B) {
+            if (e != t || s0 != 0) {
+#pragma unroll
+                for (int j = 0; j < B; ++j) cv[j] = part_load(pp + (size_t)min(s0 + j, nact - 1) * (D + 2) + dd);
+            }
+#pragma unroll
+            for (int j = 0; j < B; ++j)
+                if (s0 + j < nact) acc = fmaf(cv[j], w_lds[r * 64 + s0 + j], acc);
+        }
+        out_group[r * D + dd] = acc * linv_lds[r];
+    }
+}
+
 // How the cached rows [0, pos) are cut into slices for one decode step: only
 // as many slices as give each at least one full trip of rows take part, the
 // others return at once.  The new token (row `pos`) belongs to the last
