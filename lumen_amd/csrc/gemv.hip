@@ -412,7 +412,13 @@ int launch_gemv(lumen_ctx *ctx, const GemvArgs &a) {
         LUMEN_FAIL(LUMEN_ERR_SHAPE, "paired-row epilogue needs an even row count, got %d", a.N);
     const int nunits = (a.N + R - 1) / R;
     int blocks = (nunits + GEMV_WAVES - 1) / GEMV_WAVES;
-    const int cap = ctx->num_cus * 4;
+    // one wave of workgroups: at most 4 per compute unit, fewer when their staged x would not fit the
+    // compute unit's 160 KiB of LDS side by side (a second, partial wave of workgroups costs more
+    // than longer row loops: 4.0 -> 4.7 TB/s at K = 11008 with bf16 weights)
+    int per_cu = (int)((size_t)(160 * 1024) / (lds + 256));
+    if (per_cu > 4) per_cu = 4;
+    if (per_cu < 1) per_cu = 1;
+    const int cap = ctx->num_cus * per_cu;
     if (blocks > cap) blocks = cap;
     dim3 grid(blocks);
     if (a.w_bf16) {
