@@ -26,24 +26,92 @@ struct DecodeWaves {
     static constexpr int value = 8;
 };
 
-// Short contexts (up to ATTN_SHORT_ROWS cached rows, q already rotated): one query head per
+// Short contexts (up to ATTN_SHORT_ROWS cached rows, 256 for head_dim 128): one query head per
 // workgroup over ALL rows, 8 row loads per lane in flight, so that nothing has to travel between
 // workgroups -- at these lengths the hand-over of partial results through memory (an atomic and
 // a round of agent-scope loads, each a trip to the memory side) costs more than reading the few
 // hundred K/V rows once per query head instead of once per KV head.
 #define ATTN_SHORT_ROWS 512
-template <int D, int WAVES>
-__device__ __forceinline__ void attn_decode_short(const AttnDecodeArgs &a, int hq, int hk, int bb, int pos, float *sm,
-                                                  float *sl, float *sacc) {
-    constexpr int LPR = D / 4, RPW = 64 / LPR, RPI = WAVES * RPW, UB = 8;
+// row loads per lane in flight in one trip of the short form: 256 rows per trip for head_dim 64 and 128
+template <int D>
+struct ShortTrip {
+    static constexpr int loads = (D >= 128) ? 16 : 8;
+};
+// PRE: q is rotated and cache row pos_new written already; otherwise this workgroup normalises and
+// rotates its own query head and the group's new key itself (a few hundred flops, repeated by
+// every head of the group so that nothing has to be exchanged), the first head of the group
+// stores the new row, and every head takes that row from LDS (q_raw .. v_new: D floats each).
+template <int D, int WAVES, bool PRE>
+__device__ __forceinline__ void attn_decode_short(const AttnDecodeArgs &a, int r, int nrep, int hk, int bb, int pos_new,
+                                                  float *q_raw, float *q_rot, float *k_raw, float *k_new,
+                                                  float *v_new, float *sm, float *sl, float *sacc) {
+    constexpr int LPR = D / 4, RPW = 64 / LPR, RPI = WAVES * RPW, UB = ShortTrip<D>::loads, THREADS = WAVES * 64;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int off = wave * RPW + lane / LPR, c = lane % LPR;
+    const int hq = hk * nrep + r;
+    const int pos = PRE ? pos_new + 1 : pos_new;  // rows read from the cache
     const size_t head_base = ((size_t)bb * a.hkv + hk) * a.max_seq * D;
     const float *Kb = a.k_cache + head_base + c * 4, *Vb = a.v_cache + head_base + c * 4;
     AttnState<1> st;
     state_init<1>(st);
     v4f q[1];
     bool have_q = false;
+    auto get_q = [&]() {
+        if (PRE) {
+            load_q_scaled<D, 1>(q, a.q + ((size_t)bb * a.hq + hq) * D, c, a.scale);
+        } else {
+            // wavefront 0 takes the query head, wavefront 1 the new key, wavefront 2 copies the new value:
+            // lane j holds the pair (j, j + D/2); everything they need from memory is requested at once
+            constexpr int HALF = D / 2;
+            const float *cs = a.cos_t + (size_t)pos_new * D, *sn = a.sin_t + (size_t)pos_new * D;
+            if (wave < 2) {
+                const float *src = wave == 0 ? a.q + ((size_t)bb * a.hq + hq) * D : a.k_new + ((size_t)bb * a.hkv + hk) * D;
+                const float *g = wave == 0 ? a.q_norm_w : a.k_norm_w;
+                float x1 = 0.f, x2 = 0.f, cc = 0.f, ss_ = 0.f, g1 = 1.f, g2 = 1.f;
+                if (lane < HALF) {
+                    x1 = src[lane];
+                    x2 = src[lane + HALF];
+                    cc = cs[lane];
+                    ss_ = sn[lane];
+                    if (g) {
+                        g1 = g[lane];
+                        g2 = g[lane + HALF];
+                    }
+                }
+                if (g) {  // per-head RMSNorm before the rotation
+                    float sq = x1 * x1 + x2 * x2;
+#pragma unroll
+                    for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o, 64);
+                    const float inv = 1.0f / sqrtf(sq / (float)D + a.norm_eps);
+                    x1 = x1 * inv * g1;
+                    x2 = x2 * inv * g2;
+                }
+                float o1, o2;
+                {
+#pragma clang fp contract(off)  // separate multiplies and add, like the reference's compiled code
+                    o1 = x1 * cc - x2 * ss_;
+                    o2 = x1 * ss_ + x2 * cc;
+                }
+                float *dst = wave == 0 ? q_rot : k_new;
+                if (lane < HALF) {
+                    dst[lane] = o1;
+                    dst[lane + HALF] = o2;
+                }
+            } else if (wave == 2) {
+                const float *v_src = a.v_new + ((size_t)bb * a.hkv + hk) * D;
+                for (int i = lane; i < D; i += 64) v_new[i] = v_src[i];
+            }
+            __syncthreads();
+            if (r == 0) {  // self_attention.rs:161-176: rotated k and raw v go to cache row pos_new
+                for (int i = threadIdx.x; i < D; i += THREADS) {
+                    a.k_cache[head_base + (size_t)pos_new * D + i] = k_new[i];
+                    a.v_cache[head_base + (size_t)pos_new * D + i] = v_new[i];
+                }
+            }
+            load_q_scaled<D, 1>(q, q_rot, c, a.scale);
+        }
+        have_q = true;
+    };
     for (int base = 0; base < pos; base += RPI * UB) {
         v4f kv[UB], vv[UB];
 #pragma unroll
@@ -52,17 +120,21 @@ __device__ __forceinline__ void attn_decode_short(const AttnDecodeArgs &a, int h
             kv[u] = *(const v4f *)(Kb + (size_t)j * D);
             vv[u] = *(const v4f *)(Vb + (size_t)j * D);
         }
-        if (!have_q) {
-            load_q_scaled<D, 1>(q, a.q + ((size_t)bb * a.hq + hq) * D, c, a.scale);
-            have_q = true;
-        }
+        if (!have_q) get_q();  // after the first rows have been requested: they do not depend on q
 #pragma unroll
         for (int u = 0; u < UB; ++u)
             if (base + u * RPI < pos) attn_step<D, 1>(st, q, kv[u], vv[u], base + u * RPI + off < pos);
     }
+    if (!PRE) {
+        if (!have_q) get_q();  // empty cache: the new token attends to itself only
+        if (wave == 0) {       // the new row, from LDS (lane group 0 of wavefront 0)
+            const v4f kn = *(const v4f *)(k_new + c * 4), vn = *(const v4f *)(v_new + c * 4);
+            attn_step<D, 1>(st, q, kn, vn, lane / LPR == 0);
+        }
+    }
     wave_merge_publish<D, 1>(st, sm, sl, sacc);
     __syncthreads();
-    for (int dd = threadIdx.x; dd < D; dd += WAVES * 64) {
+    for (int dd = threadIdx.x; dd < D; dd += THREADS) {
         float mm, ls, cx;
         wave_fold<D, 1, WAVES>(sm, sl, sacc, 0, dd, mm, ls, cx);
         a.out[((size_t)bb * a.hq + hq) * D + dd] = cx * (1.0f / (ls + 1e-9f));  // self_attention.rs:287-290
@@ -87,13 +159,15 @@ __global__ __launch_bounds__(WAVES * 64) void attn_decode_kernel(AttnDecodeArgs 
     const int split = blockIdx.x, hk = blockIdx.y, bb = blockIdx.z;
     const int pos_new = a.pos_dev ? *a.pos_dev : a.pos_host;  // == past_len, the new token's position
     const int pos = PRE ? pos_new + 1 : pos_new;             // rows that come from the cache
-    if (PRE && pos <= ATTN_SHORT_ROWS && (int)gridDim.x >= NREP) {
+    // the short form walks the rows in trips, one after the other: two trips at most
+    constexpr int SHORT_ROWS = (2 * ShortTrip<D>::loads * G::RPI < ATTN_SHORT_ROWS) ? 2 * ShortTrip<D>::loads * G::RPI : ATTN_SHORT_ROWS;
+    if (pos_new + 1 <= SHORT_ROWS && (int)gridDim.x >= NREP) {
         // Workgroups are dealt round-robin over the 8 XCDs, each with an L2 of its own.  With 32 or
         // more workgroups per KV head the heads of a group are placed 8 apart, four to an XCD, so
         // that a group's K/V rows are fetched into two L2s instead of eight.
         int r = split;
         if (NREP == 8 && gridDim.x >= 32 && (gridDim.x & 7) == 0) r = (split & 7) < 2 && split < 32 ? (split >> 3) + 4 * (split & 7) : NREP;
-        if (r < NREP) attn_decode_short<D, WAVES>(a, hk * NREP + r, hk, bb, pos, sm, sl, sacc);
+        if (r < NREP) attn_decode_short<D, WAVES, PRE>(a, r, NREP, hk, bb, pos_new, q_raw, q_rot, k_raw, k_new, v_new, sm, sl, sacc);
         return;
     }
     int nact, chunk;
