@@ -26,16 +26,17 @@ struct DecodeWaves {
     static constexpr int value = 8;
 };
 
-// Short contexts (up to ATTN_SHORT_ROWS cached rows, 256 for head_dim 128): one query head per
+// Short contexts (up to ATTN_SHORT_ROWS cached rows; 256 for head_dim 128): one query head per
 // workgroup over ALL rows, 8 row loads per lane in flight, so that nothing has to travel between
 // workgroups -- at these lengths the hand-over of partial results through memory (an atomic and
 // a round of agent-scope loads, each a trip to the memory side) costs more than reading the few
 // hundred K/V rows once per query head instead of once per KV head.
 #define ATTN_SHORT_ROWS 512
-// row loads per lane in flight in one trip of the short form: 256 rows per trip for head_dim 64 and 128
+// row loads per lane in flight in one trip of the short form (256 rows per trip for head_dim 64, 128 for
+// head_dim 128; 16 loads there would double the kernel's registers and halve the split form's occupancy)
 template <int D>
 struct ShortTrip {
-    static constexpr int loads = (D >= 128) ? 16 : 8;
+    static constexpr int loads = 8;
 };
 // PRE: q is rotated and cache row pos_new written already; otherwise this workgroup normalises and
 // rotates its own query head and the group's new key itself (a few hundred flops, repeated by

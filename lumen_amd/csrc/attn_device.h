@@ -283,19 +283,18 @@ __device__ __forceinline__ float fold_slices(const float *pp, int nact, int dd) 
 // after the barrier the partials are already there.  More than 32 slices take a second trip.
 // part_group: partials of the group's first head; heads are nsplit * (D + 2) floats apart.
 // w_lds [NREP][64], linv_lds [NREP].  All threads of the workgroup call it; nsplit <= 64.
-template <int D, int NREP, int WAVES>
-__device__ __forceinline__ void fold_slices_block(const float *part_group, int nsplit, int nact, float *w_lds,
-                                                  float *linv_lds, float *out_group) {
-    constexpr int THREADS = WAVES * 64, B = 32;
+template <int D, int NREP, int WAVES, int B>
+__device__ __forceinline__ void fold_slices_block_b(const float *part_group, int nsplit, int nact, float *w_lds,
+                                                    float *linv_lds, float *out_group) {
+    constexpr int THREADS = WAVES * 64;
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const size_t head_stride = (size_t)nsplit * (D + 2);
     // context partials of the first output element of this thread
     float cv[B];
-    {
-        const int r = (t / D) % NREP, dd = t % D;  // t < NREP * D, or a harmless in-range duplicate
-        const float *pp = part_group + r * head_stride;
+    if (t < NREP * D) {
+        const float *pp = part_group + (t / D) * head_stride + t % D;
 #pragma unroll
-        for (int j = 0; j < B; ++j) cv[j] = part_load(pp + (size_t)min(j, nact - 1) * (D + 2) + dd);
+        for (int j = 0; j < B; ++j) cv[j] = part_load(pp + (size_t)min(j, nact - 1) * (D + 2));
     }
     for (int r = wave; r < NREP; r += WAVES) {
         const float *pp = part_group + r * head_stride + (size_t)min(lane, nact - 1) * (D + 2);
@@ -317,12 +316,12 @@ __device__ __forceinline__ void fold_slices_block(const float *part_group, int n
     __syncthreads();
     for (int e = t; e < NREP * D; e += THREADS) {
         const int r = e / D, dd = e % D;
-        const float *pp = part_group + r * head_stride;
+        const float *pp = part_group + r * head_stride + dd;
         float acc = 0.f;
         for (int s0 = 0; s0 < nact; s0 += B) {
             if (e != t || s0 != 0) {
 #pragma unroll
-                for (int j = 0; j < B; ++j) cv[j] = part_load(pp + (size_t)min(s0 + j, nact - 1) * (D + 2) + dd);
+                for (int j = 0; j < B; ++j) cv[j] = part_load(pp + (size_t)min(s0 + j, nact - 1) * (D + 2));
             }
 #pragma unroll
             for (int j = 0; j < B; ++j)
@@ -330,6 +329,14 @@ __device__ __forceinline__ void fold_slices_block(const float *part_group, int n
         }
         out_group[r * D + dd] = acc * linv_lds[r];
     }
+}
+
+template <int D, int NREP, int WAVES>
+__device__ __forceinline__ void fold_slices_block(const float *part_group, int nsplit, int nact, float *w_lds,
+                                                  float *linv_lds, float *out_group) {
+    if (nact <= 8) fold_slices_block_b<D, NREP, WAVES, 8>(part_group, nsplit, nact, w_lds, linv_lds, out_group);
+    else if (nact <= 16) fold_slices_block_b<D, NREP, WAVES, 16>(part_group, nsplit, nact, w_lds, linv_lds, out_group);
+    else fold_slices_block_b<D, NREP, WAVES, 32>(part_group, nsplit, nact, w_lds, linv_lds, out_group);
 }
 
 // How the cached rows [0, pos) are cut into slices for one decode step: only
