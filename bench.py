@@ -37,8 +37,10 @@ def main():
                     help="how decode steps are issued: a HIP graph replay per token (default) or kernel by kernel "
                          "(for rocprofv3 --kernel-trace, which cannot follow graph replays here)")
     ap.add_argument("--cpu-tokens", type=int, default=48)
-    ap.add_argument("--workload", choices=["decode", "gemv", "copy"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "gemv", "gemm", "prefill", "copy"], default="decode",
                     help="decode: the headline batch-1 decode benchmark; gemv: the isolated M=1 GEMV shapes; "
+                         "gemm: the prompt-pass GEMM shapes against the fp32 matrix-core peak; prefill: one long "
+                         "prompt pass (3968 tokens, TinyLlama shape with a 4096-row cache); "
                          "copy: a plain 1 GiB copy kernel (calibrates the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -49,6 +51,10 @@ def main():
         return gemv_microbench(args)
     if args.workload == "copy":
         return copy_bench(args)
+    if args.workload == "gemm":
+        return gemm_microbench(args)
+    if args.workload == "prefill":
+        return prefill_bench(args)
 
     import numpy as np
 
@@ -241,6 +247,72 @@ def gemv_microbench(args):
         del slab
     print(json.dumps({"metric": "M=1 GEMV HBM GB/s", "unit": "GB/s", "n_gpus": 1, "dtype": "f32", "data": "synthetic",
                       "layout": "[N,K] row-major (out,in)", "shapes": rows}))
+
+
+GEMM_SHAPES = [(128, 2048, 2048), (128, 2560, 2048), (128, 11264, 2048), (128, 2048, 5632), (512, 2048, 2048),
+               (512, 11264, 2048), (3968, 2048, 2048), (3968, 11264, 2048), (3968, 2048, 5632), (512, 4096, 4096)]
+
+
+def gemm_microbench(args):
+    """C[M,N] = A[M,K] W[N,K]^T in fp32 on the matrix cores (the M > 1 branch of matmul, the prompt
+    pass): M = prompt rows, (N, K) the projection shapes.  Flops 2 M N K against 157.3 TFLOP/s."""
+    import ctypes as C
+
+    import numpy as np
+
+    from lumen_amd._lib import check, lib
+    from lumen_amd.autograd import Tensor, default_ctx
+
+    ctx = default_ctx()
+    rng = np.random.default_rng(0)
+    rows = []
+    for M, N, K in GEMM_SHAPES:
+        A = rng.standard_normal((M, K), dtype=np.float32)
+        W = rng.standard_normal((N, K), dtype=np.float32) * np.float32(0.02)
+        Ad, Wd = Tensor.from_array_no_grad(A, ctx), Tensor.from_array_no_grad(W, ctx)
+        Cd = Tensor.empty((M, N), np.float32, ctx)
+        ms = C.c_float()
+        for iters in (3, 20):
+            check(lib.lumen_timer_start(ctx.handle))
+            for _ in range(iters):
+                check(lib.lumen_gemm_f32(ctx.handle, Ad.ptr, Wd.ptr, Cd.ptr, M, N, K))
+            check(lib.lumen_timer_stop(ctx.handle, C.byref(ms)))
+        us = ms.value * 1e3 / 20
+        ref = A[:32].astype(np.float64) @ W.T.astype(np.float64)
+        err = float(np.abs(Cd.data()[:32] - ref).max() / np.abs(ref).max())
+        tf = 2.0 * M * N * K / us / 1e6
+        rows.append({"M": M, "N": N, "K": K, "us": round(us, 1), "TFLOPs": round(tf, 1),
+                     "frac_of_mfma_fp32_peak": round(tf / MFMA_FP32_PEAK_TF, 4), "max_rel_err": err})
+    print(json.dumps({"metric": "prompt-pass GEMM fp32 TFLOP/s", "unit": "TFLOP/s", "n_gpus": 1, "dtype": "f32",
+                      "data": "synthetic", "peak_TFLOPs": MFMA_FP32_PEAK_TF, "shapes": rows}))
+
+
+def prefill_bench(args):
+    """One long prompt pass: TinyLlama shape, 4096-row cache, 3968 random ids, last-row logits."""
+    import numpy as np
+
+    from lumen_amd import synth
+    from lumen_amd.models import LlamaModel
+
+    cfg = dict(synth.TINYLLAMA_1B_LONG)
+    S = 3968 if args.prompt == 128 else args.prompt
+    model = LlamaModel(cfg)
+    for name, a in synth.iter_params(cfg, seed=0):
+        model.set_param(name, a)
+    ids = synth.make_tokens(S, cfg["vocab_size"], seed=0)
+    passes = []
+    for _ in range(3):
+        model.reset_kv_caches()
+        model.ctx.timer_start()
+        model.forward(ids, all_rows=False)
+        passes.append(model.ctx.timer_stop())
+    out = {"metric": "prompt tokens/s", "value": round(S / passes[-1] * 1e3, 1), "unit": "tokens/s", "n_gpus": 1,
+           "dtype": "f32", "data": "synthetic",
+           "config": {"workload": "TinyLlama-1.1B-shaped Llama fp32 random-init seed 0, batch 1, one prompt pass of %d "
+                                  "random ids into an empty cache of %d rows" % (S, cfg["max_seq_len"])}}
+    out.update(prefill_report(cfg, S, passes[-1]))
+    out["passes_ms"] = [round(x, 3) for x in passes]
+    print(json.dumps(out))
 
 
 def cpu_baseline(cfg, params, prompt, n_tokens):
