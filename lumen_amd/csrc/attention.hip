@@ -8,10 +8,14 @@
 //    online-softmax state (m, l, ctx); states are merged across lane groups
 //    with shuffles, across wavefronts through LDS and across slices through
 //    a small global scratch by the last workgroup to finish (fixed order, so
-//    results are reproducible run to run).
+//    results are reproducible run to run).  Short caches take another form:
+//    one workgroup per query head over all rows, nothing handed between
+//    workgroups (attn_decode_short).
 //  * prefill (S > 1), self_attention.rs:308-419 + :519-678: rotate q/k and
-//    append to the cache, then one workgroup per (query position, KV group)
-//    runs the same row loop over the causal prefix.
+//    append to the cache, then either the matrix-core kernel of
+//    prefill_attention.hip (head_dim 64 / 128, long prompts) or one workgroup
+//    per (query position, KV group) running the decode row loop over the
+//    causal prefix.
 #include "internal.h"
 #include "attn_device.h"
 

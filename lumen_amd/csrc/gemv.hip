@@ -6,8 +6,9 @@
 // on the way in).  One 64-lane wavefront owns R whole rows at a time; each
 // lane streams 16-byte pieces of the rows (a wavefront covers 1 KiB of a row
 // per load instruction, fully coalesced), multiplies them with its slice of x
-// from LDS and the 64 partial sums are folded with cross-lane shuffles.  The
-// row loop keeps 8 independent 16-byte loads per lane in flight.
+// from LDS and the 64 partial sums are folded with cross-lane shuffles.  A
+// wavefront's rows are walked in pieces of 8 independent 16-byte loads per
+// lane and two pieces are kept in flight (16 loads per lane).
 #include "internal.h"
 
 typedef float v4f __attribute__((ext_vector_type(4)));
