@@ -10,7 +10,10 @@
 // cache serves all n_rep heads of the group and 128 / n_rep positions at once.
 //
 // Per wavefront (32 rows) and key tile:
-//   S  = Q K^T        D/2 v_mfma_f32_32x32x2_f32, Q fragments in registers, K from LDS
+//   S  = Q K^T        D/2 v_mfma_f32_32x32x2_f32, Q fragments in registers, K from LDS.  The two
+//                     k-values an instruction consumes are (kk, D/2 + kk): a lane then needs D/2
+//                     CONSECUTIVE floats of its K row, fetched with 16-byte LDS reads (the sum over
+//                     the head dimension does not care how its terms are paired; P V likewise)
 //   row max           across the 32 lanes that hold a row's 32 keys (DPP + one shuffle)
 //   P  = exp2(S - m)  scores are kept in log2 units (Q is pre-multiplied by scale * log2 e);
 //                     the row sums stay per lane and are folded across lanes once at the end
@@ -48,10 +51,11 @@ __global__ __launch_bounds__(FA_THREADS) void attn_prefill_mfma_kernel(AttnPrefi
     constexpr int BQ = FA_ROWS / NREP;       // positions per workgroup
     constexpr int DT = D / 32;               // 32-wide output tiles per row
     constexpr int PIECES = D * FA_KEYS / 4 / FA_THREADS;  // 16-byte pieces of a K (or V) tile per thread
-    constexpr int LDK = D + 1;
-    __shared__ float Ks[FA_KEYS][LDK];
-    __shared__ __align__(16) float Vs[FA_KEYS][D];
-    __shared__ float Ps[FA_THREADS / 64][32][33];
+    // row strides = 4 mod 32 words: 16-byte reads of 8 neighbouring rows fall into distinct banks
+    constexpr int LDK = D + 4, LDV = FA_KEYS + 4, LDP = FA_KEYS + 4;
+    __shared__ __align__(16) float Ks[FA_KEYS][LDK];   // [key][element]
+    __shared__ __align__(16) float Vt[D][LDV];         // [element][key]: V transposed
+    __shared__ __align__(16) float Ps[FA_THREADS / 64][32][LDP];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = lane & 31, half = lane >> 5;
@@ -64,14 +68,17 @@ __global__ __launch_bounds__(FA_THREADS) void attn_prefill_mfma_kernel(AttnPrefi
     // accumulator register r of lane l belongs to row 8*(r/4) + 4*(l/32) + r%4 of the wavefront's 32
     auto row_of = [&](int r) { return 8 * (r >> 2) + 4 * half + (r & 3); };
 
-    // Q fragments: lane l feeds row l%32, element 2*kk + l/32 of the dot product
+    // Q fragments: lane l feeds row l%32, element (l/32) * D/2 + kk of the dot product
     const int my_row = wave * 32 + c;                 // row this lane feeds as an A operand
     const int my_i = min(q0 + my_row / NREP, a.s - 1);  // clamped: rows past S are computed and dropped
     const float *qrow = a.q_rot + (((size_t)bb * a.s + my_i) * a.hq + (size_t)hk * NREP + my_row % NREP) * D;
     const float qf_scale = a.scale * LUMEN_LOG2E;
     float qf[D / 2];
 #pragma unroll
-    for (int kk = 0; kk < D / 2; ++kk) qf[kk] = qrow[2 * kk + half] * qf_scale;
+    for (int kk = 0; kk < D / 2; kk += 4) {
+        const v4f v = *(const v4f *)(qrow + half * (D / 2) + kk);
+        qf[kk] = v.x * qf_scale; qf[kk + 1] = v.y * qf_scale; qf[kk + 2] = v.z * qf_scale; qf[kk + 3] = v.w * qf_scale;
+    }
 
     // keys this workgroup needs: up to the last position's own key
     const int q_last = min(q0 + BQ, a.s) - 1;
@@ -114,8 +121,8 @@ __global__ __launch_bounds__(FA_THREADS) void attn_prefill_mfma_kernel(AttnPrefi
         for (int p = 0; p < PIECES; ++p) {
             const int idx = tid + p * FA_THREADS;
             const int key = idx / (D / 4), k4 = (idx % (D / 4)) * 4;
-            Ks[key][k4 + 0] = kreg[p].x; Ks[key][k4 + 1] = kreg[p].y; Ks[key][k4 + 2] = kreg[p].z; Ks[key][k4 + 3] = kreg[p].w;
-            *(v4f *)&Vs[key][k4] = vreg[p];
+            *(v4f *)&Ks[key][k4] = kreg[p];
+            Vt[k4 + 0][key] = vreg[p].x; Vt[k4 + 1][key] = vreg[p].y; Vt[k4 + 2][key] = vreg[p].z; Vt[k4 + 3][key] = vreg[p].w;
         }
         __syncthreads();
         if (j0 + FA_KEYS < kmax) fetch(j0 + FA_KEYS);  // in flight during the matrix instructions below
@@ -125,8 +132,13 @@ __global__ __launch_bounds__(FA_THREADS) void attn_prefill_mfma_kernel(AttnPrefi
 #pragma unroll
             for (int r = 0; r < 16; ++r) S[r] = 0.f;
 #pragma unroll
-            for (int kk = 0; kk < D / 2; ++kk)
-                S = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[kk], Ks[c][2 * kk + half], S, 0, 0, 0);
+            for (int kk = 0; kk < D / 2; kk += 4) {
+                const v4f kf = *(const v4f *)&Ks[c][half * (D / 2) + kk];
+                S = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[kk], kf.x, S, 0, 0, 0);
+                S = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[kk + 1], kf.y, S, 0, 0, 0);
+                S = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[kk + 2], kf.z, S, 0, 0, 0);
+                S = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[kk + 3], kf.w, S, 0, 0, 0);
+            }
 
             const int j = j0 + c;  // this lane's key
             float alpha[16];
@@ -150,12 +162,18 @@ __global__ __launch_bounds__(FA_THREADS) void attn_prefill_mfma_kernel(AttnPrefi
 #pragma unroll
                 for (int r = 0; r < 16; ++r) O[t][r] *= alpha[r];
             __builtin_amdgcn_wave_barrier();  // P: written above by this wavefront, read below in another lane order
+            // keys (kk, 16 + kk) per instruction: 16 consecutive floats of the P row and of each V^T row
 #pragma unroll
-            for (int kk = 0; kk < FA_KEYS / 2; ++kk) {
-                const float pf = Ps[wave][c][2 * kk + half];
+            for (int kk = 0; kk < FA_KEYS / 2; kk += 4) {
+                const v4f pf = *(const v4f *)&Ps[wave][c][half * (FA_KEYS / 2) + kk];
 #pragma unroll
-                for (int t = 0; t < DT; ++t)
-                    O[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(pf, Vs[2 * kk + half][32 * t + c], O[t], 0, 0, 0);
+                for (int t = 0; t < DT; ++t) {
+                    const v4f vf = *(const v4f *)&Vt[32 * t + c][half * (FA_KEYS / 2) + kk];
+                    O[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(pf.x, vf.x, O[t], 0, 0, 0);
+                    O[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(pf.y, vf.y, O[t], 0, 0, 0);
+                    O[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(pf.z, vf.z, O[t], 0, 0, 0);
+                    O[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(pf.w, vf.w, O[t], 0, 0, 0);
+                }
             }
         }
         __syncthreads();
