@@ -221,6 +221,30 @@ def test_decode_modes_agree_with_each_other_and_the_oracle(cfg, bf16, n_prompt):
     assert np.array_equal(results["graph"][1], results["eager"][1])
 
 
+@pytest.mark.parametrize("cfg_extra,n_prompt", [
+    (dict(num_attention_heads=8, num_key_value_heads=1, max_seq_len=640), 505),             # head_dim 64, n_rep 8: 512
+    (dict(num_attention_heads=8, num_key_value_heads=2, max_seq_len=1100), 506),            # n_rep 4, 16 slices offered
+    (dict(hidden_size=256, num_attention_heads=2, num_key_value_heads=1, max_seq_len=330, intermediate_size=704), 250),  # head_dim 128: 256
+    (dict(num_attention_heads=8, num_key_value_heads=2, max_seq_len=600, qk_norm=True, head_dim=64), 507),  # norm in the kernel
+], ids=["d64-nrep8", "d64-nrep4", "d128-nrep2", "d64-qknorm"])
+def test_decode_across_the_short_to_split_attention_boundary(cfg_extra, n_prompt):
+    """Decode attention changes form where the cache passes 512 rows (256 for head_dim 128): steps on both sides of
+    the boundary, and the step that crosses it, agree with the checker."""
+    cfg = dict(vocab_size=900, hidden_size=512, intermediate_size=1408, num_hidden_layers=2, rms_norm_eps=1e-5,
+               rope_theta=10000.0)
+    cfg.update(cfg_extra)
+    gpu, ora, _ = build(cfg, seed=33)
+    ids = synth.make_tokens(n_prompt + 14, cfg["vocab_size"], seed=33)
+    got = gpu.forward(ids[:n_prompt], all_rows=False)
+    rc, ref = ora.forward(ids[:n_prompt])
+    assert rc == lo.LO_OK and max_rel(got, ref[-1]) <= 1e-4
+    for t in range(n_prompt, n_prompt + 14):
+        g = gpu.forward(ids[t:t + 1], all_rows=False)
+        _, r = ora.forward(ids[t:t + 1])
+        assert max_rel(g, r[0]) <= 1e-4, t
+    assert gpu.kv_len == n_prompt + 14
+
+
 @pytest.mark.slow
 def test_tinyllama_1b_shape_prefill_128_decode_teacher_forced():
     """The headline configuration at full size: 22 layers, hidden 2048, 32/4 heads, vocab 32000,
