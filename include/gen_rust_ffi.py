@@ -2,7 +2,8 @@
 
 Usage: python include/gen_rust_ffi.py [--check]    (--check: exit 1 when the committed file is out of date)
 
-The reference crate is Rust; this file is what a maintainer drops into it as src/ffi.rs.
+The reference crate is Rust; this file is what a maintainer drops into it as src/ffi.rs (add `mod ffi;` and
+link liblumen_hip.so from build.rs).
 No Rust toolchain exists where this library is built, so the output is generated text, not compiled code."""
 import os
 import re
@@ -75,7 +76,7 @@ def struct_fields(text, name):
 def generate():
     text = open(HEADER).read()
     out = ["// Generated from include/lumen_hip.h by include/gen_rust_ffi.py -- do not edit.",
-           "// Rust binding of liblumen_hip.so: `mod ffi;` in the reference crate, see INTEGRATION.md.",
+           "// Rust binding of liblumen_hip.so: src/ffi.rs + `mod ffi;` in the reference crate; link the library from build.rs.",
            "#![allow(non_camel_case_types, dead_code)]",
            "use std::os::raw::{c_char, c_float, c_int, c_void};", ""]
     for o in OPAQUE:

@@ -1,5 +1,5 @@
 // Generated from include/lumen_hip.h by include/gen_rust_ffi.py -- do not edit.
-// Rust binding of liblumen_hip.so: `mod ffi;` in the reference crate, see INTEGRATION.md.
+// Rust binding of liblumen_hip.so: src/ffi.rs + `mod ffi;` in the reference crate; link the library from build.rs.
 #![allow(non_camel_case_types, dead_code)]
 use std::os::raw::{c_char, c_float, c_int, c_void};
 
