@@ -242,10 +242,10 @@ int lumen_llama_get_config(const lumen_llama *model, lumen_llama_config *cfg_out
 int lumen_llama_decode_profile(lumen_llama *model, int first_id, int n, double *ms_sum_out,
                                int *count_out, int n_classes);
 /* how S == 1 steps are issued (no reference counterpart; the results are the same):
- * PERSISTENT (default when head_dim is 64 or 128): one cooperative kernel runs all
- * layers of all requested steps, weights of the next stage streaming across each
- * grid barrier; GRAPH: one captured HIP graph replay per token (5 kernels per layer);
- * EAGER: the same kernels launched one by one (for kernel tracing tools). */
+ * GRAPH (default): one captured HIP graph replay per token (5 kernels per layer);
+ * EAGER: the same kernels launched one by one (for kernel tracing tools);
+ * PERSISTENT: one cooperative kernel for all layers of all requested steps -- switched
+ * off in this build, lumen_llama_set_decode_mode returns LUMEN_ERR_UNSUPPORTED for it. */
 #define LUMEN_DECODE_EAGER 0
 #define LUMEN_DECODE_GRAPH 1
 #define LUMEN_DECODE_PERSISTENT 2
