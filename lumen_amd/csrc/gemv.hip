@@ -329,7 +329,11 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(GemvArgs a) {
                 }
             if (bi == 0x7fffffff) bi = 0;  // all NaN: index 0 like a sequential scan
             *a.tok_out = bi;
-            if (a.pos_inc) *a.pos_inc += 1;
+            if (a.pos_inc) {
+                const int pos = *a.pos_inc;
+                if (a.tok_hist) a.tok_hist[pos + 1] = bi;  // the pick is the token of the next position
+                *a.pos_inc = pos + 1;
+            }
         }
     }
 }

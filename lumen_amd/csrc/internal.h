@@ -95,6 +95,7 @@ struct GemvArgs {
     int *amax_idx;     // [gridDim.x]
     int *amax_counter; // zero between launches
     int *tok_out, *pos_inc;
+    int *tok_hist;     // optional [max_seq + 1]: the pick is also stored at index *pos_inc + 1
     // EPI_ROPE_QKV: rows are q|k|v heads of D; a unit is the RoPE pair (j, j + D/2) of one head.
     // q is rotated into y, k rotated and v as is go to row *pos of the KV cache.
     const float *cos_t, *sin_t;

@@ -40,6 +40,7 @@ struct lumen_llama {
     // decode state
     float *x = nullptr, *h = nullptr, *qkv = nullptr, *attn = nullptr, *act = nullptr, *logits = nullptr;
     int *d_tok = nullptr, *d_pos = nullptr;
+    int *tok_hist = nullptr;  // [max_seq + 1]: greedy pick made at position p sits at index p + 1
     float *part = nullptr;
     int *counters = nullptr;
     int nsplit = 1;
@@ -173,6 +174,7 @@ extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg,
     M_TRY(dmalloc_t(m, &m->logits, (size_t)V));
     M_TRY(dmalloc_t(m, &m->d_tok, 4));
     M_TRY(dmalloc_t(m, &m->d_pos, 4));
+    M_TRY(dmalloc_t(m, &m->tok_hist, (size_t)cfg->max_seq_len + 1));
     m->nsplit = attn_decode_nsplit(cfg->max_seq_len);
     M_TRY(dmalloc_t(m, &m->part, attn_decode_part_floats(1, Hq, D, m->nsplit)));
     M_TRY(dmalloc_t(m, &m->counters, (size_t)Hkv));
@@ -466,7 +468,7 @@ static int enqueue_decode_step(lumen_llama *m, StepProbe *pr = nullptr) {
     g.pro = PRO_RMSNORM; g.norm_w = m->final_norm; g.eps = c.rms_norm_eps;
     // the greedy pick is folded in: it becomes the next token id and the position counter advances
     g.epi = EPI_ARGMAX; g.amax_val = m->amax_val; g.amax_idx = m->amax_idx; g.amax_counter = m->amax_counter;
-    g.tok_out = m->d_tok; g.pos_inc = m->d_pos;
+    g.tok_out = m->d_tok; g.pos_inc = m->d_pos; g.tok_hist = m->tok_hist;
     pr->before(KC_LMHEAD);
     const int rc = launch_gemv(ctx, g);
     pr->after();
@@ -703,9 +705,9 @@ extern "C" int lumen_llama_decode_greedy(lumen_llama *m, int first_id, int n, in
     const size_t V = (size_t)m->cfg.vocab_size;
     HIP_TRY(hipMemcpyAsync(m->d_tok, &first_id, sizeof(int), hipMemcpyHostToDevice, st));
     HIP_TRY(hipStreamSynchronize(st));
-    int *ids_dev = nullptr;
-    if (ids_out) HIP_TRY(hipMalloc((void **)&ids_dev, sizeof(int) * (size_t)n));
     if (m->decode_mode == LUMEN_DECODE_PERSISTENT) {
+        int *ids_dev = nullptr;
+        if (ids_out) HIP_TRY(hipMalloc((void **)&ids_dev, sizeof(int) * (size_t)n));
         float *logits_dev = nullptr;
         if (logits_out && hipMalloc((void **)&logits_dev, sizeof(float) * V * (size_t)n) != hipSuccess) {
             hipFree(ids_dev);
@@ -721,11 +723,11 @@ extern "C" int lumen_llama_decode_greedy(lumen_llama *m, int first_id, int n, in
         if (prc == LUMEN_OK && pe != hipSuccess) LUMEN_FAIL(LUMEN_ERR_HIP, "decode_greedy: %s", hipGetErrorString(pe));
         return prc;
     }
+    // the arg-max epilogue leaves every pick in tok_hist at the index of the position it is the token of
+    const int len0 = m->len;
     int rc = LUMEN_OK;
     for (int t = 0; t < n && rc == LUMEN_OK; ++t) {
         hipError_t e = launch_step(m);
-        if (e == hipSuccess && ids_dev)
-            e = hipMemcpyAsync(ids_dev + t, m->d_tok, sizeof(int), hipMemcpyDeviceToDevice, st);
         if (e == hipSuccess && logits_out)
             e = hipMemcpyAsync(logits_out + (size_t)t * V, m->logits, sizeof(float) * V, hipMemcpyDeviceToHost, st);
         if (e != hipSuccess) {
@@ -736,9 +738,8 @@ extern "C" int lumen_llama_decode_greedy(lumen_llama *m, int first_id, int n, in
         }
     }
     hipError_t e = hipStreamSynchronize(st);
-    if (rc == LUMEN_OK && e == hipSuccess && ids_dev)
-        e = hipMemcpy(ids_out, ids_dev, sizeof(int) * (size_t)n, hipMemcpyDeviceToHost);
-    hipFree(ids_dev);
+    if (rc == LUMEN_OK && e == hipSuccess && ids_out)
+        e = hipMemcpy(ids_out, m->tok_hist + len0 + 1, sizeof(int) * (size_t)n, hipMemcpyDeviceToHost);
     if (rc == LUMEN_OK && e != hipSuccess) LUMEN_FAIL(LUMEN_ERR_HIP, "decode_greedy: %s", hipGetErrorString(e));
     return rc;
 }
