@@ -46,21 +46,40 @@ struct ShortTrip {
 // rotates its own query head and the group's new key itself (a few hundred flops, repeated by
 // every head of the group so that nothing has to be exchanged), the first head of the group
 // stores the new row, and every head takes that row from LDS (q_raw .. v_new: D floats each).
+//
+// pos_new < 0: the position is not known yet.  The first trip of rows and the query are requested
+// before it is read -- they do not depend on it: a row past the cached ones is only masked later --
+// so the position's own trip to memory is off the critical path.  Returns false, having done
+// nothing, when the position then turns out to lie past short_rows.
 template <int D, int WAVES, bool PRE>
-__device__ __forceinline__ void attn_decode_short(const AttnDecodeArgs &a, int r, int nrep, int hk, int bb, int pos_new,
-                                                  float *q_raw, float *q_rot, float *k_raw, float *k_new,
-                                                  float *v_new, float *sm, float *sl, float *sacc) {
+__device__ __forceinline__ bool attn_decode_short(const AttnDecodeArgs &a, int r, int nrep, int hk, int bb, int pos_new,
+                                                  int short_rows, float *q_raw, float *q_rot, float *k_raw,
+                                                  float *k_new, float *v_new, float *sm, float *sl, float *sacc) {
     constexpr int LPR = D / 4, RPW = 64 / LPR, RPI = WAVES * RPW, UB = ShortTrip<D>::loads, THREADS = WAVES * 64;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int off = wave * RPW + lane / LPR, c = lane % LPR;
     const int hq = hk * nrep + r;
-    const int pos = PRE ? pos_new + 1 : pos_new;  // rows read from the cache
     const size_t head_base = ((size_t)bb * a.hkv + hk) * a.max_seq * D;
     const float *Kb = a.k_cache + head_base + c * 4, *Vb = a.v_cache + head_base + c * 4;
     AttnState<1> st;
     state_init<1>(st);
     v4f q[1];
     bool have_q = false;
+    // first trip: rows u * RPI + off, clamped to the cache (not to the position: see above)
+    v4f kv0[UB], vv0[UB];
+#pragma unroll
+    for (int u = 0; u < UB; ++u) {
+        const int j = min(u * RPI + off, a.max_seq - 1);
+        kv0[u] = *(const v4f *)(Kb + (size_t)j * D);
+        vv0[u] = *(const v4f *)(Vb + (size_t)j * D);
+    }
+    if (PRE) {
+        load_q_scaled<D, 1>(q, a.q + ((size_t)bb * a.hq + hq) * D, c, a.scale);
+        have_q = true;
+    }
+    if (pos_new < 0) pos_new = a.pos_dev ? *a.pos_dev : a.pos_host;
+    if (pos_new + 1 > short_rows) return false;
+    const int pos = PRE ? pos_new + 1 : pos_new;  // rows read from the cache
     auto get_q = [&]() {
         if (PRE) {
             load_q_scaled<D, 1>(q, a.q + ((size_t)bb * a.hq + hq) * D, c, a.scale);
@@ -117,7 +136,11 @@ __device__ __forceinline__ void attn_decode_short(const AttnDecodeArgs &a, int r
         }
         have_q = true;
     };
-    for (int base = 0; base < pos; base += RPI * UB) {
+    if (!have_q && pos > 0) get_q();
+#pragma unroll
+    for (int u = 0; u < UB; ++u)
+        if (u * RPI < pos) attn_step<D, 1>(st, q, kv0[u], vv0[u], u * RPI + off < pos);
+    for (int base = RPI * UB; base < pos; base += RPI * UB) {
         v4f kv[UB], vv[UB];
 #pragma unroll
         for (int u = 0; u < UB; ++u) {  // rows past the end are clamped here and masked in attn_step
@@ -125,7 +148,6 @@ __device__ __forceinline__ void attn_decode_short(const AttnDecodeArgs &a, int r
             kv[u] = *(const v4f *)(Kb + (size_t)j * D);
             vv[u] = *(const v4f *)(Vb + (size_t)j * D);
         }
-        if (!have_q) get_q();  // after the first rows have been requested: they do not depend on q
 #pragma unroll
         for (int u = 0; u < UB; ++u)
             if (base + u * RPI < pos) attn_step<D, 1>(st, q, kv[u], vv[u], base + u * RPI + off < pos);
@@ -144,6 +166,7 @@ __device__ __forceinline__ void attn_decode_short(const AttnDecodeArgs &a, int r
         wave_fold<D, 1, WAVES>(sm, sl, sacc, 0, dd, mm, ls, cx);
         a.out[((size_t)bb * a.hq + hq) * D + dd] = cx * (1.0f / (ls + 1e-9f));  // self_attention.rs:287-290
     }
+    return true;
 }
 
 // PRE: q arrives rotated and cache row `pos` is already written (both done by the q|k|v GEMV's
@@ -162,17 +185,24 @@ __global__ __launch_bounds__(WAVES * 64) void attn_decode_kernel(AttnDecodeArgs 
     __shared__ int s_last;
 
     const int split = blockIdx.x, hk = blockIdx.y, bb = blockIdx.z;
-    const int pos_new = a.pos_dev ? *a.pos_dev : a.pos_host;  // == past_len, the new token's position
-    const int pos = PRE ? pos_new + 1 : pos_new;             // rows that come from the cache
     // the short form walks the rows in trips, one after the other: two trips at most
     constexpr int SHORT_ROWS = (2 * ShortTrip<D>::loads * G::RPI < ATTN_SHORT_ROWS) ? 2 * ShortTrip<D>::loads * G::RPI : ATTN_SHORT_ROWS;
-    if (pos_new + 1 <= SHORT_ROWS && (int)gridDim.x >= NREP) {
-        // Workgroups are dealt round-robin over the 8 XCDs, each with an L2 of its own.  With 32 or
-        // more workgroups per KV head the heads of a group are placed 8 apart, four to an XCD, so
-        // that a group's K/V rows are fetched into two L2s instead of eight.
-        int r = split;
-        if (NREP == 8 && gridDim.x >= 32 && (gridDim.x & 7) == 0) r = (split & 7) < 2 && split < 32 ? (split >> 3) + 4 * (split & 7) : NREP;
-        if (r < NREP) attn_decode_short<D, WAVES, PRE>(a, r, NREP, hk, bb, pos_new, q_raw, q_rot, k_raw, k_new, v_new, sm, sl, sacc);
+    // Short form: workgroup `split` takes query head r of the group.  Workgroups are dealt
+    // round-robin over the 8 XCDs, each with an L2 of its own; with 32 or more workgroups per KV
+    // head the heads of a group are placed 8 apart, four to an XCD, so that a group's K/V rows are
+    // fetched into two L2s instead of eight.
+    int r = split;
+    if (NREP == 8 && gridDim.x >= 32 && (gridDim.x & 7) == 0) r = (split & 7) < 2 && split < 32 ? (split >> 3) + 4 * (split & 7) : NREP;
+    const bool short_fits = (int)gridDim.x >= NREP;
+    // the caller expects a short cache: start the short form before the position is known
+    if (a.expect_short && short_fits && r < NREP &&
+        attn_decode_short<D, WAVES, PRE>(a, r, NREP, hk, bb, -1, SHORT_ROWS, q_raw, q_rot, k_raw, k_new, v_new, sm, sl, sacc))
+        return;
+    const int pos_new = a.pos_dev ? *a.pos_dev : a.pos_host;  // == past_len, the new token's position
+    const int pos = PRE ? pos_new + 1 : pos_new;             // rows that come from the cache
+    if (pos_new + 1 <= SHORT_ROWS && short_fits) {
+        if (r < NREP && !a.expect_short)
+            attn_decode_short<D, WAVES, PRE>(a, r, NREP, hk, bb, pos_new, SHORT_ROWS, q_raw, q_rot, k_raw, k_new, v_new, sm, sl, sacc);
         return;
     }
     int nact, chunk;

@@ -149,6 +149,7 @@ struct AttnDecodeArgs {
     int *counters;
     int nsplit;
     int pre_rotated;    // q is already rotated and row pos of the cache already written (fused QKV GEMV)
+    int expect_short;   // hint: the cache is short (a few hundred rows); a wrong hint only costs time
 };
 int launch_attn_decode(lumen_ctx *ctx, const AttnDecodeArgs &a);
 

@@ -46,6 +46,7 @@ struct lumen_llama {
     int nsplit = 1;
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
+    int graph_expect_short = 0;            // the hint the captured attention launches carry
     int decode_mode = LUMEN_DECODE_GRAPH;  // persistent when the shape allows, set at create
     PkLayer *pk_layers = nullptr;          // device copy of the per-layer pointers
     float *amax_val = nullptr;
@@ -404,6 +405,10 @@ struct StepProbe {  // brackets every launch with a HIP event pair when profilin
     }
 };
 
+// Is the cache short enough for the one-workgroup-per-head form of decode attention?  A hint for the
+// kernel (it starts that form before it has read the position); a wrong one only costs time.
+static int expect_short_cache(const lumen_llama *m) { return m->len + 1 <= (m->D >= 128 ? 256 : 512); }
+
 static int enqueue_decode_step(lumen_llama *m, StepProbe *pr = nullptr) {
     StepProbe none;
     if (!pr) pr = &none;
@@ -435,6 +440,7 @@ static int enqueue_decode_step(lumen_llama *m, StepProbe *pr = nullptr) {
         a.b = 1; a.hq = c.num_attention_heads; a.hkv = c.num_key_value_heads; a.d = m->D; a.max_seq = c.max_seq_len;
         a.scale = m->scale; a.q_norm_w = w.q_norm; a.k_norm_w = w.k_norm; a.norm_eps = c.rms_norm_eps;
         a.part = m->part; a.counters = m->counters; a.nsplit = m->nsplit; a.pre_rotated = fuse_rope;
+        a.expect_short = expect_short_cache(m);
         pr->before(KC_ATTN);
         LUMEN_TRY(launch_attn_decode(ctx, a));
         pr->after();
@@ -476,7 +482,17 @@ static int enqueue_decode_step(lumen_llama *m, StepProbe *pr = nullptr) {
 }
 
 static int ensure_decode_graph(lumen_llama *m) {
-    if (m->graph_exec || m->decode_mode != LUMEN_DECODE_GRAPH) return LUMEN_OK;
+    if (m->decode_mode != LUMEN_DECODE_GRAPH) return LUMEN_OK;
+    if (m->graph_exec && m->graph_expect_short != expect_short_cache(m)) {
+        // the captured attention launches carry the hint for the other side of the boundary
+        HIP_TRY(hipStreamSynchronize(m->ctx->stream));
+        hipGraphExecDestroy(m->graph_exec);
+        hipGraphDestroy(m->graph);
+        m->graph_exec = nullptr;
+        m->graph = nullptr;
+    }
+    if (m->graph_exec) return LUMEN_OK;
+    m->graph_expect_short = expect_short_cache(m);
     hipStream_t s = m->ctx->stream;
     HIP_TRY(hipStreamSynchronize(s));
     HIP_TRY(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
