@@ -14,8 +14,9 @@
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 
-#define GEMV_THREADS 256
+#define GEMV_THREADS 256                  // default workgroup: 4 wavefronts
 #define GEMV_WAVES (GEMV_THREADS / 64)
+#define GEMV_MAX_WAVES 8                  // the kernel takes its size from blockDim.x, up to this
 
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
@@ -62,10 +63,10 @@ __device__ __forceinline__ float dot16(const v4u raw, const float *xs) {
 template <int PRO>
 __device__ __forceinline__ void stage_x(float *xs, const float *__restrict__ x, const float *__restrict__ g,
                                         float eps, int K, int kpad) {
-    __shared__ float red[GEMV_WAVES];
-    const int tid = threadIdx.x;
+    __shared__ float red[GEMV_MAX_WAVES];
+    const int tid = threadIdx.x, nthreads = blockDim.x, nwaves = nthreads >> 6;
     float ss = 0.f;
-    for (int k = tid * 4; k < kpad; k += GEMV_THREADS * 4) {
+    for (int k = tid * 4; k < kpad; k += nthreads * 4) {
         v4f v = {0.f, 0.f, 0.f, 0.f};
         if (k < K) v = *(const v4f *)(x + k);
         ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
@@ -76,11 +77,10 @@ __device__ __forceinline__ void stage_x(float *xs, const float *__restrict__ x, 
         if ((tid & 63) == 0) red[tid >> 6] = ss;
         __syncthreads();
         float tot = 0.f;
-#pragma unroll
-        for (int w = 0; w < GEMV_WAVES; ++w) tot += red[w];
+        for (int w = 0; w < nwaves; ++w) tot += red[w];
         const float rms = sqrtf(tot / (float)K + eps);
         const float inv = 1.0f / rms;
-        for (int k = tid * 4; k < K; k += GEMV_THREADS * 4) {
+        for (int k = tid * 4; k < K; k += nthreads * 4) {
             v4f v = *(const v4f *)(xs + k);
             const v4f gg = *(const v4f *)(g + k);
             v.x = v.x * inv * gg.x;
@@ -94,7 +94,7 @@ __device__ __forceinline__ void stage_x(float *xs, const float *__restrict__ x, 
 }
 
 template <bool BF16, int R, int PRO, int EPI>
-__global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(GemvArgs a) {
+__global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(GemvArgs a) {
     extern __shared__ __align__(16) float xs[];
     constexpr int VEC = BF16 ? 8 : 4;          // elements per 16-byte load
     constexpr int SWEEP = 64 * VEC;            // elements one wavefront covers per load
@@ -105,8 +105,9 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(GemvArgs a) {
     const int kpad = (K + PIECE - 1) / PIECE * PIECE;  // xs is zero from K to kpad
 
     const int lane = threadIdx.x & 63;
-    const int gw = blockIdx.x * GEMV_WAVES + (threadIdx.x >> 6);
-    const int nw = gridDim.x * GEMV_WAVES;
+    const int nwaves = blockDim.x >> 6;
+    const int gw = blockIdx.x * nwaves + (threadIdx.x >> 6);
+    const int nw = gridDim.x * nwaves;
     const int nunits = (N + R - 1) / R;
     const char *Wb = (const char *)a.W;
     const size_t row_bytes = (size_t)K * ESZ;
@@ -270,8 +271,8 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(GemvArgs a) {
     if (EPI == EPI_ARGMAX) {
         // greedy pick fused into the lm_head product: per-workgroup candidates go through memory with
         // agent-scope accesses, the last workgroup to arrive folds them (lowest index wins ties)
-        __shared__ float am_v[GEMV_WAVES];
-        __shared__ int am_i[GEMV_WAVES];
+        __shared__ float am_v[GEMV_MAX_WAVES];
+        __shared__ int am_i[GEMV_MAX_WAVES];
         __shared__ int am_last;
         const int wave = threadIdx.x >> 6;
         if (lane == 0) {
@@ -280,7 +281,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(GemvArgs a) {
         }
         __syncthreads();
         if (threadIdx.x == 0) {
-            for (int w = 1; w < GEMV_WAVES; ++w)
+            for (int w = 1; w < nwaves; ++w)
                 if (am_v[w] > best || (am_v[w] == best && am_i[w] < best_idx)) {
                     best = am_v[w];
                     best_idx = am_i[w];
@@ -298,7 +299,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(GemvArgs a) {
         if (!am_last) return;
         float bv = -INFINITY;
         int bi = 0x7fffffff;
-        for (int i = threadIdx.x; i < (int)gridDim.x; i += GEMV_THREADS) {
+        for (int i = threadIdx.x; i < (int)gridDim.x; i += (int)blockDim.x) {
             const float v = __hip_atomic_load(a.amax_val + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             const int ix = __hip_atomic_load(a.amax_idx + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if (v > bv || (v == bv && ix < bi)) {
@@ -322,7 +323,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(GemvArgs a) {
         }
         __syncthreads();
         if (threadIdx.x == 0) {
-            for (int w = 1; w < GEMV_WAVES; ++w)
+            for (int w = 1; w < nwaves; ++w)
                 if (am_v[w] > bv || (am_v[w] == bv && am_i[w] < bi)) {
                     bv = am_v[w];
                     bi = am_i[w];
@@ -360,32 +361,32 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_generic_kernel(GemvArgs a) 
 }
 
 template <bool BF16, int R, int PRO>
-static void launch_epi(const GemvArgs &a, dim3 grid, size_t lds, hipStream_t s) {
+static void launch_epi(const GemvArgs &a, dim3 grid, int threads, size_t lds, hipStream_t s) {
     switch (a.epi) {
         case EPI_STORE:
-            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_STORE>), grid, dim3(GEMV_THREADS), lds, s, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_STORE>), grid, dim3(threads), lds, s, a);
             break;
         case EPI_RESIDUAL:
-            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_RESIDUAL>), grid, dim3(GEMV_THREADS), lds, s, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_RESIDUAL>), grid, dim3(threads), lds, s, a);
             break;
         case EPI_ARGMAX:
-            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_ARGMAX>), grid, dim3(GEMV_THREADS), lds, s, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_ARGMAX>), grid, dim3(threads), lds, s, a);
             break;
         case EPI_ROPE_QKV:
-            hipLaunchKernelGGL((gemv_kernel<BF16, 2, PRO, EPI_ROPE_QKV>), grid, dim3(GEMV_THREADS), lds, s, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, 2, PRO, EPI_ROPE_QKV>), grid, dim3(threads), lds, s, a);
             break;
         default:
-            hipLaunchKernelGGL((gemv_kernel<BF16, 2, PRO, EPI_SWIGLU>), grid, dim3(GEMV_THREADS), lds, s, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, 2, PRO, EPI_SWIGLU>), grid, dim3(threads), lds, s, a);
             break;
     }
 }
 
 template <bool BF16, int R>
-static void launch_pro(const GemvArgs &a, dim3 grid, size_t lds, hipStream_t s) {
+static void launch_pro(const GemvArgs &a, dim3 grid, int threads, size_t lds, hipStream_t s) {
     if (a.pro == PRO_RMSNORM)
-        launch_epi<BF16, R, PRO_RMSNORM>(a, grid, lds, s);
+        launch_epi<BF16, R, PRO_RMSNORM>(a, grid, threads, lds, s);
     else
-        launch_epi<BF16, R, PRO_NONE>(a, grid, lds, s);
+        launch_epi<BF16, R, PRO_NONE>(a, grid, threads, lds, s);
 }
 
 int gemv_max_blocks(const lumen_ctx *ctx) { return ctx->num_cus * 4; }
@@ -416,7 +417,16 @@ int launch_gemv(lumen_ctx *ctx, const GemvArgs &a) {
     if ((a.epi == EPI_SWIGLU || a.epi == EPI_ROPE_QKV) && (a.N & 1))
         LUMEN_FAIL(LUMEN_ERR_SHAPE, "paired-row epilogue needs an even row count, got %d", a.N);
     const int nunits = (a.N + R - 1) / R;
-    int blocks = (nunits + GEMV_WAVES - 1) / GEMV_WAVES;
+    // Wavefronts per workgroup: when the units divide into exactly one workgroup of 5 to 8 wavefronts
+    // per compute unit, take that shape -- every compute unit gets the same share and stages x once
+    // (q|k|v of a 2048-wide model: 1280 pairs = 256 x 5; its o_proj and down: 2048 rows = 256 x 8).
+    int waves = GEMV_WAVES;
+    if (nunits % ctx->num_cus == 0) {
+        const int w = nunits / ctx->num_cus;
+        if (w > GEMV_WAVES && w <= GEMV_MAX_WAVES) waves = w;
+    }
+    const int threads = waves * 64;
+    int blocks = (nunits + waves - 1) / waves;
     // one wave of workgroups: at most 4 per compute unit, fewer when their staged x would not fit the
     // compute unit's 160 KiB of LDS side by side (a second, partial wave of workgroups costs more
     // than longer row loops: 4.0 -> 4.7 TB/s at K = 11008 with bf16 weights)
@@ -427,11 +437,11 @@ int launch_gemv(lumen_ctx *ctx, const GemvArgs &a) {
     if (blocks > cap) blocks = cap;
     dim3 grid(blocks);
     if (a.w_bf16) {
-        if (R == 2) launch_pro<true, 2>(a, grid, lds, ctx->stream);
-        else launch_pro<true, 1>(a, grid, lds, ctx->stream);
+        if (R == 2) launch_pro<true, 2>(a, grid, threads, lds, ctx->stream);
+        else launch_pro<true, 1>(a, grid, threads, lds, ctx->stream);
     } else {
-        if (R == 2) launch_pro<false, 2>(a, grid, lds, ctx->stream);
-        else launch_pro<false, 1>(a, grid, lds, ctx->stream);
+        if (R == 2) launch_pro<false, 2>(a, grid, threads, lds, ctx->stream);
+        else launch_pro<false, 1>(a, grid, threads, lds, ctx->stream);
     }
     LUMEN_CHECK_LAUNCH();
     return LUMEN_OK;
