@@ -431,7 +431,8 @@ int launch_gemv(lumen_ctx *ctx, const GemvArgs &a) {
     // compute unit's 160 KiB of LDS side by side (a second, partial wave of workgroups costs more
     // than longer row loops: 4.0 -> 4.7 TB/s at K = 11008 with bf16 weights)
     int per_cu = (int)((size_t)(160 * 1024) / (lds + 256));
-    if (per_cu > 4) per_cu = 4;
+    const int max_per_cu = 16 / waves > 1 ? 16 / waves : 1;  // 16 wavefronts per compute unit
+    if (per_cu > max_per_cu) per_cu = max_per_cu;
     if (per_cu < 1) per_cu = 1;
     const int cap = ctx->num_cus * per_cu;
     if (blocks > cap) blocks = cap;
