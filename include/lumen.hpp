@@ -413,6 +413,7 @@ class KVCacheInner {
         check(lumen_kv_cache_len(h_, &n));
         return (size_t)n;
     }
+    void set_len(size_t n) { check(lumen_kv_cache_set_len(h_, (int)n)); }  // a public field in the reference (:28)
     const std::vector<size_t> &shape() const { return shape_; }
     std::vector<float> k() const { return download(true); }
     std::vector<float> v() const { return download(false); }

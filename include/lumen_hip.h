@@ -141,6 +141,10 @@ int lumen_kv_cache_create(lumen_ctx *ctx, int b, int h_kv, int max_seq, int d, l
 int lumen_kv_cache_destroy(lumen_kv_cache *cache);
 int lumen_kv_cache_reset(lumen_kv_cache *cache);               /* :41-43, len = 0, data kept */
 int lumen_kv_cache_len(const lumen_kv_cache *cache, int *len_out);
+/* len is a public field of the reference's cache (:28): a caller that has filled rows itself
+ * (lumen_kv_cache_update, or through lumen_kv_cache_ptrs) says how many are valid; outside
+ * [0, max_seq] -> LUMEN_ERR_KV_OVERFLOW */
+int lumen_kv_cache_set_len(lumen_kv_cache *cache, int len);
 int lumen_kv_cache_ptrs(const lumen_kv_cache *cache, float **k_dev_out, float **v_dev_out);
 /* legacy LlamaKVCache::update / get_view, src/kv_cache.rs:31-59: k, v
  * [B, H_kv, S, D] written at start_pos (overflow -> LUMEN_ERR_KV_OVERFLOW);

@@ -89,6 +89,7 @@ extern "C" {
     pub fn lumen_kv_cache_destroy(cache: *mut lumen_kv_cache) -> c_int;
     pub fn lumen_kv_cache_reset(cache: *mut lumen_kv_cache) -> c_int;
     pub fn lumen_kv_cache_len(cache: *const lumen_kv_cache, len_out: *mut c_int) -> c_int;
+    pub fn lumen_kv_cache_set_len(cache: *mut lumen_kv_cache, len: c_int) -> c_int;
     pub fn lumen_kv_cache_ptrs(cache: *const lumen_kv_cache, k_dev_out: *mut *mut c_float, v_dev_out: *mut *mut c_float) -> c_int;
     pub fn lumen_kv_cache_update(cache: *mut lumen_kv_cache, k_dev: *const c_float, v_dev: *const c_float, s: c_int, start_pos: c_int) -> c_int;
     pub fn lumen_kv_cache_get_view(cache: *const lumen_kv_cache, current_len: c_int, k_out_dev: *mut c_float, v_out_dev: *mut c_float) -> c_int;

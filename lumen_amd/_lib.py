@@ -80,6 +80,7 @@ SIGNATURES = {
     "lumen_kv_cache_destroy": (_i, [_vp]),
     "lumen_kv_cache_reset": (_i, [_vp]),
     "lumen_kv_cache_len": (_i, [_vp, C.POINTER(_i)]),
+    "lumen_kv_cache_set_len": (_i, [_vp, _i]),
     "lumen_kv_cache_ptrs": (_i, [_vp, _pp, _pp]),
     "lumen_kv_cache_update": (_i, [_vp, _vp, _vp, _i, _i]),
     "lumen_kv_cache_get_view": (_i, [_vp, _i, _vp, _vp]),

@@ -1,16 +1,19 @@
 // Static KV cache and GQA attention over it.
 //
 //  * decode (S == 1), src/layers/attention/self_attention.rs:125-297: one
-//    workgroup per (KV head, slice of the cached positions).  The n_rep query
-//    heads of the KV group are rotated once into LDS; every K/V row is read
-//    from HBM exactly once per group as 16-byte pieces (D/4 lanes per row)
-//    and used for all n_rep heads from registers.  Each lane group keeps an
-//    online-softmax state (m, l, ctx); states are merged across lane groups
-//    with shuffles, across wavefronts through LDS and across slices through
-//    a small global scratch by the last workgroup to finish (fixed order, so
-//    results are reproducible run to run).  Short caches take another form:
-//    one workgroup per query head over all rows, nothing handed between
-//    workgroups (attn_decode_short).
+//    workgroup per (query head, slice of the cached positions).  A K/V row is
+//    read as 16-byte pieces (D/4 lanes per row), eight row loads per lane in
+//    flight; each lane group keeps an online-softmax state (m, l, ctx),
+//    merged across lane groups with shuffles and across wavefronts through
+//    LDS.  The step is bound by latency, not by bytes (a few tens of KB per
+//    compute unit), so the work is spread as widely as it goes: the n_rep
+//    heads of a KV group run in workgroups of their own, placed on the same
+//    XCD so that the group's rows come from HBM once and from that XCD's L2
+//    for the other heads.  A short cache is one slice: nothing travels
+//    between workgroups (attn_decode_short).  A long cache is cut into slices
+//    of one trip of rows each; partial states go through a small global
+//    scratch and the last workgroup of a head to finish folds them in a
+//    fixed order, so results are reproducible run to run (attn_decode_slice).
 //  * prefill (S > 1), self_attention.rs:308-419 + :519-678: rotate q/k and
 //    append to the cache, then either the matrix-core kernel of
 //    prefill_attention.hip (head_dim 64 / 128, long prompts) or one workgroup
@@ -45,7 +48,7 @@ struct ShortTrip {
 // PRE: q is rotated and cache row pos_new written already; otherwise this workgroup normalises and
 // rotates its own query head and the group's new key itself (a few hundred flops, repeated by
 // every head of the group so that nothing has to be exchanged), the first head of the group
-// stores the new row, and every head takes that row from LDS (q_raw .. v_new: D floats each).
+// stores the new row, and every head takes that row from LDS (q_rot, k_new, v_new: D floats each).
 //
 // pos_new < 0: the position is not known yet.  The first trip of rows and the query are requested
 // before it is read -- they do not depend on it: a row past the cached ones is only masked later --
@@ -53,8 +56,8 @@ struct ShortTrip {
 // nothing, when the position then turns out to lie past short_rows.
 template <int D, int WAVES, bool PRE>
 __device__ __forceinline__ bool attn_decode_short(const AttnDecodeArgs &a, int r, int nrep, int hk, int bb, int pos_new,
-                                                  int short_rows, float *q_raw, float *q_rot, float *k_raw,
-                                                  float *k_new, float *v_new, float *sm, float *sl, float *sacc) {
+                                                  int short_rows, float *q_rot, float *k_new,
+                                                  float *v_new, float *sm, float *sl, float *sacc) {
     constexpr int LPR = D / 4, RPW = 64 / LPR, RPI = WAVES * RPW, UB = ShortTrip<D>::loads, THREADS = WAVES * 64;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int off = wave * RPW + lane / LPR, c = lane % LPR;
@@ -169,19 +172,205 @@ __device__ __forceinline__ bool attn_decode_short(const AttnDecodeArgs &a, int r
     return true;
 }
 
+// Rows [0, pos) of a long cache are cut into nact slices of whole lane-group rounds, one trip of
+// rows (ShortTrip loads per lane) each unless the cache is longer than nslices trips.
+template <int D, int WAVES>
+__device__ __forceinline__ void long_slices(int pos, int nslices, int &nact, int &chunk) {
+    constexpr int RPI = WAVES * (64 / (D / 4)), TRIP = RPI * ShortTrip<D>::loads;
+    nact = (pos + TRIP - 1) / TRIP;
+    nact = nact < 1 ? 1 : (nact > nslices ? nslices : nact);
+    chunk = (pos + nact - 1) / nact;
+    chunk = (chunk + RPI - 1) / RPI * RPI;
+}
+
+// One query head (r of KV group hk) over slice `slice` of nact: rows [slice * chunk, ...) of the cache.
+// The partial state (ctx[D], m, l) goes to a.part[head][slice]; the last workgroup of the head to
+// arrive (a.counters[head]) folds the nact partials: slice weights exp2(m_s - M) from wavefront 0
+// (lane s takes slice s), the D context elements by THREADS / D thread groups that each take every
+// (THREADS / D)-th slice, their sums added in group order.  !PRE: every workgroup rotates its own
+// query head; the last slice also rotates the new key, takes the new row from LDS, and its first
+// head stores the row into the cache (self_attention.rs:161-176).
+template <int D, int WAVES, bool PRE>
+__device__ __forceinline__ void attn_decode_slice(const AttnDecodeArgs &a, int r, int nrep, int hk, int bb, int pos_new,
+                                                  int slice, int nact, int chunk, int nslices, float *q_rot,
+                                                  float *k_new, float *v_new, float *sm, float *sl, float *sacc,
+                                                  float *w_lds, int *s_last) {
+    constexpr int LPR = D / 4, RPW = 64 / LPR, RPI = WAVES * RPW, UB = ShortTrip<D>::loads, THREADS = WAVES * 64;
+    constexpr int GROUPS = THREADS / D, JMAX = (64 + GROUPS - 1) / GROUPS;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int off = wave * RPW + lane / LPR, c = lane % LPR;
+    const int hq = hk * nrep + r;
+    const int pos = PRE ? pos_new + 1 : pos_new;  // rows read from the cache
+    const int p0 = min(pos, slice * chunk), p1 = min(pos, p0 + chunk);
+    const bool has_new = !PRE && slice == nact - 1;
+    const size_t head_base = ((size_t)bb * a.hkv + hk) * a.max_seq * D;
+    const float *Kb = a.k_cache + head_base + c * 4, *Vb = a.v_cache + head_base + c * 4;
+    // first trip of rows: requested before anything else, it does not depend on q
+    v4f kv0[UB], vv0[UB];
+#pragma unroll
+    for (int u = 0; u < UB; ++u) {
+        const int j = max(min(p0 + u * RPI + off, p1 - 1), 0);
+        kv0[u] = *(const v4f *)(Kb + (size_t)j * D);
+        vv0[u] = *(const v4f *)(Vb + (size_t)j * D);
+    }
+    v4f q[1];
+    if (PRE) {
+        load_q_scaled<D, 1>(q, a.q + ((size_t)bb * a.hq + hq) * D, c, a.scale);
+    } else {
+        // wavefront 0 takes the query head; in the last slice wavefront 1 takes the new key and
+        // wavefront 2 copies the new value: lane j holds the pair (j, j + D/2)
+        constexpr int HALF = D / 2;
+        const float *cs = a.cos_t + (size_t)pos_new * D, *sn = a.sin_t + (size_t)pos_new * D;
+        if (wave == 0 || (wave == 1 && has_new)) {
+            const float *src = wave == 0 ? a.q + ((size_t)bb * a.hq + hq) * D : a.k_new + ((size_t)bb * a.hkv + hk) * D;
+            const float *g = wave == 0 ? a.q_norm_w : a.k_norm_w;
+            float x1 = 0.f, x2 = 0.f, cc = 0.f, ss_ = 0.f, g1 = 1.f, g2 = 1.f;
+            if (lane < HALF) {
+                x1 = src[lane];
+                x2 = src[lane + HALF];
+                cc = cs[lane];
+                ss_ = sn[lane];
+                if (g) {
+                    g1 = g[lane];
+                    g2 = g[lane + HALF];
+                }
+            }
+            if (g) {  // per-head RMSNorm before the rotation
+                float sq = x1 * x1 + x2 * x2;
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o, 64);
+                const float inv = 1.0f / sqrtf(sq / (float)D + a.norm_eps);
+                x1 = x1 * inv * g1;
+                x2 = x2 * inv * g2;
+            }
+            float o1, o2;
+            {
+#pragma clang fp contract(off)  // separate multiplies and add, like the reference's compiled code
+                o1 = x1 * cc - x2 * ss_;
+                o2 = x1 * ss_ + x2 * cc;
+            }
+            float *dst = wave == 0 ? q_rot : k_new;
+            if (lane < HALF) {
+                dst[lane] = o1;
+                dst[lane + HALF] = o2;
+            }
+        } else if (wave == 2 && has_new) {
+            const float *v_src = a.v_new + ((size_t)bb * a.hkv + hk) * D;
+            for (int i = lane; i < D; i += 64) v_new[i] = v_src[i];
+        }
+        __syncthreads();
+        if (has_new && r == 0) {
+            for (int i = t; i < D; i += THREADS) {
+                a.k_cache[head_base + (size_t)pos_new * D + i] = k_new[i];
+                a.v_cache[head_base + (size_t)pos_new * D + i] = v_new[i];
+            }
+        }
+        load_q_scaled<D, 1>(q, q_rot, c, a.scale);
+    }
+    AttnState<1> st;
+    state_init<1>(st);
+#pragma unroll
+    for (int u = 0; u < UB; ++u)
+        if (p0 + u * RPI < p1) attn_step<D, 1>(st, q, kv0[u], vv0[u], p0 + u * RPI + off < p1);
+    for (int base = p0 + RPI * UB; base < p1; base += RPI * UB) {  // caches longer than nslices trips
+        v4f kv[UB], vv[UB];
+#pragma unroll
+        for (int u = 0; u < UB; ++u) {
+            const int j = min(base + u * RPI + off, p1 - 1);
+            kv[u] = *(const v4f *)(Kb + (size_t)j * D);
+            vv[u] = *(const v4f *)(Vb + (size_t)j * D);
+        }
+#pragma unroll
+        for (int u = 0; u < UB; ++u)
+            if (base + u * RPI < p1) attn_step<D, 1>(st, q, kv[u], vv[u], base + u * RPI + off < p1);
+    }
+    if (has_new && wave == 0) {  // the new row, from LDS (lane group 0 of wavefront 0)
+        const v4f kn = *(const v4f *)(k_new + c * 4), vn = *(const v4f *)(v_new + c * 4);
+        attn_step<D, 1>(st, q, kn, vn, lane / LPR == 0);
+    }
+    wave_merge_publish<D, 1>(st, sm, sl, sacc);
+    __syncthreads();
+    float *out_head = a.out + ((size_t)bb * a.hq + hq) * D;
+    float *part_head = a.part + ((size_t)bb * a.hq + hq) * nslices * (D + 2);
+    for (int dd = t; dd < D; dd += THREADS) {
+        float mm, ls, cx;
+        wave_fold<D, 1, WAVES>(sm, sl, sacc, 0, dd, mm, ls, cx);
+        if (nact == 1) {
+            out_head[dd] = cx * (1.0f / (ls + 1e-9f));  // self_attention.rs:287-290
+        } else {
+            float *pp = part_head + (size_t)slice * (D + 2);
+            part_store(pp + dd, cx);
+            if (dd == 0) {
+                part_store(pp + D, mm);
+                part_store(pp + D + 1, ls);
+            }
+        }
+    }
+    if (nact == 1) return;
+    // The barrier makes every wavefront wait for its own stores before thread 0 signals.
+    __syncthreads();
+    if (t == 0) {
+        int *counter = a.counters + (size_t)bb * a.hq + hq;
+        const int old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *s_last = (old == nact - 1);
+        if (*s_last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!*s_last) return;
+    // fold: context partials of this thread's element and slices first (one trip to memory) ...
+    const int dd = t % D, grp = t / D;
+    float cv[JMAX];
+    if (grp < GROUPS) {
+#pragma unroll
+        for (int j = 0; j < JMAX; ++j) cv[j] = part_load(part_head + (size_t)min(grp + j * GROUPS, nact - 1) * (D + 2) + dd);
+    }
+    // ... then the slice weights, by wavefront 0
+    if (wave == 0) {
+        const float *pp = part_head + (size_t)min(lane, nact - 1) * (D + 2);
+        float m = part_load(pp + D), l = part_load(pp + D + 1);
+        if (lane >= nact) {
+            m = -INFINITY;
+            l = 0.f;
+        }
+        float M = m;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o, 64));
+        const float w = (m > -INFINITY) ? fast_exp2(m - M) : 0.f;
+        float L = l * w;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) L += __shfl_xor(L, o, 64);
+        w_lds[lane] = w;
+        if (lane == 0) w_lds[64] = 1.0f / (L + 1e-9f);
+    }
+    __syncthreads();
+    if (grp < GROUPS) {
+        float acc = 0.f;
+#pragma unroll
+        for (int j = 0; j < JMAX; ++j)
+            if (grp + j * GROUPS < nact) acc = fmaf(cv[j], w_lds[grp + j * GROUPS], acc);
+        sacc[grp * D + dd] = acc;  // sacc is free again: the wavefront states were consumed above
+    }
+    __syncthreads();
+    if (t < D) {
+        float acc = 0.f;
+#pragma unroll
+        for (int g = 0; g < GROUPS; ++g) acc += sacc[g * D + t];
+        out_head[t] = acc * w_lds[64];
+    }
+}
+
 // PRE: q arrives rotated and cache row `pos` is already written (both done by the q|k|v GEMV's
 // epilogue), so the kernel is only the row loop over [0, pos] and the merges.
+// Grid: x = NREP * nslices workgroups per KV head, y = KV head, z = batch.
 template <int D, int NREP, int WAVES, bool PRE>
 __global__ __launch_bounds__(WAVES * 64) void attn_decode_kernel(AttnDecodeArgs a) {
     typedef AttnGeom<D, WAVES> G;
-    constexpr int THREADS = WAVES * 64;
-    __shared__ __align__(16) float q_raw[NREP * D];
-    __shared__ __align__(16) float q_rot[NREP * D];
-    __shared__ __align__(16) float k_raw[D];
+    __shared__ __align__(16) float q_rot[D];
     __shared__ __align__(16) float k_new[D];
     __shared__ __align__(16) float v_new[D];
-    __shared__ __align__(16) float sacc[WAVES * NREP * D];
-    __shared__ float sm[WAVES * NREP], sl[WAVES * NREP];
+    // wavefront states [WAVES][D]; the fold of a long cache reuses it for one partial sum per thread
+    __shared__ __align__(16) float sacc[WAVES * (D > 64 ? D : 64)];
+    __shared__ float sm[WAVES], sl[WAVES], w_lds[65];
     __shared__ int s_last;
 
     const int split = blockIdx.x, hk = blockIdx.y, bb = blockIdx.z;
@@ -193,115 +382,42 @@ __global__ __launch_bounds__(WAVES * 64) void attn_decode_kernel(AttnDecodeArgs 
     // fetched into two L2s instead of eight.
     int r = split;
     if (NREP == 8 && gridDim.x >= 32 && (gridDim.x & 7) == 0) r = (split & 7) < 2 && split < 32 ? (split >> 3) + 4 * (split & 7) : NREP;
-    const bool short_fits = (int)gridDim.x >= NREP;
     // the caller expects a short cache: start the short form before the position is known
-    if (a.expect_short && short_fits && r < NREP &&
-        attn_decode_short<D, WAVES, PRE>(a, r, NREP, hk, bb, -1, SHORT_ROWS, q_raw, q_rot, k_raw, k_new, v_new, sm, sl, sacc))
+    if (a.expect_short && r < NREP &&
+        attn_decode_short<D, WAVES, PRE>(a, r, NREP, hk, bb, -1, SHORT_ROWS, q_rot, k_new, v_new, sm, sl, sacc))
         return;
     const int pos_new = a.pos_dev ? *a.pos_dev : a.pos_host;  // == past_len, the new token's position
     const int pos = PRE ? pos_new + 1 : pos_new;             // rows that come from the cache
-    if (pos_new + 1 <= SHORT_ROWS && short_fits) {
+    if (pos_new + 1 <= SHORT_ROWS) {
         if (r < NREP && !a.expect_short)
-            attn_decode_short<D, WAVES, PRE>(a, r, NREP, hk, bb, pos_new, SHORT_ROWS, q_raw, q_rot, k_raw, k_new, v_new, sm, sl, sacc);
+            attn_decode_short<D, WAVES, PRE>(a, r, NREP, hk, bb, pos_new, SHORT_ROWS, q_rot, k_new, v_new, sm, sl, sacc);
         return;
     }
-    int nact, chunk;
-    decode_slices<D, WAVES>(pos, gridDim.x, nact, chunk);
-    if (split >= nact) return;
-    const bool has_new = !PRE && (split == nact - 1);
-    const float *cs = a.cos_t + (size_t)pos_new * D, *sn = a.sin_t + (size_t)pos_new * D;
-    const size_t head_base = ((size_t)bb * a.hkv + hk) * a.max_seq * D;
-    const float *Kb = a.k_cache + head_base, *Vb = a.v_cache + head_base;
-
-    // this slice's share of the cached rows [0, pos); its first trip of K/V rows starts streaming
-    // before anything else: it does not depend on q
-    const int p0 = min(pos, split * chunk), p1 = min(pos, p0 + chunk);
-    v4f kv[G::U], vv[G::U];
-    attn_load_trip<D, WAVES>(Kb, Vb, p0, p1, kv, vv);
-
-    // stage raw q heads of this KV group (contiguous: hq = hk*NREP + r) and the new k / v
-    const float *q_src = a.q + ((size_t)bb * a.hq + (size_t)hk * NREP) * D;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int slot = lane / G::LPR, c = lane % G::LPR;
-    v4f q[NREP];
-    if (PRE) {
-        load_q_scaled<D, NREP>(q, q_src, c, a.scale);
+    // Long form: workgroup `split` takes query head rr over slice `slice`.  With 8 or more slices
+    // the heads of one (KV head, slice) sit 8 workgroups apart -- on one XCD -- so the slice's rows
+    // reach that XCD's L2 once for all of them.
+    const int nslices = (int)gridDim.x / NREP;  // a power of two
+    int slice, rr;
+    if (nslices >= 8) {
+        slice = (split & 7) | ((split / (8 * NREP)) << 3);
+        rr = (split >> 3) % NREP;
     } else {
-    for (int i = threadIdx.x; i < NREP * D; i += THREADS) q_raw[i] = q_src[i];
-    if (has_new) {
-        const float *k_src = a.k_new + ((size_t)bb * a.hkv + hk) * D;
-        const float *v_src = a.v_new + ((size_t)bb * a.hkv + hk) * D;
-        for (int i = threadIdx.x; i < D; i += THREADS) {
-            k_raw[i] = k_src[i];
-            v_new[i] = v_src[i];
-        }
+        slice = split % nslices;
+        rr = split / nslices;
     }
-    __syncthreads();
-    norm_rope_heads<D>(q_raw, q_rot, NREP, cs, sn, a.q_norm_w, a.norm_eps, THREADS);
-    if (has_new) norm_rope_heads<D>(k_raw, k_new, 1, cs, sn, a.k_norm_w, a.norm_eps, THREADS);
-    __syncthreads();
-    if (has_new) {
-        // self_attention.rs:161-176: rotated k and raw v go to cache row `pos`
-        for (int i = threadIdx.x; i < D; i += THREADS) {
-            a.k_cache[head_base + (size_t)pos * D + i] = k_new[i];
-            a.v_cache[head_base + (size_t)pos * D + i] = v_new[i];
-        }
-    }
-    load_q_scaled<D, NREP>(q, q_rot, c, a.scale);
-    }
-
-    AttnState<NREP> st;
-    state_init<NREP>(st);
-    if (p0 < p1) attn_compute_trip<D, NREP, WAVES>(st, q, kv, vv, p0, p1);
-    attn_rows<D, NREP, WAVES>(st, q, Kb, Vb, p0 + G::ROWS_PER_TRIP, p1);
-    if (has_new && wave == 0) {
-        // the new token's row comes from LDS (lane group 0 of wavefront 0)
-        const v4f kn = *(const v4f *)(k_new + c * 4);
-        const v4f vn = *(const v4f *)(v_new + c * 4);
-        attn_step<D, NREP>(st, q, kn, vn, slot == 0);
-    }
-
-    wave_merge_publish<D, NREP>(st, sm, sl, sacc);
-    __syncthreads();
-    const int t = threadIdx.x;
-    for (int e = t; e < NREP * D; e += THREADS) {
-        const int r = e / D, dd = e % D;
-        float mm, ls, cx;
-        wave_fold<D, NREP, WAVES>(sm, sl, sacc, r, dd, mm, ls, cx);
-        const int hq = hk * NREP + r;
-        if (nact == 1) {
-            // out = ctx / (l + 1e-9), self_attention.rs:287-290
-            a.out[((size_t)bb * a.hq + hq) * D + dd] = cx * (1.0f / (ls + 1e-9f));
-        } else {
-            float *pp = a.part + (((size_t)bb * a.hq + hq) * gridDim.x + split) * (D + 2);
-            part_store(pp + dd, cx);
-            if (dd == 0) {
-                part_store(pp + D, mm);
-                part_store(pp + D + 1, ls);
-            }
-        }
-    }
-    if (nact == 1) return;
-
-    // last workgroup of this (batch, KV head) to arrive folds the slices in index order.  The barrier
-    // makes every wavefront wait for its own stores before thread 0 signals.
-    __syncthreads();
-    if (t == 0) {
-        const int old = __hip_atomic_fetch_add(&a.counters[bb * a.hkv + hk], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_last = (old == nact - 1);
-        if (s_last) __hip_atomic_store(&a.counters[bb * a.hkv + hk], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __syncthreads();
-    if (!s_last) return;
-    // sacc is free again: slice weights [NREP][64] and the NREP reciprocals behind them
-    fold_slices_block<D, NREP, WAVES>(a.part + (((size_t)bb * a.hq + (size_t)hk * NREP) * gridDim.x) * (D + 2), gridDim.x, nact,
-                                      sacc, sacc + NREP * 64, a.out + ((size_t)bb * a.hq + (size_t)hk * NREP) * D);
+    int nact, chunk;
+    long_slices<D, WAVES>(pos, nslices, nact, chunk);
+    if (slice >= nact) return;
+    attn_decode_slice<D, WAVES, PRE>(a, rr, NREP, hk, bb, pos_new, slice, nact, chunk, nslices, q_rot, k_new, v_new, sm, sl,
+                                     sacc, w_lds, &s_last);
 }
 
-int attn_decode_nsplit(int max_seq) {
-    int n = max_seq / 64;
-    if (n < 1) n = 1;
-    if (n > 64) n = 64;
+// slices of a long cache: one trip of rows each (16384 / head_dim rows: eight 16-byte loads per lane,
+// 8 wavefronts), a power of two, 64 at most (the fold takes one slice per lane)
+int attn_decode_nsplit(int max_seq, int d) {
+    const int trip = 16384 / d;
+    int n = 1;
+    while (n < 64 && n * trip < max_seq) n *= 2;
     return n;
 }
 
@@ -309,8 +425,8 @@ size_t attn_decode_part_floats(int b, int hq, int d, int nsplit) { return (size_
 
 template <int D>
 static int launch_decode_d(lumen_ctx *ctx, const AttnDecodeArgs &a) {
-    dim3 grid(a.nsplit, a.hkv, a.b);
     const int nrep = a.hq / a.hkv;
+    dim3 grid(nrep * a.nsplit, a.hkv, a.b);
 #define LAUNCH_DECODE(NR)                                                                                     \
     do {                                                                                                      \
         if (a.pre_rotated)                                                                                    \
@@ -515,6 +631,13 @@ extern "C" int lumen_kv_cache_len(const lumen_kv_cache *c, int *len_out) {
     return LUMEN_OK;
 }
 
+extern "C" int lumen_kv_cache_set_len(lumen_kv_cache *c, int len) {
+    if (!c) LUMEN_FAIL(LUMEN_ERR_INVALID, "kv_cache_set_len: null");
+    if (len < 0 || len > c->max_seq) LUMEN_FAIL(LUMEN_ERR_KV_OVERFLOW, "kv_cache_set_len: %d outside [0, %d]", len, c->max_seq);
+    c->len = len;
+    return LUMEN_OK;
+}
+
 extern "C" int lumen_kv_cache_ptrs(const lumen_kv_cache *c, float **k_out, float **v_out) {
     if (!c || !k_out || !v_out) LUMEN_FAIL(LUMEN_ERR_INVALID, "kv_cache_ptrs: null");
     *k_out = c->k;
@@ -558,8 +681,8 @@ static int ensure_split_scratch(lumen_kv_cache *c, int hq, int nsplit) {
     c->part = nullptr;
     c->counters = nullptr;
     HIP_TRY(hipMalloc((void **)&c->part, sizeof(float) * attn_decode_part_floats(c->b, hq, c->d, nsplit)));
-    HIP_TRY(hipMalloc((void **)&c->counters, sizeof(int) * (size_t)c->b * c->h_kv));
-    HIP_TRY(hipMemsetAsync(c->counters, 0, sizeof(int) * (size_t)c->b * c->h_kv, c->ctx->stream));
+    HIP_TRY(hipMalloc((void **)&c->counters, sizeof(int) * (size_t)c->b * hq));
+    HIP_TRY(hipMemsetAsync(c->counters, 0, sizeof(int) * (size_t)c->b * hq, c->ctx->stream));
     c->part_heads = hq;
     return LUMEN_OK;
 }
@@ -575,7 +698,7 @@ extern "C" int lumen_attn_decode_f32(lumen_kv_cache *c, lumen_rope *rope, const 
         LUMEN_FAIL(LUMEN_ERR_KV_OVERFLOW, "KV cache overflow: new_len=%d > max_seq=%d", new_len, c->max_seq);
     if (past_len >= rope->max_seq)  // encoding.rs:176-181
         LUMEN_FAIL(LUMEN_ERR_ROPE_RANGE, "RoPE index out of range: pos %d >= max %d", past_len, rope->max_seq);
-    const int nsplit = attn_decode_nsplit(c->max_seq);
+    const int nsplit = attn_decode_nsplit(c->max_seq, c->d);
     LUMEN_TRY(ensure_split_scratch(c, h, nsplit));
     AttnDecodeArgs a = {};
     a.q = q3; a.k_new = k3; a.v_new = v3; a.out = out;

@@ -85,6 +85,52 @@ __device__ __forceinline__ void attn_step(AttnState<NREP> &st, const v4f (&q)[NR
     }
 }
 
+// UB rows per lane group at once for one query head: the UB scores first (independent dot products
+// and lane-group sums), then ONE online-softmax update for the batch -- one rescale of the running
+// state and one exponential per row, instead of two exponentials and a rescale per row.  Rows
+// whose bit in `valid` is clear get the weight exp2(-inf) = 0 (their loads were clamped to a row
+// inside the cache, so the values multiplied by that zero are finite).
+template <int D, int UB>
+__device__ __forceinline__ void attn_batch(AttnState<1> &st, const v4f &q, const v4f (&kv)[UB], const v4f (&vv)[UB],
+                                           unsigned valid) {
+    constexpr int LPR = D / 4;
+    float s[UB];
+#pragma unroll
+    for (int u = 0; u < UB; ++u) {
+        float d = q.x * kv[u].x;
+        d = fmaf(q.y, kv[u].y, d);
+        d = fmaf(q.z, kv[u].z, d);
+        d = fmaf(q.w, kv[u].w, d);
+        s[u] = d;
+    }
+    float mb = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < UB; ++u) {
+        s[u] = group_sum<LPR>(s[u]);
+        s[u] = (valid >> u) & 1u ? s[u] : -INFINITY;
+        mb = fmaxf(mb, s[u]);
+    }
+    const float m_new = fmaxf(st.m[0], mb);
+    if (m_new > -INFINITY) {
+        const float alpha = fast_exp2(st.m[0] - m_new);  // exp2(-inf) = 0 on the first batch
+        float l = st.l[0] * alpha;
+        v4f acc = st.acc[0];
+        acc.x *= alpha; acc.y *= alpha; acc.z *= alpha; acc.w *= alpha;
+#pragma unroll
+        for (int u = 0; u < UB; ++u) {
+            const float p = fast_exp2(s[u] - m_new);
+            l += p;
+            acc.x = fmaf(p, vv[u].x, acc.x);
+            acc.y = fmaf(p, vv[u].y, acc.y);
+            acc.z = fmaf(p, vv[u].z, acc.z);
+            acc.w = fmaf(p, vv[u].w, acc.w);
+        }
+        st.l[0] = l;
+        st.acc[0] = acc;
+        st.m[0] = m_new;
+    }
+}
+
 template <int D, int WAVES>
 struct AttnGeom {
     static constexpr int LPR = D / 4;            // lanes per row

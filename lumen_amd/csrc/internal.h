@@ -146,8 +146,8 @@ struct AttnDecodeArgs {
     const float *q_norm_w, *k_norm_w;  // per-head RMSNorm gains [D] or null
     float norm_eps;
     float *part;        // split scratch
-    int *counters;
-    int nsplit;
+    int *counters;      // one per (batch, query head), zero between launches
+    int nsplit;         // slices a long cache is cut into (attn_decode_nsplit)
     int pre_rotated;    // q is already rotated and row pos of the cache already written (fused QKV GEMV)
     int expect_short;   // hint: the cache is short (a few hundred rows); a wrong hint only costs time
 };
@@ -173,7 +173,7 @@ int launch_attn_prefill(lumen_ctx *ctx, const AttnPrefillArgs &a);
 bool attn_prefill_mfma_supported(const AttnPrefillArgs &a);
 int launch_attn_prefill_mfma(lumen_ctx *ctx, const AttnPrefillArgs &a);
 
-int attn_decode_nsplit(int max_seq);
+int attn_decode_nsplit(int max_seq, int d);
 size_t attn_decode_part_floats(int b, int hq, int d, int nsplit);
 
 void rope_tables_host(std::vector<float> &cos_t, std::vector<float> &sin_t, int dim, int max_seq, float theta);

@@ -43,7 +43,8 @@ struct lumen_llama {
     int *tok_hist = nullptr;  // [max_seq + 1]: greedy pick made at position p sits at index p + 1
     float *part = nullptr;
     int *counters = nullptr;
-    int nsplit = 1;
+    int nsplit = 1;     // slices of a long cache in the decode attention kernel
+    int pk_nsplit = 1;  // the same for the persistent kernel (its own slicing: 64 rows per slice, 64 at most)
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
     int graph_expect_short = 0;            // the hint the captured attention launches carry
@@ -176,10 +177,11 @@ extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg,
     M_TRY(dmalloc_t(m, &m->d_tok, 4));
     M_TRY(dmalloc_t(m, &m->d_pos, 4));
     M_TRY(dmalloc_t(m, &m->tok_hist, (size_t)cfg->max_seq_len + 1));
-    m->nsplit = attn_decode_nsplit(cfg->max_seq_len);
-    M_TRY(dmalloc_t(m, &m->part, attn_decode_part_floats(1, Hq, D, m->nsplit)));
-    M_TRY(dmalloc_t(m, &m->counters, (size_t)Hkv));
-    if (hipMemsetAsync(m->counters, 0, sizeof(int) * Hkv, ctx->stream) != hipSuccess ||
+    m->nsplit = attn_decode_nsplit(cfg->max_seq_len, D);
+    m->pk_nsplit = cfg->max_seq_len / 64 < 1 ? 1 : (cfg->max_seq_len / 64 > 64 ? 64 : cfg->max_seq_len / 64);
+    M_TRY(dmalloc_t(m, &m->part, attn_decode_part_floats(1, Hq, D, m->nsplit > m->pk_nsplit ? m->nsplit : m->pk_nsplit)));
+    M_TRY(dmalloc_t(m, &m->counters, (size_t)Hq));
+    if (hipMemsetAsync(m->counters, 0, sizeof(int) * Hq, ctx->stream) != hipSuccess ||
         hipMemsetAsync(m->d_tok, 0, 4 * sizeof(int), ctx->stream) != hipSuccess ||
         hipMemsetAsync(m->d_pos, 0, 4 * sizeof(int), ctx->stream) != hipSuccess ||
         hipStreamSynchronize(ctx->stream) != hipSuccess) {
@@ -521,7 +523,7 @@ static void fill_pk_args(const lumen_llama *m, PkArgs &a) {
     a.layers = m->pk_layers; a.n_layers = c.num_hidden_layers;
     a.H = c.hidden_size; a.I = c.intermediate_size; a.V = c.vocab_size; a.qd = m->qd; a.kvd = m->kvd;
     a.hq = c.num_attention_heads; a.hkv = c.num_key_value_heads; a.D = m->D; a.max_seq = c.max_seq_len;
-    a.nsplit = m->nsplit; a.eps = c.rms_norm_eps; a.scale = m->scale; a.w_bf16 = m->bf16;
+    a.nsplit = m->pk_nsplit; a.eps = c.rms_norm_eps; a.scale = m->scale; a.w_bf16 = m->bf16;
     a.embed = m->embed; a.lm_head = m->lm_head; a.final_norm = m->final_norm;
     a.cos_t = m->cos_dev; a.sin_t = m->sin_dev;
     a.x = m->x; a.h = m->h; a.qkv = m->qkv; a.attn = m->attn; a.act = m->act; a.logits = m->logits;

@@ -154,6 +154,10 @@ class KVCacheInner:
         check(lib.lumen_kv_cache_len(self.handle, C.byref(n)))
         return n.value
 
+    @len.setter
+    def len(self, n):  # a public field in the reference (self_attention.rs:28)
+        check(lib.lumen_kv_cache_set_len(self.handle, int(n)))
+
     def reset(self):
         check(lib.lumen_kv_cache_reset(self.handle))
 

@@ -66,6 +66,46 @@ def test_decode_steps_match_oracle(h, h_kv, d, max_seq, prefill, steps):
     assert not g.k[:, :, n:].any() and not g.v[:, :, n:].any()  # untouched rows stay zero
 
 
+@pytest.mark.parametrize("h,h_kv,d,max_seq,filled,steps", [
+    (32, 4, 64, 4096, 3990, 3),     # the long-context benchmark shape: 16 slices, heads of a slice grouped per XCD
+    (16, 8, 128, 2048, 1500, 3),    # head_dim 128, n_rep 2: 12 of 16 slices in use
+    (32, 32, 128, 1024, 700, 2),    # one query head per KV head
+    (8, 2, 16, 4096, 3000, 2),      # head_dim 16: 1024 rows per slice, 4 slices (the ungrouped placement)
+    (4, 1, 64, 640, 520, 3),        # 3 of 4 slices in use
+    (2, 1, 128, 16384, 9000, 2),    # longer than 64 slices of one trip: two trips per slice
+    (8, 1, 32, 40000, 36000, 2),    # 64 slices of 576 rows; n_rep 8
+], ids=["d64-nrep8-4096", "d128-nrep2", "d128-mha", "d16", "d64-nrep4-short-tail", "d128-two-trips", "d32-64-slices"])
+def test_decode_over_a_long_cache_filled_directly(h, h_kv, d, max_seq, filled, steps):
+    """Decode attention over caches of thousands of rows: the rows are written straight into both caches
+    (lumen_kv_cache_update + lumen_kv_cache_set_len here, the arrays there), so no quadratic prompt pass is needed."""
+    scale = 1.0 / math.sqrt(d)
+    rope = RotaryEmbedding(d, max_seq, 10000.0)
+    cos, sin = lo.rope_table(d, max_seq, 10000.0)
+    g, o = KVCacheInner(1, h_kv, max_seq, d), lo.KVCache(1, h_kv, max_seq, d)
+    k0 = f32(RNG.normal(0, 1, (1, h_kv, filled, d)))
+    v0 = f32(RNG.normal(0, 1, (1, h_kv, filled, d)))
+    kd, vd = dev(k0), dev(v0)
+    check(lib.lumen_kv_cache_update(g.handle, kd.ptr, vd.ptr, filled, 0))
+    g.len = filled
+    o.k[:, :, :filled] = k0
+    o.v[:, :, :filled] = v0
+    o._c.contents.len = filled
+    for t in range(steps):
+        q = f32(RNG.normal(0, 1, (1, h, d)))
+        k = f32(RNG.normal(0, 1, (1, h_kv, d)))
+        v = f32(RNG.normal(0, 1, (1, h_kv, d)))
+        got = gpu_decode(g, rope, q, k, v, h, scale)
+        rc, ref = lo.attn_decode(o, q, k, v, cos, sin, scale)
+        assert rc == lo.LO_OK
+        assert max_rel(got, ref) <= TOL, (t, max_rel(got, ref))
+        assert g.len == o.len == filled + t + 1
+    n = filled + steps
+    assert np.array_equal(g.k[:, :, filled:n], o.k[:, :, filled:n]) and np.array_equal(g.v[:, :, filled:n], o.v[:, :, filled:n])
+    with pytest.raises(_lib.LumenError) as e:
+        g.len = max_seq + 1
+    assert e.value.status == _lib.ERR_KV_OVERFLOW
+
+
 def test_decode_degenerate_and_gqa_mapping():
     h, h_kv, d, max_seq = 8, 2, 64, 128
     rope = RotaryEmbedding(d, max_seq, 10000.0)
