@@ -45,6 +45,22 @@ template <int D>
 struct ShortTrip {
     static constexpr int loads = 8;
 };
+// 16 bytes of row j of one KV head: a uniform base pointer and a 32-bit byte offset (a head of the
+// cache stays below 4 GiB; the launcher checks), so that a row costs one address register
+template <int D>
+__device__ __forceinline__ v4f ld_row(const float *head, int j, unsigned c4) {
+    return *(const v4f *)((const char *)head + ((unsigned)j * D + c4) * 4u);
+}
+
+// bit u set: row first + u * stride lies before `end`
+template <int UB>
+__device__ __forceinline__ unsigned rows_mask(int first, int stride, int end) {
+    unsigned m = 0;
+#pragma unroll
+    for (int u = 0; u < UB; ++u) m |= (first + u * stride < end ? 1u : 0u) << u;
+    return m;
+}
+
 // PRE: q is rotated and cache row pos_new written already; otherwise this workgroup normalises and
 // rotates its own query head and the group's new key itself (a few hundred flops, repeated by
 // every head of the group so that nothing has to be exchanged), the first head of the group
@@ -63,7 +79,9 @@ __device__ __forceinline__ bool attn_decode_short(const AttnDecodeArgs &a, int r
     const int off = wave * RPW + lane / LPR, c = lane % LPR;
     const int hq = hk * nrep + r;
     const size_t head_base = ((size_t)bb * a.hkv + hk) * a.max_seq * D;
-    const float *Kb = a.k_cache + head_base + c * 4, *Vb = a.v_cache + head_base + c * 4;
+    // uniform head pointers plus one 32-bit element offset per row, shared by the K and the V load
+    const float *Kb = a.k_cache + head_base, *Vb = a.v_cache + head_base;
+    const unsigned c4 = c * 4;
     AttnState<1> st;
     state_init<1>(st);
     v4f q[1];
@@ -73,8 +91,8 @@ __device__ __forceinline__ bool attn_decode_short(const AttnDecodeArgs &a, int r
 #pragma unroll
     for (int u = 0; u < UB; ++u) {
         const int j = min(u * RPI + off, a.max_seq - 1);
-        kv0[u] = *(const v4f *)(Kb + (size_t)j * D);
-        vv0[u] = *(const v4f *)(Vb + (size_t)j * D);
+        kv0[u] = ld_row<D>(Kb, j, c4);
+        vv0[u] = ld_row<D>(Vb, j, c4);
     }
     if (PRE) {
         load_q_scaled<D, 1>(q, a.q + ((size_t)bb * a.hq + hq) * D, c, a.scale);
@@ -140,20 +158,16 @@ __device__ __forceinline__ bool attn_decode_short(const AttnDecodeArgs &a, int r
         have_q = true;
     };
     if (!have_q && pos > 0) get_q();
-#pragma unroll
-    for (int u = 0; u < UB; ++u)
-        if (u * RPI < pos) attn_step<D, 1>(st, q, kv0[u], vv0[u], u * RPI + off < pos);
+    attn_batch<D, UB>(st, q[0], kv0, vv0, rows_mask<UB>(off, RPI, pos));
     for (int base = RPI * UB; base < pos; base += RPI * UB) {
         v4f kv[UB], vv[UB];
 #pragma unroll
-        for (int u = 0; u < UB; ++u) {  // rows past the end are clamped here and masked in attn_step
+        for (int u = 0; u < UB; ++u) {  // rows past the end are clamped here and masked in attn_batch
             const int j = min(base + u * RPI + off, pos - 1);
-            kv[u] = *(const v4f *)(Kb + (size_t)j * D);
-            vv[u] = *(const v4f *)(Vb + (size_t)j * D);
+            kv[u] = ld_row<D>(Kb, j, c4);
+            vv[u] = ld_row<D>(Vb, j, c4);
         }
-#pragma unroll
-        for (int u = 0; u < UB; ++u)
-            if (base + u * RPI < pos) attn_step<D, 1>(st, q, kv[u], vv[u], base + u * RPI + off < pos);
+        attn_batch<D, UB>(st, q[0], kv, vv, rows_mask<UB>(base + off, RPI, pos));
     }
     if (!PRE) {
         if (!have_q) get_q();  // empty cache: the new token attends to itself only
@@ -191,28 +205,50 @@ __device__ __forceinline__ void long_slices(int pos, int nslices, int &nact, int
 // query head; the last slice also rotates the new key, takes the new row from LDS, and its first
 // head stores the row into the cache (self_attention.rs:161-176).
 template <int D, int WAVES, bool PRE>
-__device__ __forceinline__ void attn_decode_slice(const AttnDecodeArgs &a, int r, int nrep, int hk, int bb, int pos_new,
-                                                  int slice, int nact, int chunk, int nslices, float *q_rot,
+__device__ __forceinline__ bool attn_decode_slice(const AttnDecodeArgs &a, int r, int nrep, int hk, int bb, int pos_new,
+                                                  int slice, int nslices, bool fixed, int short_rows, float *q_rot,
                                                   float *k_new, float *v_new, float *sm, float *sl, float *sacc,
                                                   float *w_lds, int *s_last) {
     constexpr int LPR = D / 4, RPW = 64 / LPR, RPI = WAVES * RPW, UB = ShortTrip<D>::loads, THREADS = WAVES * 64;
-    constexpr int GROUPS = THREADS / D, JMAX = (64 + GROUPS - 1) / GROUPS;
+    constexpr int TRIP = RPI * UB, GROUPS = THREADS / D, JMAX = (64 + GROUPS - 1) / GROUPS;
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int off = wave * RPW + lane / LPR, c = lane % LPR;
     const int hq = hk * nrep + r;
-    const int pos = PRE ? pos_new + 1 : pos_new;  // rows read from the cache
+    const size_t head_base = ((size_t)bb * a.hkv + hk) * a.max_seq * D;
+    // uniform head pointers plus one 32-bit element offset per row, shared by the K and the V load
+    const float *Kb = a.k_cache + head_base, *Vb = a.v_cache + head_base;
+    const unsigned c4 = c * 4;
+    // first trip of rows: requested before anything else, it does not depend on q -- nor, with fixed
+    // slices, on the position: a row past the cached ones is only masked later
+    v4f kv0[UB], vv0[UB];
+    int nact = 0, chunk = TRIP, pos = 0;
+    if (pos_new >= 0) {
+        pos = PRE ? pos_new + 1 : pos_new;
+        if (fixed) nact = max(1, (pos + TRIP - 1) / TRIP);
+        else long_slices<D, WAVES>(pos, nslices, nact, chunk);
+        if (slice >= nact) return true;
+        const int first = min(pos, slice * chunk), last = min(pos, first + chunk) - 1;
+#pragma unroll
+        for (int u = 0; u < UB; ++u) {
+            const int j = max(min(first + u * RPI + off, last), 0);
+            kv0[u] = ld_row<D>(Kb, j, c4);
+            vv0[u] = ld_row<D>(Vb, j, c4);
+        }
+    } else {
+#pragma unroll
+        for (int u = 0; u < UB; ++u) {
+            const int j = min(slice * TRIP + u * RPI + off, a.max_seq - 1);
+            kv0[u] = ld_row<D>(Kb, j, c4);
+            vv0[u] = ld_row<D>(Vb, j, c4);
+        }
+        pos_new = *a.pos_dev;
+        if (pos_new + 1 <= short_rows) return false;
+        pos = PRE ? pos_new + 1 : pos_new;
+        nact = max(1, (pos + TRIP - 1) / TRIP);
+        if (slice >= nact) return true;
+    }
     const int p0 = min(pos, slice * chunk), p1 = min(pos, p0 + chunk);
     const bool has_new = !PRE && slice == nact - 1;
-    const size_t head_base = ((size_t)bb * a.hkv + hk) * a.max_seq * D;
-    const float *Kb = a.k_cache + head_base + c * 4, *Vb = a.v_cache + head_base + c * 4;
-    // first trip of rows: requested before anything else, it does not depend on q
-    v4f kv0[UB], vv0[UB];
-#pragma unroll
-    for (int u = 0; u < UB; ++u) {
-        const int j = max(min(p0 + u * RPI + off, p1 - 1), 0);
-        kv0[u] = *(const v4f *)(Kb + (size_t)j * D);
-        vv0[u] = *(const v4f *)(Vb + (size_t)j * D);
-    }
     v4f q[1];
     if (PRE) {
         load_q_scaled<D, 1>(q, a.q + ((size_t)bb * a.hq + hq) * D, c, a.scale);
@@ -269,20 +305,16 @@ __device__ __forceinline__ void attn_decode_slice(const AttnDecodeArgs &a, int r
     }
     AttnState<1> st;
     state_init<1>(st);
-#pragma unroll
-    for (int u = 0; u < UB; ++u)
-        if (p0 + u * RPI < p1) attn_step<D, 1>(st, q, kv0[u], vv0[u], p0 + u * RPI + off < p1);
+    attn_batch<D, UB>(st, q[0], kv0, vv0, rows_mask<UB>(p0 + off, RPI, p1));
     for (int base = p0 + RPI * UB; base < p1; base += RPI * UB) {  // caches longer than nslices trips
         v4f kv[UB], vv[UB];
 #pragma unroll
         for (int u = 0; u < UB; ++u) {
             const int j = min(base + u * RPI + off, p1 - 1);
-            kv[u] = *(const v4f *)(Kb + (size_t)j * D);
-            vv[u] = *(const v4f *)(Vb + (size_t)j * D);
+            kv[u] = ld_row<D>(Kb, j, c4);
+            vv[u] = ld_row<D>(Vb, j, c4);
         }
-#pragma unroll
-        for (int u = 0; u < UB; ++u)
-            if (base + u * RPI < p1) attn_step<D, 1>(st, q, kv[u], vv[u], base + u * RPI + off < p1);
+        attn_batch<D, UB>(st, q[0], kv, vv, rows_mask<UB>(base + off, RPI, p1));
     }
     if (has_new && wave == 0) {  // the new row, from LDS (lane group 0 of wavefront 0)
         const v4f kn = *(const v4f *)(k_new + c * 4), vn = *(const v4f *)(v_new + c * 4);
@@ -306,7 +338,7 @@ __device__ __forceinline__ void attn_decode_slice(const AttnDecodeArgs &a, int r
             }
         }
     }
-    if (nact == 1) return;
+    if (nact == 1) return true;
     // The barrier makes every wavefront wait for its own stores before thread 0 signals.
     __syncthreads();
     if (t == 0) {
@@ -316,7 +348,7 @@ __device__ __forceinline__ void attn_decode_slice(const AttnDecodeArgs &a, int r
         if (*s_last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
-    if (!*s_last) return;
+    if (!*s_last) return true;
     // fold: context partials of this thread's element and slices first (one trip to memory) ...
     const int dd = t % D, grp = t / D;
     float cv[JMAX];
@@ -357,13 +389,14 @@ __device__ __forceinline__ void attn_decode_slice(const AttnDecodeArgs &a, int r
         for (int g = 0; g < GROUPS; ++g) acc += sacc[g * D + t];
         out_head[t] = acc * w_lds[64];
     }
+    return true;
 }
 
 // PRE: q arrives rotated and cache row `pos` is already written (both done by the q|k|v GEMV's
 // epilogue), so the kernel is only the row loop over [0, pos] and the merges.
 // Grid: x = NREP * nslices workgroups per KV head, y = KV head, z = batch.
 template <int D, int NREP, int WAVES, bool PRE>
-__global__ __launch_bounds__(WAVES * 64) void attn_decode_kernel(AttnDecodeArgs a) {
+__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void attn_decode_kernel(AttnDecodeArgs a) {
     typedef AttnGeom<D, WAVES> G;
     __shared__ __align__(16) float q_rot[D];
     __shared__ __align__(16) float k_new[D];
@@ -382,17 +415,6 @@ __global__ __launch_bounds__(WAVES * 64) void attn_decode_kernel(AttnDecodeArgs 
     // fetched into two L2s instead of eight.
     int r = split;
     if (NREP == 8 && gridDim.x >= 32 && (gridDim.x & 7) == 0) r = (split & 7) < 2 && split < 32 ? (split >> 3) + 4 * (split & 7) : NREP;
-    // the caller expects a short cache: start the short form before the position is known
-    if (a.expect_short && r < NREP &&
-        attn_decode_short<D, WAVES, PRE>(a, r, NREP, hk, bb, -1, SHORT_ROWS, q_rot, k_new, v_new, sm, sl, sacc))
-        return;
-    const int pos_new = a.pos_dev ? *a.pos_dev : a.pos_host;  // == past_len, the new token's position
-    const int pos = PRE ? pos_new + 1 : pos_new;             // rows that come from the cache
-    if (pos_new + 1 <= SHORT_ROWS) {
-        if (r < NREP && !a.expect_short)
-            attn_decode_short<D, WAVES, PRE>(a, r, NREP, hk, bb, pos_new, SHORT_ROWS, q_rot, k_new, v_new, sm, sl, sacc);
-        return;
-    }
     // Long form: workgroup `split` takes query head rr over slice `slice`.  With 8 or more slices
     // the heads of one (KV head, slice) sit 8 workgroups apart -- on one XCD -- so the slice's rows
     // reach that XCD's L2 once for all of them.
@@ -405,15 +427,39 @@ __global__ __launch_bounds__(WAVES * 64) void attn_decode_kernel(AttnDecodeArgs 
         slice = split % nslices;
         rr = split / nslices;
     }
-    int nact, chunk;
-    long_slices<D, WAVES>(pos, nslices, nact, chunk);
-    if (slice >= nact) return;
-    attn_decode_slice<D, WAVES, PRE>(a, rr, NREP, hk, bb, pos_new, slice, nact, chunk, nslices, q_rot, k_new, v_new, sm, sl,
-                                     sacc, w_lds, &s_last);
+    // slices of exactly one trip wherever the whole cache fits into nslices of them; then a
+    // workgroup's rows do not depend on the position and are requested before it is read
+    const bool fixed = a.max_seq <= nslices * ShortTrip<D>::loads * G::RPI;
+
+    // The form follows the position where it is known (pos_host), the caller's hint where it sits in
+    // device memory: then the hinted form starts before the position is read and hands over to the
+    // other one if the hint was wrong.  One call site per form: two would let the compiler keep the
+    // first one's loaded rows alive for the second across everything in between.
+    int pos_new = a.pos_dev ? -1 : a.pos_host;  // == past_len, the new token's position
+    bool want_short = pos_new >= 0 ? pos_new + 1 <= SHORT_ROWS : a.expect_short != 0;
+#pragma unroll 1
+    for (int attempt = 0; attempt < 2; ++attempt) {
+        if (want_short) {
+            if (r < NREP && attn_decode_short<D, WAVES, PRE>(a, r, NREP, hk, bb, pos_new, SHORT_ROWS, q_rot, k_new, v_new, sm, sl, sacc))
+                return;
+            if (pos_new < 0) pos_new = *a.pos_dev;
+            if (pos_new + 1 <= SHORT_ROWS) return;  // short indeed: not one of the short form's workgroups
+            want_short = false;
+        } else {
+            if (pos_new < 0 && !fixed) pos_new = *a.pos_dev;
+            if (pos_new >= 0 && pos_new + 1 <= SHORT_ROWS) {
+                want_short = true;
+                continue;
+            }
+            if (attn_decode_slice<D, WAVES, PRE>(a, rr, NREP, hk, bb, pos_new, slice, nslices, fixed, SHORT_ROWS, q_rot, k_new,
+                                                 v_new, sm, sl, sacc, w_lds, &s_last))
+                return;
+            pos_new = *a.pos_dev;  // the slice form found a short cache
+            want_short = true;
+        }
+    }
 }
 
-// slices of a long cache: one trip of rows each (16384 / head_dim rows: eight 16-byte loads per lane,
-// 8 wavefronts), a power of two, 64 at most (the fold takes one slice per lane)
 int attn_decode_nsplit(int max_seq, int d) {
     const int trip = 16384 / d;
     int n = 1;

@@ -110,25 +110,27 @@ __device__ __forceinline__ void attn_batch(AttnState<1> &st, const v4f &q, const
         s[u] = (valid >> u) & 1u ? s[u] : -INFINITY;
         mb = fmaxf(mb, s[u]);
     }
+    // no branch around the update (the compiler would sink the V loads into it, behind the wait for
+    // the K rows): while nothing valid has been seen, m_new = -inf and every weight below is
+    // exp2(-inf - 0) = 0
     const float m_new = fmaxf(st.m[0], mb);
-    if (m_new > -INFINITY) {
-        const float alpha = fast_exp2(st.m[0] - m_new);  // exp2(-inf) = 0 on the first batch
-        float l = st.l[0] * alpha;
-        v4f acc = st.acc[0];
-        acc.x *= alpha; acc.y *= alpha; acc.z *= alpha; acc.w *= alpha;
+    const float m_ref = m_new > -INFINITY ? m_new : 0.f;
+    const float alpha = fast_exp2(st.m[0] - m_ref);  // exp2(-inf) = 0 on the first batch
+    float l = st.l[0] * alpha;
+    v4f acc = st.acc[0];
+    acc.x *= alpha; acc.y *= alpha; acc.z *= alpha; acc.w *= alpha;
 #pragma unroll
-        for (int u = 0; u < UB; ++u) {
-            const float p = fast_exp2(s[u] - m_new);
-            l += p;
-            acc.x = fmaf(p, vv[u].x, acc.x);
-            acc.y = fmaf(p, vv[u].y, acc.y);
-            acc.z = fmaf(p, vv[u].z, acc.z);
-            acc.w = fmaf(p, vv[u].w, acc.w);
-        }
-        st.l[0] = l;
-        st.acc[0] = acc;
-        st.m[0] = m_new;
+    for (int u = 0; u < UB; ++u) {
+        const float p = fast_exp2(s[u] - m_ref);
+        l += p;
+        acc.x = fmaf(p, vv[u].x, acc.x);
+        acc.y = fmaf(p, vv[u].y, acc.y);
+        acc.z = fmaf(p, vv[u].z, acc.z);
+        acc.w = fmaf(p, vv[u].w, acc.w);
     }
+    st.l[0] = l;
+    st.acc[0] = acc;
+    st.m[0] = m_new;
 }
 
 template <int D, int WAVES>
