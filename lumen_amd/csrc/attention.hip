@@ -28,7 +28,7 @@
 // WAVES wavefronts per workgroup: 8, i.e. one trip covers 128 rows of D = 64; the step is ALU-bound
 // (scores, exponentials and weighted sums for n_rep heads per row), so slices are kept short and
 // spread over many compute units rather than packed into few large workgroups.
-template <int D, int NREP>
+template <int D>
 struct DecodeWaves {
     static constexpr int value = 8;
 };
@@ -394,8 +394,9 @@ __device__ __forceinline__ bool attn_decode_slice(const AttnDecodeArgs &a, int r
 
 // PRE: q arrives rotated and cache row `pos` is already written (both done by the q|k|v GEMV's
 // epilogue), so the kernel is only the row loop over [0, pos] and the merges.
-// Grid: x = NREP * nslices workgroups per KV head, y = KV head, z = batch.
-template <int D, int NREP, int WAVES, bool PRE>
+// Grid: x = n_rep * nslices workgroups per KV head, y = KV head, z = batch.  NREP_T: the group size
+// n_rep where it is one of the common ones (index arithmetic with constants), 0 for any other.
+template <int D, int NREP_T, int WAVES, bool PRE>
 __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void attn_decode_kernel(AttnDecodeArgs a) {
     typedef AttnGeom<D, WAVES> G;
     __shared__ __align__(16) float q_rot[D];
@@ -407,12 +408,13 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
     __shared__ int s_last;
 
     const int split = blockIdx.x, hk = blockIdx.y, bb = blockIdx.z;
+    const int NREP = NREP_T ? NREP_T : a.hq / a.hkv;  // query heads per KV head
     // the short form walks the rows in trips, one after the other: two trips at most
     constexpr int SHORT_ROWS = (2 * ShortTrip<D>::loads * G::RPI < ATTN_SHORT_ROWS) ? 2 * ShortTrip<D>::loads * G::RPI : ATTN_SHORT_ROWS;
     // Short form: workgroup `split` takes query head r of the group.  Workgroups are dealt
     // round-robin over the 8 XCDs, each with an L2 of its own; with 32 or more workgroups per KV
     // head the heads of a group are placed 8 apart, four to an XCD, so that a group's K/V rows are
-    // fetched into two L2s instead of eight.
+    // fetched into two L2s instead of eight (that placement is for groups of eight heads).
     int r = split;
     if (NREP == 8 && gridDim.x >= 32 && (gridDim.x & 7) == 0) r = (split & 7) < 2 && split < 32 ? (split >> 3) + 4 * (split & 7) : NREP;
     // Long form: workgroup `split` takes query head rr over slice `slice`.  With 8 or more slices
@@ -460,6 +462,8 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
     }
 }
 
+// slices of a long cache: one trip of rows each (16384 / head_dim rows: eight 16-byte loads per lane,
+// 8 wavefronts), a power of two, 64 at most (the fold takes one slice per lane)
 int attn_decode_nsplit(int max_seq, int d) {
     const int trip = 16384 / d;
     int n = 1;
@@ -471,23 +475,24 @@ size_t attn_decode_part_floats(int b, int hq, int d, int nsplit) { return (size_
 
 template <int D>
 static int launch_decode_d(lumen_ctx *ctx, const AttnDecodeArgs &a) {
+    constexpr int WAVES = DecodeWaves<D>::value;
     const int nrep = a.hq / a.hkv;
     dim3 grid(nrep * a.nsplit, a.hkv, a.b);
-#define LAUNCH_DECODE(NR)                                                                                     \
-    do {                                                                                                      \
-        if (a.pre_rotated)                                                                                    \
-            hipLaunchKernelGGL((attn_decode_kernel<D, NR, DecodeWaves<D, NR>::value, true>), grid,            \
-                               dim3(DecodeWaves<D, NR>::value * 64), 0, ctx->stream, a);                      \
-        else                                                                                                  \
-            hipLaunchKernelGGL((attn_decode_kernel<D, NR, DecodeWaves<D, NR>::value, false>), grid,           \
-                               dim3(DecodeWaves<D, NR>::value * 64), 0, ctx->stream, a);                      \
+    if ((size_t)a.max_seq * D * sizeof(float) >= ((size_t)1 << 32))  // 32-bit byte offsets inside a head
+        LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "decode attention: a KV head of %d rows x %d exceeds 4 GiB", a.max_seq, D);
+#define LAUNCH_DECODE(NR)                                                                                          \
+    do {                                                                                                           \
+        if (a.pre_rotated)                                                                                         \
+            hipLaunchKernelGGL((attn_decode_kernel<D, NR, WAVES, true>), grid, dim3(WAVES * 64), 0, ctx->stream, a);  \
+        else                                                                                                       \
+            hipLaunchKernelGGL((attn_decode_kernel<D, NR, WAVES, false>), grid, dim3(WAVES * 64), 0, ctx->stream, a); \
     } while (0)
     switch (nrep) {
         case 1: LAUNCH_DECODE(1); break;
         case 2: LAUNCH_DECODE(2); break;
         case 4: LAUNCH_DECODE(4); break;
         case 8: LAUNCH_DECODE(8); break;
-        default: LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "decode attention: n_rep=%d (supported 1, 2, 4, 8)", nrep);
+        default: LAUNCH_DECODE(0); break;
     }
 #undef LAUNCH_DECODE
     LUMEN_CHECK_LAUNCH();
@@ -553,11 +558,12 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_prefill_kernel(AttnPrefillAr
     typedef AttnGeom<D, ATT_WAVES> G;
     __shared__ __align__(16) float sacc[ATT_WAVES * NREP * D];
     __shared__ float sm[ATT_WAVES * NREP], sl[ATT_WAVES * NREP];
+    // blockIdx.y: KV head, or (NREP == 1 with a.kv_div = n_rep) query head of KV head blockIdx.y / n_rep
     const int i = blockIdx.x, hk = blockIdx.y, bb = blockIdx.z;
     const int L = a.past_len + a.s;
     const int q_abs = a.past_len + i;
     const int p1 = a.causal ? min(L, q_abs + 1) : L;
-    const size_t head_base = ((size_t)bb * a.hkv + hk) * a.max_seq * D;
+    const size_t head_base = ((size_t)bb * a.hkv + hk / a.kv_div) * a.max_seq * D;
     const int c = (threadIdx.x & 63) % G::LPR;
     const float *qr = a.q_rot + (((size_t)bb * a.s + i) * a.hq + (size_t)hk * NREP) * D;
     v4f q[NREP];
@@ -587,13 +593,19 @@ static int launch_prefill_d(lumen_ctx *ctx, const AttnPrefillArgs &a) {
         case 2: hipLaunchKernelGGL((attn_prefill_kernel<D, 2>), grid, block, 0, ctx->stream, a); break;
         case 4: hipLaunchKernelGGL((attn_prefill_kernel<D, 4>), grid, block, 0, ctx->stream, a); break;
         case 8: hipLaunchKernelGGL((attn_prefill_kernel<D, 8>), grid, block, 0, ctx->stream, a); break;
-        default: LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "prefill attention: n_rep=%d (supported 1, 2, 4, 8)", nrep);
+        default: {  // any other group size: one query head per workgroup, its KV head = head / n_rep
+            AttnPrefillArgs b = a;
+            b.kv_div = nrep;
+            hipLaunchKernelGGL((attn_prefill_kernel<D, 1>), dim3(a.s, a.hq, a.b), block, 0, ctx->stream, b);
+        }
     }
     LUMEN_CHECK_LAUNCH();
     return LUMEN_OK;
 }
 
-int launch_attn_prefill(lumen_ctx *ctx, const AttnPrefillArgs &a) {
+int launch_attn_prefill(lumen_ctx *ctx, const AttnPrefillArgs &a_in) {
+    AttnPrefillArgs a = a_in;
+    a.kv_div = 1;
     if (a.hkv <= 0 || a.hq % a.hkv) LUMEN_FAIL(LUMEN_ERR_SHAPE, "heads %d not a multiple of kv heads %d", a.hq, a.hkv);
     if (a.s <= 0) return LUMEN_OK;
     switch (a.d) {

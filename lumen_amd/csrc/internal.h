@@ -164,6 +164,7 @@ struct AttnPrefillArgs {
     int q_stride, k_stride, v_stride;  // floats between consecutive positions
     float scale;
     int causal;
+    int kv_div;  // set by the launcher: KV head of grid row y is y / kv_div (1 unless one query head per row)
     const float *q_norm_w, *k_norm_w;
     float norm_eps;
     float *q_rot;    // scratch [B, S, Hq, D]

@@ -108,8 +108,9 @@ extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg,
         LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_create: weight_dtype %d", cfg->weight_dtype);
     const int D = cfg->head_dim > 0 ? cfg->head_dim : H / Hq;
     const int nrep = Hq / Hkv;
-    if (!(D == 16 || D == 32 || D == 64 || D == 128) || !(nrep == 1 || nrep == 2 || nrep == 4 || nrep == 8))
-        LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "head_dim %d / n_rep %d outside the attention kernels (16..128, 1..8)", D, nrep);
+    if (!(D == 16 || D == 32 || D == 64 || D == 128))
+        LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "head_dim %d outside the attention kernels (16, 32, 64, 128)", D);
+    (void)nrep;
     if (H % 8 || I % 8 || (Hq * D) % 8)
         LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "hidden %d, intermediate %d and n_head*head_dim %d must be multiples of 8", H, I, Hq * D);
     if (H > 16384 || I > 16384 || Hq * D > 16384)

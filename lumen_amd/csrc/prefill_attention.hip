@@ -62,7 +62,7 @@ __global__ __launch_bounds__(FA_THREADS) void attn_prefill_mfma_kernel(AttnPrefi
     // workgroups are dealt in index order: the blocks of late positions (most keys) go first
     const int q0 = (int)(gridDim.x - 1 - blockIdx.x) * BQ, hk = blockIdx.y, bb = blockIdx.z;
     const int L = a.past_len + a.s;
-    const size_t head_base = ((size_t)bb * a.hkv + hk) * a.max_seq * D;
+    const size_t head_base = ((size_t)bb * a.hkv + hk / a.kv_div) * a.max_seq * D;  // kv_div > 1: grid row = query head
     const float *Kc = a.k_cache + head_base, *Vc = a.v_cache + head_base;
 
     // accumulator register r of lane l belongs to row 8*(r/4) + 4*(l/32) + r%4 of the wavefront's 32
@@ -205,7 +205,12 @@ static int launch_fa_d(lumen_ctx *ctx, const AttnPrefillArgs &a) {
         case 2: LAUNCH_FA(2); break;
         case 4: LAUNCH_FA(4); break;
         case 8: LAUNCH_FA(8); break;
-        default: LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "prefill attention: n_rep=%d (supported 1, 2, 4, 8)", nrep);
+        default: {  // any other group size: one query head per grid row, its KV head = head / n_rep
+            AttnPrefillArgs b = a;
+            b.kv_div = nrep;
+            hipLaunchKernelGGL((attn_prefill_mfma_kernel<D, 1>), dim3((a.s + FA_ROWS - 1) / FA_ROWS, a.hq, a.b), block, 0,
+                               ctx->stream, b);
+        }
     }
 #undef LAUNCH_FA
     LUMEN_CHECK_LAUNCH();

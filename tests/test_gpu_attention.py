@@ -39,7 +39,8 @@ def gpu_prefill(cache, rope, q, k, v, scale):
 
 @pytest.mark.parametrize("h,h_kv,d,max_seq,prefill,steps", [
     (32, 4, 64, 2048, 0, 40), (32, 4, 64, 2048, 300, 6), (16, 8, 128, 512, 100, 5), (32, 32, 128, 256, 61, 4),
-    (8, 2, 16, 64, 0, 64), (8, 1, 32, 4096, 4000, 3), (2, 2, 64, 32, 1, 3)])
+    (8, 2, 16, 64, 0, 64), (8, 1, 32, 4096, 4000, 3), (2, 2, 64, 32, 1, 3),
+    (6, 2, 64, 640, 250, 4), (28, 4, 128, 1024, 300, 3), (5, 1, 32, 64, 0, 6)])  # group sizes 3, 7, 5
 def test_decode_steps_match_oracle(h, h_kv, d, max_seq, prefill, steps):
     scale = 1.0 / math.sqrt(d)
     rope = RotaryEmbedding(d, max_seq, 10000.0)
@@ -74,7 +75,10 @@ def test_decode_steps_match_oracle(h, h_kv, d, max_seq, prefill, steps):
     (4, 1, 64, 640, 520, 3),        # 3 of 4 slices in use
     (2, 1, 128, 16384, 9000, 2),    # longer than 64 slices of one trip: two trips per slice
     (8, 1, 32, 40000, 36000, 2),    # 64 slices of 576 rows; n_rep 8
-], ids=["d64-nrep8-4096", "d128-nrep2", "d128-mha", "d16", "d64-nrep4-short-tail", "d128-two-trips", "d32-64-slices"])
+    (12, 4, 64, 4096, 2500, 2),     # groups of three query heads, 10 of 16 slices
+    (14, 2, 128, 1024, 900, 2),     # groups of seven
+], ids=["d64-nrep8-4096", "d128-nrep2", "d128-mha", "d16", "d64-nrep4-short-tail", "d128-two-trips", "d32-64-slices",
+        "d64-nrep3", "d128-nrep7"])
 def test_decode_over_a_long_cache_filled_directly(h, h_kv, d, max_seq, filled, steps):
     """Decode attention over caches of thousands of rows: the rows are written straight into both caches
     (lumen_kv_cache_update + lumen_kv_cache_set_len here, the arrays there), so no quadratic prompt pass is needed."""
@@ -157,7 +161,9 @@ def test_cache_state_machine_overflow_and_reset():
 # lengths that are no multiple of the tile sizes, with and without rows already in the cache)
 @pytest.mark.parametrize("h,h_kv,d,s,past", [(32, 4, 64, 128, 0), (16, 8, 128, 50, 17), (4, 4, 32, 3, 9), (8, 2, 16, 33, 31),
                                              (16, 2, 64, 331, 0), (8, 4, 128, 200, 45), (4, 4, 64, 193, 230),
-                                             (8, 2, 64, 257, 63)])
+                                             (8, 2, 64, 257, 63),
+                                             (6, 2, 64, 40, 11), (12, 4, 64, 300, 21), (14, 2, 128, 210, 0),  # groups of 3, 3, 7
+                                             (5, 1, 32, 70, 0)])
 def test_prefill_with_and_without_past(h, h_kv, d, s, past):
     max_seq = past + s + 3
     scale = 1.0 / math.sqrt(d)
