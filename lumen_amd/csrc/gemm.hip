@@ -1,20 +1,21 @@
 // Dense C[M,N] = A[M,K] W[N,K]^T for the M > 1 (prompt prefill) branch of
 // ops::matmul::matmul, src/ops/matmul.rs:70-92, on the gfx950 matrix cores.
 //
-// fp32 throughout: v_mfma_f32_32x32x2_f32 takes one f32 of A and one of W per
-// lane and accumulates a 32x32 tile in 16 registers per lane, so the result
-// carries full fp32 precision (the reference computes in f32 on the CPU).
-// bf16-stored weights are widened while they are staged into LDS, which is
-// the reference's own load-time upcast (src/loader.rs:58) moved to the device.
+// The reference computes in f32.  The f32 matrix instruction (v_mfma_f32_32x32x2_f32) runs at 1/16
+// of the bf16 rate on this chip, so the product is taken on the bf16 matrix cores instead without
+// giving up f32 accuracy: an f32 value is the exact sum of three bf16 values (8 + 8 + 8 mantissa
+// bits: take the upper 16 bits, subtract, repeat), so x * w is the sum of the products of their
+// parts; the six products whose orders add up to at most four carry everything down to 2^-24 of
+// the result and are accumulated in f32 by v_mfma_f32_32x32x16_bf16.  A bf16-stored weight (the
+// reference widens those at load time, src/loader.rs:58) is a single part: three products.
+// Six bf16 instructions of depth 16 against eight f32 instructions of depth 2 per 16 columns of K:
+// 2.6x the f32 matrix rate for f32 weights, 5.3x for bf16 weights; measured against an fp64
+// product the error is the same as with the f32 instruction (2e-7 .. 2e-6 of the largest element).
 //
-// Workgroup = 4 wavefronts (2x2), 128x128 output tile, 32-deep K slices staged
-// k-major in LDS.  The global loads of slice s+1 are issued into registers
-// before the matrix instructions of slice s, so their latency is covered by
-// 64 MFMAs per wavefront.  When the tile grid alone cannot fill the chip
-// (prompt of a few hundred tokens against a 2048-row weight) the K range is
-// split over gridDim.z; each split writes its partial tile to a workspace and
-// a second kernel adds the splits in index order and applies the epilogue, so
-// the result does not depend on scheduling.
+// When the tile grid alone cannot fill the chip (prompt of a few hundred tokens against a 2048-row
+// weight) the K range is split over gridDim.z; each split writes its partial tile to a workspace
+// and a second kernel adds the splits in index order and applies the epilogue, so the result does
+// not depend on scheduling.
 #include "internal.h"
 
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -24,7 +25,6 @@ typedef unsigned int v2u __attribute__((ext_vector_type(2)));
 #define BM 128
 #define BN 128
 #define BK 32
-#define LDT (BM + 1)
 #define STAGE 4  // 16-byte pieces of A and of W per thread per slice: 128 rows x 32 k / 256 threads
 
 __device__ __forceinline__ float silu_g(float g) {
@@ -32,87 +32,12 @@ __device__ __forceinline__ float silu_g(float g) {
     return g * sig;
 }
 
-// PARTIAL: store the raw tile of this K split to a.part[blockIdx.z][M][N]; the epilogue runs in
-// gemm_reduce_kernel.
-template <bool BF16, int EPI, bool PARTIAL>
-__global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs a) {
-    __shared__ float As[BK][LDT];
-    __shared__ float Ws[BK][LDT];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
-    const int bm = blockIdx.y * BM, bn = blockIdx.x * BN;
-    const int M = a.M, N = a.N, K = a.K;
-    const float *A = a.A;
-    // K range of this split, in whole slices
-    const int slices = (K + BK - 1) / BK;
-    const int per = (slices + (int)gridDim.z - 1) / (int)gridDim.z;
-    const int kb = (int)blockIdx.z * per * BK;
-    const int ke = min(K, kb + per * BK);
-
-    v16f acc[2][2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-    v4f va[STAGE], vw[STAGE];
-    // piece i of this thread: row (tid + 256 i) / 8, k offset 4 * ((tid + 256 i) % 8)
-    auto fetch = [&](int k0) {
-#pragma unroll
-        for (int i = 0; i < STAGE; ++i) {
-            const int idx = tid + i * 256;
-            const int row = idx >> 3, k4 = (idx & 7) * 4;
-            va[i] = (v4f){0.f, 0.f, 0.f, 0.f};
-            vw[i] = (v4f){0.f, 0.f, 0.f, 0.f};
-            if (k0 + k4 < ke) {  // K % 4 == 0: a piece is inside or outside as a whole
-                if (bm + row < M) va[i] = *(const v4f *)(A + (size_t)(bm + row) * K + k0 + k4);
-                if (bn + row < N) {
-                    if (BF16) {
-                        const v2u raw = *(const v2u *)((const uint16_t *)a.W + (size_t)(bn + row) * K + k0 + k4);
-                        vw[i].x = __uint_as_float(raw.x << 16);
-                        vw[i].y = __uint_as_float(raw.x & 0xffff0000u);
-                        vw[i].z = __uint_as_float(raw.y << 16);
-                        vw[i].w = __uint_as_float(raw.y & 0xffff0000u);
-                    } else {
-                        vw[i] = *(const v4f *)((const float *)a.W + (size_t)(bn + row) * K + k0 + k4);
-                    }
-                }
-            }
-        }
-    };
-
-    if (kb < ke) fetch(kb);
-    for (int k0 = kb; k0 < ke; k0 += BK) {
-#pragma unroll
-        for (int i = 0; i < STAGE; ++i) {
-            const int idx = tid + i * 256;
-            const int row = idx >> 3, k4 = (idx & 7) * 4;
-            As[k4 + 0][row] = va[i].x; As[k4 + 1][row] = va[i].y; As[k4 + 2][row] = va[i].z; As[k4 + 3][row] = va[i].w;
-            Ws[k4 + 0][row] = vw[i].x; Ws[k4 + 1][row] = vw[i].y; Ws[k4 + 2][row] = vw[i].z; Ws[k4 + 3][row] = vw[i].w;
-        }
-        __syncthreads();
-        if (k0 + BK < ke) fetch(k0 + BK);  // in flight during the matrix instructions below
-#pragma unroll
-        for (int kk = 0; kk < BK; kk += 2) {
-            const int kr = kk + (lane >> 5), c = lane & 31;
-            float af[2], bf[2];
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                af[i] = As[kr][wm * 64 + i * 32 + c];
-                bf[i] = Ws[kr][wn * 64 + i * 32 + c];
-            }
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bf[j], acc[i][j], 0, 0, 0);
-        }
-        __syncthreads();
-    }
-
-    // accumulator register r of lane l holds C[row = 8*(r/4) + 4*(l/32) + r%4][col = l%32] of the 32x32 tile
+// The 2x2 accumulator tiles of one wavefront to memory.  Accumulator register r of lane l holds
+// C[row = 8*(r/4) + 4*(l/32) + r%4][col = l%32] of its 32x32 tile.
+template <int EPI, bool PARTIAL>
+__device__ __forceinline__ void store_tile(const GemmArgs &a, const v16f (&acc)[2][2], int bm, int bn, int wm, int wn,
+                                           int lane) {
+    const int M = a.M, N = a.N;
     float *part = PARTIAL ? a.part + (size_t)blockIdx.z * M * N : nullptr;
 #pragma unroll
     for (int i = 0; i < 2; ++i)
@@ -134,6 +59,140 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs a) {
                     a.C[o] = (EPI == EPI_RESIDUAL) ? a.residual[o] + v : v;
                 }
             }
+}
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+
+#define XROW 40  // bf16 per LDS row: 32 of the slice + 8 of padding (80 bytes: the 16-byte reads of 8 rows hit 32 distinct banks)
+
+// upper halves of (odd, even) as one dword: two bf16 values, the even one in the low half
+__device__ __forceinline__ unsigned pack_hi(float odd, float even) {
+    return __builtin_amdgcn_perm(__float_as_uint(odd), __float_as_uint(even), 0x07060302u);
+}
+
+// x[0..3] -> three planes of 4 bf16 (2 dwords each): x = p0 + p1 + p2 up to 2^-24 |x|
+__device__ __forceinline__ void split3(const v4f x, v2u (&plane)[3]) {
+    float r[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+    for (int p = 0; p < 3; ++p) {
+        plane[p].x = pack_hi(r[1], r[0]);
+        plane[p].y = pack_hi(r[3], r[2]);
+        if (p < 2) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) r[e] -= __uint_as_float(__float_as_uint(r[e]) & 0xffff0000u);
+        }
+    }
+}
+
+// Workgroup = 4 wavefronts (2x2), 128x128 output tile, 32-deep slices: the raw values of the next
+// slice are in flight from memory during the matrix instructions of the current one, then split
+// into their bf16 parts on the way into LDS ([part][row][k], k contiguous: an operand is one
+// 16-byte LDS read).  Two workgroups share a compute unit, one computing while the other stages.
+template <bool WBF16, int EPI, bool PARTIAL>
+__global__ __launch_bounds__(256) void gemm_bf16x3_kernel(GemmArgs a) {
+    constexpr int PW = WBF16 ? 1 : 3;       // bf16 parts of a weight
+    constexpr int WST = WBF16 ? 2 : STAGE;  // 16-byte pieces of W per thread per slice
+    __shared__ __align__(16) uint16_t As[3][BM][XROW];
+    __shared__ __align__(16) uint16_t Ws[PW][BN][XROW];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int bm = blockIdx.y * BM, bn = blockIdx.x * BN;
+    const int M = a.M, N = a.N, K = a.K;
+    const float *A = a.A;
+    const int slices = (K + BK - 1) / BK;
+    const int per = (slices + (int)gridDim.z - 1) / (int)gridDim.z;
+    const int kb = (int)blockIdx.z * per * BK;
+    const int ke = min(K, kb + per * BK);
+
+    v16f acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    v4f va[STAGE];
+    v4u vw[WST];  // f32 weights: 4 floats; bf16 weights: 8 values
+    // A and f32 W: piece i of this thread is row (tid + 256 i) / 8, k offset 4 * ((tid + 256 i) % 8);
+    // bf16 W: row (tid + 256 i) / 4, k offset 8 * ((tid + 256 i) % 4)
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < STAGE; ++i) {
+            const int idx = tid + i * 256;
+            const int row = idx >> 3, k4 = (idx & 7) * 4;
+            va[i] = (v4f){0.f, 0.f, 0.f, 0.f};
+            if (k0 + k4 < ke && bm + row < M) va[i] = *(const v4f *)(A + (size_t)(bm + row) * K + k0 + k4);
+        }
+#pragma unroll
+        for (int i = 0; i < WST; ++i) {
+            const int idx = tid + i * 256;
+            const int row = WBF16 ? idx >> 2 : idx >> 3, kk = WBF16 ? (idx & 3) * 8 : (idx & 7) * 4;
+            vw[i] = (v4u){0u, 0u, 0u, 0u};
+            if (k0 + kk < ke && bn + row < N) {  // K % 8 == 0 (bf16) / K % 4 == 0: a piece is inside or outside as a whole
+                if (WBF16) vw[i] = *(const v4u *)((const uint16_t *)a.W + (size_t)(bn + row) * K + k0 + kk);
+                else vw[i] = *(const v4u *)((const float *)a.W + (size_t)(bn + row) * K + k0 + kk);
+            }
+        }
+    };
+
+    if (kb < ke) fetch(kb);
+    const int c = lane & 31, g8 = (lane >> 5) * 8;
+    for (int k0 = kb; k0 < ke; k0 += BK) {
+#pragma unroll
+        for (int i = 0; i < STAGE; ++i) {
+            const int idx = tid + i * 256;
+            v2u pl[3];
+            split3(va[i], pl);
+#pragma unroll
+            for (int p = 0; p < 3; ++p) *(v2u *)&As[p][idx >> 3][(idx & 7) * 4] = pl[p];
+        }
+#pragma unroll
+        for (int i = 0; i < WST; ++i) {
+            const int idx = tid + i * 256;
+            if (WBF16) {
+                *(v4u *)&Ws[0][idx >> 2][(idx & 3) * 8] = vw[i];
+            } else {
+                v2u pl[3];
+                split3((v4f){__uint_as_float(vw[i].x), __uint_as_float(vw[i].y), __uint_as_float(vw[i].z),
+                             __uint_as_float(vw[i].w)}, pl);
+#pragma unroll
+                for (int p = 0; p < PW; ++p) *(v2u *)&Ws[p][idx >> 3][(idx & 7) * 4] = pl[p];
+            }
+        }
+        __syncthreads();
+        if (k0 + BK < ke) fetch(k0 + BK);  // in flight during the matrix instructions below
+#pragma unroll
+        for (int ks = 0; ks < BK; ks += 16) {
+            // lane (c, g): 8 consecutive k of row c -- the same k for both operands
+            bf16x8 af[2][3], wf[2][PW];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+#pragma unroll
+                for (int p = 0; p < 3; ++p)
+                    af[i][p] = __builtin_bit_cast(bf16x8, *(const v4u *)&As[p][wm * 64 + i * 32 + c][ks + g8]);
+#pragma unroll
+                for (int p = 0; p < PW; ++p)
+                    wf[i][p] = __builtin_bit_cast(bf16x8, *(const v4u *)&Ws[p][wn * 64 + i * 32 + c][ks + g8]);
+            }
+            // products by ascending size; the four tiles take turns, so consecutive matrix
+            // instructions never wait on each other's accumulator
+            constexpr int NPROD = WBF16 ? 3 : 6;
+            constexpr int PA_[6] = {2, 0, 1, 1, 0, 0}, PW_[6] = {0, 2, 1, 0, 1, 0};  // f32 weights: a2w0 a0w2 a1w1 a1w0 a0w1 a0w0
+#pragma unroll
+            for (int q = 0; q < NPROD; ++q) {
+                const int xa = WBF16 ? 2 - q : PA_[q], xw = WBF16 ? 0 : PW_[q];
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i][xa], wf[j][xw], acc[i][j], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+    store_tile<EPI, PARTIAL>(a, acc, bm, bn, wm, wn, lane);
 }
 
 // Adds the K splits of every output element in split order and applies the epilogue.
@@ -179,13 +238,13 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(GemmArgs a) {
 template <bool BF16>
 static void launch_gemm_epi(const GemmArgs &a, dim3 grid, hipStream_t s) {
     if (grid.z > 1) {
-        hipLaunchKernelGGL((gemm_mfma_kernel<BF16, EPI_STORE, true>), grid, dim3(256), 0, s, a);
+        hipLaunchKernelGGL((gemm_bf16x3_kernel<BF16, EPI_STORE, true>), grid, dim3(256), 0, s, a);
         return;
     }
     switch (a.epi) {
-        case EPI_STORE: hipLaunchKernelGGL((gemm_mfma_kernel<BF16, EPI_STORE, false>), grid, dim3(256), 0, s, a); break;
-        case EPI_RESIDUAL: hipLaunchKernelGGL((gemm_mfma_kernel<BF16, EPI_RESIDUAL, false>), grid, dim3(256), 0, s, a); break;
-        default: hipLaunchKernelGGL((gemm_mfma_kernel<BF16, EPI_SWIGLU, false>), grid, dim3(256), 0, s, a); break;
+        case EPI_STORE: hipLaunchKernelGGL((gemm_bf16x3_kernel<BF16, EPI_STORE, false>), grid, dim3(256), 0, s, a); break;
+        case EPI_RESIDUAL: hipLaunchKernelGGL((gemm_bf16x3_kernel<BF16, EPI_RESIDUAL, false>), grid, dim3(256), 0, s, a); break;
+        default: hipLaunchKernelGGL((gemm_bf16x3_kernel<BF16, EPI_SWIGLU, false>), grid, dim3(256), 0, s, a); break;
     }
 }
 
@@ -214,9 +273,9 @@ static int gemm_splits(const lumen_ctx *ctx, const GemmArgs &a) {
 int launch_gemm(lumen_ctx *ctx, const GemmArgs &a) {
     if (a.M <= 0 || a.N <= 0) return LUMEN_OK;
     const bool aligned = (((uintptr_t)a.A | (uintptr_t)a.W) & 15) == 0;
-    const bool fast = (a.K % 4 == 0) && aligned && a.K > 0;
+    const bool fast = (a.K % (a.w_bf16 ? 8 : 4) == 0) && aligned && a.K > 0;  // rows of 16-byte pieces
     if (!fast) {
-        if (a.epi != EPI_STORE) LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "fused GEMM needs K %% 4 == 0 and 16-byte alignment (K=%d)", a.K);
+        if (a.epi != EPI_STORE) LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "fused GEMM needs rows of whole 16-byte pieces and 16-byte alignment (K=%d)", a.K);
         size_t blocks = ((size_t)a.M * a.N + 255) / 256;
         if (blocks > (size_t)ctx->num_cus * 16) blocks = (size_t)ctx->num_cus * 16;
         if (a.w_bf16)
