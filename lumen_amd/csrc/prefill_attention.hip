@@ -28,13 +28,26 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 #define FA_KEYS 32   // keys per tile
 #define FA_THREADS 256
 
+// Last step of a reduction over 32 lanes: combine lane l with lane l ^ 16.  v_permlane16_swap
+// exchanges the odd 16-lane rows of one register with the even rows of another on the vector ALU
+// (no trip through the LDS crossbar): with both operands v it leaves (row0,row0,row2,row2) and
+// (row1,row1,row3,row3).
+__device__ __forceinline__ float fmaxf16(float v) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float add16(float v) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // max over the 32 lanes of a half-wavefront; every lane gets the result
 __device__ __forceinline__ float half_max(float v) {
     v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false)));  // row_ror:8
     v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xf, 0xf, false)));  // row_ror:4
     v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xf, 0xf, false)));  // row_ror:2
     v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xf, 0xf, false)));  // row_ror:1
-    return fmaxf(v, __shfl_xor(v, 16, 64));
+    return fmaxf16(v);
 }
 
 __device__ __forceinline__ float half_sum(float v) {
@@ -42,7 +55,7 @@ __device__ __forceinline__ float half_sum(float v) {
     v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xf, 0xf, false));
     v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xf, 0xf, false));
     v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xf, 0xf, false));
-    return v + __shfl_xor(v, 16, 64);
+    return add16(v);
 }
 
 // q_rot [B,S,Hq,D] rotated queries; K (rotated) and V already in the cache up to past_len + S.
