@@ -178,7 +178,7 @@ def prefill_report(cfg, S, ms):
     return {"tokens": S, "ms": round(ms, 3), "tokens_per_s": round(S / ms * 1e3, 1),
             "gemm_flops": gemm_flops, "attention_flops": attn_flops, "achieved_TFLOPs": round(tf, 2),
             "matrix_path": "GEMM: f32 values as 3 bf16 parts, 6 v_mfma_f32_32x32x16_bf16 products per f32 product; "
-                           "attention: the same for head_dim 64, v_mfma_f32_32x32x2_f32 for 128",
+                           "attention: the same scheme",
             "mfma_fp32_peak_TFLOPs": MFMA_FP32_PEAK_TF, "vs_mfma_fp32_peak": round(tf / MFMA_FP32_PEAK_TF, 4),
             "gemm_bf16_TFLOPs_issued": round(issued, 1), "mfma_bf16_peak_TFLOPs": MFMA_BF16_PEAK_TF,
             "frac_of_mfma_bf16_peak": round(issued / MFMA_BF16_PEAK_TF, 4)}

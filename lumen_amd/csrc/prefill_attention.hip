@@ -9,16 +9,21 @@
 // so scores never leave the compute unit and every K/V tile read from the
 // cache serves all n_rep heads of the group and 128 / n_rep positions at once.
 //
+// The products run on the bf16 matrix cores at f32 accuracy, as in the prompt-pass GEMM: an f32
+// value is the exact sum of three bf16 values, a product the sum of the six part products whose
+// orders add up to at most four, accumulated in f32 by v_mfma_f32_32x32x16_bf16 (for head_dim 64:
+// 24 + 24 instructions of 8 passes per key tile and wavefront; the f32 instruction would take
+// 32 + 32 of 16 passes).
+//
 // Per wavefront (32 rows) and key tile:
-//   S  = Q K^T        D/2 v_mfma_f32_32x32x2_f32, Q fragments in registers, K from LDS.  The two
-//                     k-values an instruction consumes are (kk, D/2 + kk): a lane then needs D/2
-//                     CONSECUTIVE floats of its K row, fetched with 16-byte LDS reads (the sum over
-//                     the head dimension does not care how its terms are paired; P V likewise)
-//   row max           across the 32 lanes that hold a row's 32 keys (DPP + one shuffle)
+//   S  = Q K^T        Q split once into registers, K on its way into LDS ([part][key][element]);
+//                     an operand is one 16-byte LDS read of 8 consecutive elements; two
+//                     accumulators take turns so that consecutive instructions do not wait
+//   row max           across the 32 lanes that hold a row's 32 keys (DPP + one permlane swap)
 //   P  = exp2(S - m)  scores are kept in log2 units (Q is pre-multiplied by scale * log2 e);
 //                     the row sums stay per lane and are folded across lanes once at the end
-//   O  = alpha O + P V   P goes through a per-wavefront LDS patch to become an A operand
-// fp32 operands and accumulation throughout.
+//   O  = alpha O + P V   P goes through a per-wavefront LDS patch (f32) to become an A operand
+//                     and is split after that read; V is staged transposed ([part][element][key])
 #include "internal.h"
 #include "attn_device.h"
 
@@ -56,154 +61,6 @@ __device__ __forceinline__ float half_sum(float v) {
     v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xf, 0xf, false));
     v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xf, 0xf, false));
     return add16(v);
-}
-
-// q_rot [B,S,Hq,D] rotated queries; K (rotated) and V already in the cache up to past_len + S.
-template <int D, int NREP>
-__global__ __launch_bounds__(FA_THREADS) void attn_prefill_mfma_kernel(AttnPrefillArgs a) {
-    constexpr int BQ = FA_ROWS / NREP;       // positions per workgroup
-    constexpr int DT = D / 32;               // 32-wide output tiles per row
-    constexpr int PIECES = D * FA_KEYS / 4 / FA_THREADS;  // 16-byte pieces of a K (or V) tile per thread
-    // row strides = 4 mod 32 words: 16-byte reads of 8 neighbouring rows fall into distinct banks
-    constexpr int LDK = D + 4, LDV = FA_KEYS + 4, LDP = FA_KEYS + 4;
-    __shared__ __align__(16) float Ks[FA_KEYS][LDK];   // [key][element]
-    __shared__ __align__(16) float Vt[D][LDV];         // [element][key]: V transposed
-    __shared__ __align__(16) float Ps[FA_THREADS / 64][32][LDP];
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int c = lane & 31, half = lane >> 5;
-    // workgroups are dealt in index order: the blocks of late positions (most keys) go first
-    const int q0 = (int)(gridDim.x - 1 - blockIdx.x) * BQ, hk = blockIdx.y, bb = blockIdx.z;
-    const int L = a.past_len + a.s;
-    const size_t head_base = ((size_t)bb * a.hkv + hk / a.kv_div) * a.max_seq * D;  // kv_div > 1: grid row = query head
-    const float *Kc = a.k_cache + head_base, *Vc = a.v_cache + head_base;
-
-    // accumulator register r of lane l belongs to row 8*(r/4) + 4*(l/32) + r%4 of the wavefront's 32
-    auto row_of = [&](int r) { return 8 * (r >> 2) + 4 * half + (r & 3); };
-
-    // Q fragments: lane l feeds row l%32, element (l/32) * D/2 + kk of the dot product
-    const int my_row = wave * 32 + c;                 // row this lane feeds as an A operand
-    const int my_i = min(q0 + my_row / NREP, a.s - 1);  // clamped: rows past S are computed and dropped
-    const float *qrow = a.q_rot + (((size_t)bb * a.s + my_i) * a.hq + (size_t)hk * NREP + my_row % NREP) * D;
-    const float qf_scale = a.scale * LUMEN_LOG2E;
-    float qf[D / 2];
-#pragma unroll
-    for (int kk = 0; kk < D / 2; kk += 4) {
-        const v4f v = *(const v4f *)(qrow + half * (D / 2) + kk);
-        qf[kk] = v.x * qf_scale; qf[kk + 1] = v.y * qf_scale; qf[kk + 2] = v.z * qf_scale; qf[kk + 3] = v.w * qf_scale;
-    }
-
-    // keys this workgroup needs: up to the last position's own key
-    const int q_last = min(q0 + BQ, a.s) - 1;
-    const int kmax = a.causal ? min(L, a.past_len + q_last + 1) : L;
-    // last key the rows of this wavefront may see (uniform per wavefront)
-    const int wave_i_last = min(q0 + (wave * 32 + 31) / NREP, a.s - 1);
-    const int wave_kmax = a.causal ? min(L, a.past_len + wave_i_last + 1) : L;
-
-    v16f O[DT];
-    float m_run[16], l_run[16];
-#pragma unroll
-    for (int t = 0; t < DT; ++t)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) O[t][r] = 0.f;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        m_run[r] = -INFINITY;
-        l_run[r] = 0.f;
-    }
-    // position (absolute) of the row behind each accumulator register
-    int pos_r[16];
-#pragma unroll
-    for (int r = 0; r < 16; ++r) pos_r[r] = a.past_len + q0 + (wave * 32 + row_of(r)) / NREP;
-
-    v4f kreg[PIECES], vreg[PIECES];
-    auto fetch = [&](int j0) {
-#pragma unroll
-        for (int p = 0; p < PIECES; ++p) {
-            const int idx = tid + p * FA_THREADS;
-            const int key = idx / (D / 4), k4 = (idx % (D / 4)) * 4;
-            const int j = min(j0 + key, L - 1);  // keys past L are masked below
-            kreg[p] = *(const v4f *)(Kc + (size_t)j * D + k4);
-            vreg[p] = *(const v4f *)(Vc + (size_t)j * D + k4);
-        }
-    };
-
-    if (kmax > 0) fetch(0);
-    for (int j0 = 0; j0 < kmax; j0 += FA_KEYS) {
-#pragma unroll
-        for (int p = 0; p < PIECES; ++p) {
-            const int idx = tid + p * FA_THREADS;
-            const int key = idx / (D / 4), k4 = (idx % (D / 4)) * 4;
-            *(v4f *)&Ks[key][k4] = kreg[p];
-            Vt[k4 + 0][key] = vreg[p].x; Vt[k4 + 1][key] = vreg[p].y; Vt[k4 + 2][key] = vreg[p].z; Vt[k4 + 3][key] = vreg[p].w;
-        }
-        __syncthreads();
-        if (j0 + FA_KEYS < kmax) fetch(j0 + FA_KEYS);  // in flight during the matrix instructions below
-
-        if (j0 < wave_kmax) {  // uniform per wavefront: tiles wholly above the causal diagonal are skipped
-            v16f S;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) S[r] = 0.f;
-#pragma unroll
-            for (int kk = 0; kk < D / 2; kk += 4) {
-                const v4f kf = *(const v4f *)&Ks[c][half * (D / 2) + kk];
-                S = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[kk], kf.x, S, 0, 0, 0);
-                S = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[kk + 1], kf.y, S, 0, 0, 0);
-                S = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[kk + 2], kf.z, S, 0, 0, 0);
-                S = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[kk + 3], kf.w, S, 0, 0, 0);
-            }
-
-            const int j = j0 + c;  // this lane's key
-            float alpha[16];
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const bool valid = j < L && (!a.causal || j <= pos_r[r]);
-                const float s = valid ? S[r] : -INFINITY;
-                const float m_new = fmaxf(m_run[r], half_max(s));
-                float p = 0.f;
-                alpha[r] = 1.0f;
-                if (m_new > -INFINITY) {
-                    alpha[r] = fast_exp2(m_run[r] - m_new);  // exp2(-inf) = 0 on the row's first live tile
-                    p = fast_exp2(s - m_new);
-                }
-                l_run[r] = fmaf(l_run[r], alpha[r], p);
-                m_run[r] = m_new;
-                Ps[wave][row_of(r)][c] = p;
-            }
-#pragma unroll
-            for (int t = 0; t < DT; ++t)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) O[t][r] *= alpha[r];
-            __builtin_amdgcn_wave_barrier();  // P: written above by this wavefront, read below in another lane order
-            // keys (kk, 16 + kk) per instruction: 16 consecutive floats of the P row and of each V^T row
-#pragma unroll
-            for (int kk = 0; kk < FA_KEYS / 2; kk += 4) {
-                const v4f pf = *(const v4f *)&Ps[wave][c][half * (FA_KEYS / 2) + kk];
-#pragma unroll
-                for (int t = 0; t < DT; ++t) {
-                    const v4f vf = *(const v4f *)&Vt[32 * t + c][half * (FA_KEYS / 2) + kk];
-                    O[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(pf.x, vf.x, O[t], 0, 0, 0);
-                    O[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(pf.y, vf.y, O[t], 0, 0, 0);
-                    O[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(pf.z, vf.z, O[t], 0, 0, 0);
-                    O[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(pf.w, vf.w, O[t], 0, 0, 0);
-                }
-            }
-        }
-        __syncthreads();
-    }
-
-    // out = ctx / (sum + 1e-9), self_attention.rs:670-676; [B,S,Hq,D]
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const float inv = 1.0f / (half_sum(l_run[r]) + 1e-9f);
-        const int row = wave * 32 + row_of(r);
-        const int i = q0 + row / NREP;
-        if (i < a.s) {
-            float *o = a.out + (((size_t)bb * a.s + i) * a.hq + (size_t)hk * NREP + row % NREP) * D;
-#pragma unroll
-            for (int t = 0; t < DT; ++t) o[32 * t + c] = O[t][r] * inv;
-        }
-    }
 }
 
 // ---- the same tile loop on the bf16 matrix cores at f32 accuracy (head_dim 64) ----
@@ -423,13 +280,9 @@ template <int D>
 static int launch_fa_d(lumen_ctx *ctx, const AttnPrefillArgs &a) {
     const int nrep = a.hq / a.hkv;
     dim3 block(FA_THREADS);
-    // head_dim 64: bf16-part kernel; 128: the f32-instruction kernel (the part kernel's LDS would pass 64 KiB)
-#define LAUNCH_FA(NR)                                                                                          \
-    do {                                                                                                       \
-        dim3 grid((a.s + FA_ROWS / NR - 1) / (FA_ROWS / NR), a.hkv, a.b);                                      \
-        if (D == 64) hipLaunchKernelGGL((attn_prefill_bf16x3_kernel<64, NR>), grid, block, 0, ctx->stream, a); \
-        else hipLaunchKernelGGL((attn_prefill_mfma_kernel<D, NR>), grid, block, 0, ctx->stream, a);            \
-    } while (0)
+#define LAUNCH_FA(NR)                                                                                    \
+    hipLaunchKernelGGL((attn_prefill_bf16x3_kernel<D, NR>), dim3((a.s + FA_ROWS / NR - 1) / (FA_ROWS / NR), a.hkv, a.b), \
+                       block, 0, ctx->stream, a)
     switch (nrep) {
         case 1: LAUNCH_FA(1); break;
         case 2: LAUNCH_FA(2); break;
@@ -438,9 +291,8 @@ static int launch_fa_d(lumen_ctx *ctx, const AttnPrefillArgs &a) {
         default: {  // any other group size: one query head per grid row, its KV head = head / n_rep
             AttnPrefillArgs b = a;
             b.kv_div = nrep;
-            dim3 grid((a.s + FA_ROWS - 1) / FA_ROWS, a.hq, a.b);
-            if (D == 64) hipLaunchKernelGGL((attn_prefill_bf16x3_kernel<64, 1>), grid, block, 0, ctx->stream, b);
-            else hipLaunchKernelGGL((attn_prefill_mfma_kernel<D, 1>), grid, block, 0, ctx->stream, b);
+            hipLaunchKernelGGL((attn_prefill_bf16x3_kernel<D, 1>), dim3((a.s + FA_ROWS - 1) / FA_ROWS, a.hq, a.b), block, 0,
+                               ctx->stream, b);
         }
     }
 #undef LAUNCH_FA
