@@ -110,6 +110,36 @@ def test_decode_over_a_long_cache_filled_directly(h, h_kv, d, max_seq, filled, s
     assert e.value.status == _lib.ERR_KV_OVERFLOW
 
 
+@pytest.mark.parametrize("b,h,h_kv,d,max_seq,prefill,steps", [
+    (2, 8, 2, 64, 128, 20, 4),       # short form
+    (3, 4, 4, 128, 640, 300, 3),     # long form (3 slices), one head per KV head
+    (2, 16, 2, 64, 1024, 200, 2),    # prompt pass on the matrix cores, then the short form
+])
+def test_batch_of_sequences(b, h, h_kv, d, max_seq, prefill, steps):
+    """The operator entry points take a batch (KVCacheInner::new(b, ...), self_attention.rs:33); every sequence of
+    the batch is at the same position."""
+    scale = 1.0 / math.sqrt(d)
+    rope = RotaryEmbedding(d, max_seq, 10000.0)
+    cos, sin = lo.rope_table(d, max_seq, 10000.0)
+    g, o = KVCacheInner(b, h_kv, max_seq, d), lo.KVCache(b, h_kv, max_seq, d)
+    q = f32(RNG.normal(0, 1, (b, prefill, h, d)))
+    k = f32(RNG.normal(0, 1, (b, prefill, h_kv, d)))
+    v = f32(RNG.normal(0, 1, (b, prefill, h_kv, d)))
+    got = gpu_prefill(g, rope, q, k, v, scale)
+    rc, ref = lo.attn_prefill(o, q, k, v, cos, sin, scale)
+    assert rc == lo.LO_OK and max_rel(got, ref) <= TOL
+    for t in range(steps):
+        q = f32(RNG.normal(0, 1, (b, h, d)))
+        k = f32(RNG.normal(0, 1, (b, h_kv, d)))
+        v = f32(RNG.normal(0, 1, (b, h_kv, d)))
+        got = gpu_decode(g, rope, q, k, v, h, scale)
+        rc, ref = lo.attn_decode(o, q, k, v, cos, sin, scale)
+        assert rc == lo.LO_OK and max_rel(got, ref) <= TOL, t
+    n = prefill + steps
+    assert g.len == o.len == n
+    assert np.array_equal(g.k[:, :, :n], o.k[:, :, :n]) and np.array_equal(g.v[:, :, :n], o.v[:, :, :n])
+
+
 def test_decode_degenerate_and_gqa_mapping():
     h, h_kv, d, max_seq = 8, 2, 64, 128
     rope = RotaryEmbedding(d, max_seq, 10000.0)
