@@ -82,6 +82,35 @@ def test_gemm_against_oracle(M, N, K):
     assert max_rel(C, A[0].astype(np.float64) @ W.T.astype(np.float64)) <= 1e-5
 
 
+def test_gemm_keeps_f32_accuracy_across_magnitudes():
+    """The prompt-pass product runs on the bf16 matrix cores with every f32 operand taken as three bf16 parts;
+    that must not cost accuracy whatever the magnitudes: rows of A and of W scaled by powers of ten from 1e-12 to
+    1e12, entries of one row spread over six decades, exact cancellation, and each output compared with the fp64
+    product relative to the size of its own terms (sum |a||w|), where an f32 dot product of this length is good
+    to a few 1e-7."""
+    M, N, K = 96, 160, 512
+    A = RNG.normal(0, 1, (M, K)) * 10.0 ** RNG.uniform(-3, 3, (M, K))
+    W = RNG.normal(0, 1, (N, K)) * 10.0 ** RNG.uniform(-3, 3, (N, K))
+    A *= 10.0 ** RNG.integers(-12, 13, (M, 1))
+    W *= 10.0 ** RNG.integers(-12, 13, (N, 1))
+    A[5, 1::2] = -A[5, 0::2]          # row 5 against row 7 of W cancels exactly
+    W[7, 1::2] = W[7, 0::2]
+    A, W = f32(A), f32(W)
+    C = ops.matmul(dev(A[None]), dev(W)).data()[0]
+    a64, w64 = A.astype(np.float64), W.astype(np.float64)
+    ref, size = a64 @ w64.T, np.abs(a64) @ np.abs(w64).T
+    assert np.isfinite(C).all()
+    err = np.abs(C - ref) / size
+    assert err.max() <= 1e-6, err.max()
+    assert abs(C[5, 7]) <= 1e-6 * size[5, 7]
+    # bf16-stored weights: the weight is one part, the activation still three
+    bits = lo.f32_to_bf16(W)
+    Wb = lo.bf16_to_f32(bits)
+    Cb = ops.matmul(dev(A[None]), dev(bits)).data()[0]
+    errb = np.abs(Cb - a64 @ Wb.astype(np.float64).T) / (np.abs(a64) @ np.abs(Wb.astype(np.float64)).T)
+    assert errb.max() <= 1e-6, errb.max()
+
+
 def test_gemm_bf16_weights():
     M, N, K = 48, 300, 256
     A = f32(RNG.normal(0, 1, (M, K)))
