@@ -64,7 +64,12 @@ __device__ __forceinline__ void store_tile(const GemmArgs &a, const v16f (&acc)[
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 
-#define XROW 40  // bf16 per LDS row: 32 of the slice + 8 of padding (80 bytes: the 16-byte reads of 8 rows hit 32 distinct banks)
+// LDS rows hold the 32 bf16 of a slice (64 bytes, no padding) as four 16-byte chunks; chunk q of row r sits
+// at position q ^ ((r >> 1) & 3).  Even rows start at bank 0, odd rows at bank 16, so the 16-byte operand
+// reads of 8 neighbouring rows (same chunk index) and the 8-byte staging writes of two neighbouring rows
+// each cover all 32 banks exactly once.
+#define XROW 32
+__device__ __forceinline__ int lds_col(int row, int k) { return ((((k >> 3) ^ (row >> 1)) & 3) << 3) | (k & 7); }
 
 // upper halves of (odd, even) as one dword: two bf16 values, the even one in the low half
 __device__ __forceinline__ unsigned pack_hi(float odd, float even) {
@@ -146,19 +151,19 @@ __global__ __launch_bounds__(256) void gemm_bf16x3_kernel(GemmArgs a) {
             v2u pl[3];
             split3(va[i], pl);
 #pragma unroll
-            for (int p = 0; p < 3; ++p) *(v2u *)&As[p][idx >> 3][(idx & 7) * 4] = pl[p];
+            for (int p = 0; p < 3; ++p) *(v2u *)&As[p][idx >> 3][lds_col(idx >> 3, (idx & 7) * 4)] = pl[p];
         }
 #pragma unroll
         for (int i = 0; i < WST; ++i) {
             const int idx = tid + i * 256;
             if (WBF16) {
-                *(v4u *)&Ws[0][idx >> 2][(idx & 3) * 8] = vw[i];
+                *(v4u *)&Ws[0][idx >> 2][lds_col(idx >> 2, (idx & 3) * 8)] = vw[i];
             } else {
                 v2u pl[3];
                 split3((v4f){__uint_as_float(vw[i].x), __uint_as_float(vw[i].y), __uint_as_float(vw[i].z),
                              __uint_as_float(vw[i].w)}, pl);
 #pragma unroll
-                for (int p = 0; p < PW; ++p) *(v2u *)&Ws[p][idx >> 3][(idx & 7) * 4] = pl[p];
+                for (int p = 0; p < PW; ++p) *(v2u *)&Ws[p][idx >> 3][lds_col(idx >> 3, (idx & 7) * 4)] = pl[p];
             }
         }
         __syncthreads();
@@ -171,10 +176,10 @@ __global__ __launch_bounds__(256) void gemm_bf16x3_kernel(GemmArgs a) {
             for (int i = 0; i < 2; ++i) {
 #pragma unroll
                 for (int p = 0; p < 3; ++p)
-                    af[i][p] = __builtin_bit_cast(bf16x8, *(const v4u *)&As[p][wm * 64 + i * 32 + c][ks + g8]);
+                    af[i][p] = __builtin_bit_cast(bf16x8, *(const v4u *)&As[p][wm * 64 + i * 32 + c][lds_col(c, ks + g8)]);
 #pragma unroll
                 for (int p = 0; p < PW; ++p)
-                    wf[i][p] = __builtin_bit_cast(bf16x8, *(const v4u *)&Ws[p][wn * 64 + i * 32 + c][ks + g8]);
+                    wf[i][p] = __builtin_bit_cast(bf16x8, *(const v4u *)&Ws[p][wn * 64 + i * 32 + c][lds_col(c, ks + g8)]);
             }
             // products by ascending size; the four tiles take turns, so consecutive matrix
             // instructions never wait on each other's accumulator
