@@ -15,15 +15,17 @@
 // 24 + 24 instructions of 8 passes per key tile and wavefront; the f32 instruction would take
 // 32 + 32 of 16 passes).
 //
-// Per wavefront (32 rows) and key tile:
-//   S  = Q K^T        Q split once into registers, K on its way into LDS ([part][key][element]);
-//                     an operand is one 16-byte LDS read of 8 consecutive elements; two
-//                     accumulators take turns so that consecutive instructions do not wait
-//   row max           across the 32 lanes that hold a row's 32 keys (DPP + one permlane swap)
-//   P  = exp2(S - m)  scores are kept in log2 units (Q is pre-multiplied by scale * log2 e);
-//                     the row sums stay per lane and are folded across lanes once at the end
-//   O  = alpha O + P V   P goes through a per-wavefront LDS patch (f32) to become an A operand
-//                     and is split after that read; V is staged transposed ([part][element][key])
+// Per wavefront (32 rows) and key tile, everything transposed so that a lane owns one query row:
+//   S^T = K Q^T       K from LDS ([part][key][element], split on its way in) is the A operand, Q
+//                     (split once, in registers) the B operand; two accumulators take turns so
+//                     that consecutive instructions do not wait.  A lane then holds 16 of the
+//                     tile's 32 scores of ITS row, lane ^ 32 the other 16
+//   softmax           row max and sum in the lane (one exchange with lane ^ 32 for the max, one at
+//                     the very end for the sum); scores in log2 units (Q pre-multiplied by
+//                     scale * log2 e), P = exp2(S - m)
+//   O^T += V^T P^T    V is staged transposed ([part][element][key position]) as the A operand; the
+//                     lane's 16 weights are the B operand as they stand (split in the lane), no
+//                     trip through LDS; the rescale by alpha is a per-lane scalar
 #include "internal.h"
 #include "attn_device.h"
 
@@ -33,45 +35,6 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 #define FA_KEYS 32   // keys per tile
 #define FA_THREADS 256
 
-// Last step of a reduction over 32 lanes: combine lane l with lane l ^ 16.  v_permlane16_swap
-// exchanges the odd 16-lane rows of one register with the even rows of another on the vector ALU
-// (no trip through the LDS crossbar): with both operands v it leaves (row0,row0,row2,row2) and
-// (row1,row1,row3,row3).
-__device__ __forceinline__ float fmaxf16(float v) {
-    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-__device__ __forceinline__ float add16(float v) {
-    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
-}
-
-// max over the 32 lanes of a half-wavefront; every lane gets the result
-__device__ __forceinline__ float half_max(float v) {
-    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false)));  // row_ror:8
-    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xf, 0xf, false)));  // row_ror:4
-    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xf, 0xf, false)));  // row_ror:2
-    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xf, 0xf, false)));  // row_ror:1
-    return fmaxf16(v);
-}
-
-__device__ __forceinline__ float half_sum(float v) {
-    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false));
-    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xf, 0xf, false));
-    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xf, 0xf, false));
-    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xf, 0xf, false));
-    return add16(v);
-}
-
-// ---- the same tile loop on the bf16 matrix cores at f32 accuracy (head_dim 64) ----
-// As in the prompt-pass GEMM: an f32 value is the exact sum of three bf16 values, a product the sum
-// of the six part products whose orders add up to at most four, accumulated in f32 by
-// v_mfma_f32_32x32x16_bf16 -- 24 + 24 instructions of 8 passes per key tile and wavefront instead
-// of 32 + 32 of 16 passes with the f32 instruction.  Q is split once into registers, K and V on
-// their way into LDS ([part][key][element] and, transposed, [part][element][key]), P after the
-// transposing trip through the per-wavefront LDS patch; K and V operands are single 16-byte LDS
-// reads of 8 consecutive elements (keys).  Two accumulators take turns under Q K^T so that consecutive matrix
-// instructions do not wait on each other.
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 typedef unsigned int v2u __attribute__((ext_vector_type(2)));
@@ -104,13 +67,12 @@ __device__ __forceinline__ void fa_split1(float x, uint16_t (&part)[3]) {
 template <int D, int NREP>
 __global__ __launch_bounds__(FA_THREADS) void attn_prefill_bf16x3_kernel(AttnPrefillArgs a) {
     constexpr int BQ = FA_ROWS / NREP;  // positions per workgroup
-    constexpr int DT = D / 32;          // 32-wide output tiles per row
+    constexpr int DT = D / 32;          // 32-wide tiles of the head dimension
     constexpr int PIECES = D * FA_KEYS / 4 / FA_THREADS;  // 16-byte pieces of a K (or V) tile per thread
     // rows of 4 words more than a multiple of 32: the 16-byte reads of 8 neighbouring rows hit distinct banks
     constexpr int LDK = D + 8, LDV = FA_KEYS + 8;
-    __shared__ __align__(16) uint16_t Ks[3][FA_KEYS][LDK];            // [part][key][element]
-    __shared__ __align__(16) uint16_t Vt[3][D][LDV];                  // [part][element][key]
-    __shared__ __align__(16) float Ps[FA_THREADS / 64][32][FA_KEYS + 4];  // [wavefront][row][key], f32: split after the transposing read
+    __shared__ __align__(16) uint16_t Ks[3][FA_KEYS][LDK];  // [part][key][element]
+    __shared__ __align__(16) uint16_t Vt[3][D][LDV];        // [part][element][key position]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = lane & 31, half = lane >> 5;
@@ -119,13 +81,14 @@ __global__ __launch_bounds__(FA_THREADS) void attn_prefill_bf16x3_kernel(AttnPre
     const int L = a.past_len + a.s;
     const size_t head_base = ((size_t)bb * a.hkv + hk / a.kv_div) * a.max_seq * D;  // kv_div > 1: grid row = query head
     const float *Kc = a.k_cache + head_base, *Vc = a.v_cache + head_base;
-    auto row_of = [&](int r) { return 8 * (r >> 2) + 4 * half + (r & 3); };
 
-    // Q operand: lane (row c, half g) holds elements ks * 16 + g * 8 .. + 7 of its row for every 16-deep step
+    // This lane's query row (the COLUMN it owns in S^T and O^T): (position, head) row wave * 32 + c of the workgroup
     const int my_row = wave * 32 + c;
     const int my_i = min(q0 + my_row / NREP, a.s - 1);  // clamped: rows past S are computed and dropped
+    const int my_pos = a.past_len + q0 + my_row / NREP;  // absolute position: keys up to it are visible
     const float *qrow = a.q_rot + (((size_t)bb * a.s + my_i) * a.hq + (size_t)hk * NREP + my_row % NREP) * D;
     const float qf_scale = a.scale * LUMEN_LOG2E;
+    // Q as the B operand of S^T = K Q^T: lane (column c, half g) holds elements ks * 16 + g * 8 .. + 7 of its row
     v4u qp[D / 16][3];
 #pragma unroll
     for (int ks = 0; ks < D / 16; ++ks) {
@@ -145,20 +108,13 @@ __global__ __launch_bounds__(FA_THREADS) void attn_prefill_bf16x3_kernel(AttnPre
     const int wave_i_last = min(q0 + (wave * 32 + 31) / NREP, a.s - 1);
     const int wave_kmax = a.causal ? min(L, a.past_len + wave_i_last + 1) : L;
 
+    // O^T: register r of tile t belongs to element 32 t + 8 (r / 4) + 4 half + r % 4 of this lane's row
     v16f O[DT];
-    float m_run[16], l_run[16];
 #pragma unroll
     for (int t = 0; t < DT; ++t)
 #pragma unroll
         for (int r = 0; r < 16; ++r) O[t][r] = 0.f;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        m_run[r] = -INFINITY;
-        l_run[r] = 0.f;
-    }
-    int pos_r[16];
-#pragma unroll
-    for (int r = 0; r < 16; ++r) pos_r[r] = a.past_len + q0 + (wave * 32 + row_of(r)) / NREP;
+    float m_run = -INFINITY, l_run = 0.f;  // of this lane's row; l over this lane's half of the keys
 
     v4f kreg[PIECES], vreg[PIECES];
     auto fetch = [&](int j0) {
@@ -183,19 +139,23 @@ __global__ __launch_bounds__(FA_THREADS) void attn_prefill_bf16x3_kernel(AttnPre
             fa_split4(kreg[p], kp);
 #pragma unroll
             for (int q = 0; q < 3; ++q) *(v2u *)&Ks[q][key][k4] = kp[q];
+            // V^T, with bits 2 and 3 of the key index exchanged: the 8 keys a lane holds of S^T
+            // (4 + 4, eight apart) then sit next to each other for the 16-byte operand read
+            const int kpos = (key & ~12) | ((key & 4) << 1) | ((key & 8) >> 1);
             const float ve[4] = {vreg[p].x, vreg[p].y, vreg[p].z, vreg[p].w};
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 uint16_t vp[3];
                 fa_split1(ve[e], vp);
 #pragma unroll
-                for (int q = 0; q < 3; ++q) Vt[q][k4 + e][key] = vp[q];
+                for (int q = 0; q < 3; ++q) Vt[q][k4 + e][kpos] = vp[q];
             }
         }
         __syncthreads();
         if (j0 + FA_KEYS < kmax) fetch(j0 + FA_KEYS);  // in flight during the matrix instructions below
 
         if (j0 < wave_kmax) {  // uniform per wavefront: tiles wholly above the causal diagonal are skipped
+            // S^T = K Q^T: register r holds key 8 (r / 4) + 4 half + r % 4 of the tile against this lane's row
             v16f Sa, Sb;
 #pragma unroll
             for (int r = 0; r < 16; ++r) Sa[r] = Sb[r] = 0.f;
@@ -209,40 +169,47 @@ __global__ __launch_bounds__(FA_THREADS) void attn_prefill_bf16x3_kernel(AttnPre
                 }
 #pragma unroll
                 for (int q = 0; q < 6; q += 2) {
-                    Sa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qf[PA_[q]], kf[PB_[q]], Sa, 0, 0, 0);
-                    Sb = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qf[PA_[q + 1]], kf[PB_[q + 1]], Sb, 0, 0, 0);
+                    Sa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[PA_[q]], qf[PB_[q]], Sa, 0, 0, 0);
+                    Sb = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[PA_[q + 1]], qf[PB_[q + 1]], Sb, 0, 0, 0);
                 }
             }
 
-            const int j = j0 + c;  // this lane's key
-            float alpha[16];
+            // softmax of this lane's row, in the lane: 16 of the tile's 32 keys here, 16 in lane ^ 32
+            float sc[16];
+            float m_tile = -INFINITY;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const bool valid = j < L && (!a.causal || j <= pos_r[r]);
-                const float s = valid ? Sa[r] + Sb[r] : -INFINITY;
-                const float m_new = fmaxf(m_run[r], half_max(s));
-                float p = 0.f;
-                alpha[r] = 1.0f;
-                if (m_new > -INFINITY) {
-                    alpha[r] = fast_exp2(m_run[r] - m_new);  // exp2(-inf) = 0 on the row's first live tile
-                    p = fast_exp2(s - m_new);
-                }
-                l_run[r] = fmaf(l_run[r], alpha[r], p);
-                m_run[r] = m_new;
-                Ps[wave][row_of(r)][c] = p;
+                const int j = j0 + 8 * (r >> 2) + 4 * half + (r & 3);
+                const bool valid = j < L && (!a.causal || j <= my_pos);
+                sc[r] = valid ? Sa[r] + Sb[r] : -INFINITY;
+                m_tile = fmaxf(m_tile, sc[r]);
             }
+            m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
+            const float m_new = fmaxf(m_run, m_tile);
+            const float m_ref = m_new > -INFINITY ? m_new : 0.f;  // nothing visible yet: every weight below is exp2(-inf) = 0
+            const float alpha = fast_exp2(m_run - m_ref);
+            m_run = m_new;
+            float psum = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                sc[r] = fast_exp2(sc[r] - m_ref);
+                psum += sc[r];
+            }
+            l_run = fmaf(l_run, alpha, psum);
 #pragma unroll
             for (int t = 0; t < DT; ++t)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) O[t][r] *= alpha[r];
-            __builtin_amdgcn_wave_barrier();  // P: written above by this wavefront, read below in another lane order
+                for (int r = 0; r < 16; ++r) O[t][r] *= alpha;
+
+            // O^T += V^T P^T: P^T is this lane's 16 weights, already where the B operand wants them
+            // (registers 8 ks .. 8 ks + 7 are the keys at positions 16 ks + 8 half .. + 7 of V^T)
 #pragma unroll
             for (int ks = 0; ks < FA_KEYS / 16; ++ks) {
                 bf16x8 pf[3];
                 {
                     v2u lo[3], hi[3];
-                    fa_split4(*(const v4f *)&Ps[wave][c][ks * 16 + half * 8], lo);
-                    fa_split4(*(const v4f *)&Ps[wave][c][ks * 16 + half * 8 + 4], hi);
+                    fa_split4((v4f){sc[8 * ks], sc[8 * ks + 1], sc[8 * ks + 2], sc[8 * ks + 3]}, lo);
+                    fa_split4((v4f){sc[8 * ks + 4], sc[8 * ks + 5], sc[8 * ks + 6], sc[8 * ks + 7]}, hi);
 #pragma unroll
                     for (int p = 0; p < 3; ++p) pf[p] = __builtin_bit_cast(bf16x8, (v4u){lo[p].x, lo[p].y, hi[p].x, hi[p].y});
                 }
@@ -256,23 +223,24 @@ __global__ __launch_bounds__(FA_THREADS) void attn_prefill_bf16x3_kernel(AttnPre
                 for (int q = 0; q < 6; ++q)
 #pragma unroll
                     for (int t = 0; t < DT; ++t)
-                        O[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[PA_[q]], vf[t][PB_[q]], O[t], 0, 0, 0);
+                        O[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[t][PA_[q]], pf[PB_[q]], O[t], 0, 0, 0);
             }
         }
         __syncthreads();
     }
 
     // out = ctx / (sum + 1e-9), self_attention.rs:670-676; [B,S,Hq,D]
+    const float inv = 1.0f / ((l_run + __shfl_xor(l_run, 32, 64)) + 1e-9f);
+    const int i = q0 + my_row / NREP;
+    if (i < a.s) {
+        float *o = a.out + (((size_t)bb * a.s + i) * a.hq + (size_t)hk * NREP + my_row % NREP) * D;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const float inv = 1.0f / (half_sum(l_run[r]) + 1e-9f);
-        const int row = wave * 32 + row_of(r);
-        const int i = q0 + row / NREP;
-        if (i < a.s) {
-            float *o = a.out + (((size_t)bb * a.s + i) * a.hq + (size_t)hk * NREP + row % NREP) * D;
+        for (int t = 0; t < DT; ++t)
 #pragma unroll
-            for (int t = 0; t < DT; ++t) o[32 * t + c] = O[t][r] * inv;
-        }
+            for (int g = 0; g < 4; ++g) {
+                v4f v = {O[t][4 * g] * inv, O[t][4 * g + 1] * inv, O[t][4 * g + 2] * inv, O[t][4 * g + 3] * inv};
+                *(v4f *)(o + 32 * t + 8 * g + 4 * half) = v;
+            }
     }
 }
 
