@@ -266,7 +266,7 @@ static void launch_gemm_reduce(const GemmArgs &a, int splits, int blocks, hipStr
 static int gemm_splits(const lumen_ctx *ctx, const GemmArgs &a) {
     const long tiles = (long)((a.N + BN - 1) / BN) * ((a.M + BM - 1) / BM);
     const long want = 2L * ctx->num_cus;
-    if (tiles >= want) return 1;
+    if (tiles * 4 >= want * 3) return 1;  // three quarters of the slots filled: a split would cost more in partial tiles than it gains
     long s = (want + tiles - 1) / tiles;
     const long max_by_k = a.K / (4 * BK);
     if (s > max_by_k) s = max_by_k;
