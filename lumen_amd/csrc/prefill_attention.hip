@@ -64,14 +64,17 @@ __device__ __forceinline__ void fa_split1(float x, uint16_t (&part)[3]) {
     }
 }
 
-template <int D, int NREP>
-__global__ __launch_bounds__(FA_THREADS) void attn_prefill_bf16x3_kernel(AttnPrefillArgs a) {
+// KT: key tiles of 32 per trip of the loop (2 for head_dim 64: one barrier pair, one row maximum and one rescale of
+// O per 64 keys; 1 for head_dim 128, whose K and V tiles fill LDS twice as fast).
+template <int D, int NREP, int KT>
+__global__ __launch_bounds__(FA_THREADS, (D == 64 ? 2 : 1)) void attn_prefill_bf16x3_kernel(AttnPrefillArgs a) {
     constexpr int BQ = FA_ROWS / NREP;  // positions per workgroup
+    constexpr int KEYS = FA_KEYS * KT;   // keys per trip
     constexpr int DT = D / 32;          // 32-wide tiles of the head dimension
-    constexpr int PIECES = D * FA_KEYS / 4 / FA_THREADS;  // 16-byte pieces of a K (or V) tile per thread
+    constexpr int PIECES = D * KEYS / 4 / FA_THREADS;  // 16-byte pieces of a K (or V) tile per thread
     // rows of 4 words more than a multiple of 32: the 16-byte reads of 8 neighbouring rows hit distinct banks
-    constexpr int LDK = D + 8, LDV = FA_KEYS + 8;
-    __shared__ __align__(16) uint16_t Ks[3][FA_KEYS][LDK];  // [part][key][element]
+    constexpr int LDK = D + 8, LDV = KEYS + 8;
+    __shared__ __align__(16) uint16_t Ks[3][KEYS][LDK];  // [part][key][element]
     __shared__ __align__(16) uint16_t Vt[3][D][LDV];        // [part][element][key position]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -130,7 +133,7 @@ __global__ __launch_bounds__(FA_THREADS) void attn_prefill_bf16x3_kernel(AttnPre
 
     constexpr int PA_[6] = {2, 0, 1, 1, 0, 0}, PB_[6] = {0, 2, 1, 0, 1, 0};  // part products by ascending size
     if (kmax > 0) fetch(0);
-    for (int j0 = 0; j0 < kmax; j0 += FA_KEYS) {
+    for (int j0 = 0; j0 < kmax; j0 += KEYS) {
 #pragma unroll
         for (int p = 0; p < PIECES; ++p) {
             const int idx = tid + p * FA_THREADS;
@@ -152,38 +155,46 @@ __global__ __launch_bounds__(FA_THREADS) void attn_prefill_bf16x3_kernel(AttnPre
             }
         }
         __syncthreads();
-        if (j0 + FA_KEYS < kmax) fetch(j0 + FA_KEYS);  // in flight during the matrix instructions below
+        if (j0 + KEYS < kmax) fetch(j0 + KEYS);  // in flight during the matrix instructions below
 
         if (j0 < wave_kmax) {  // uniform per wavefront: tiles wholly above the causal diagonal are skipped
-            // S^T = K Q^T: register r holds key 8 (r / 4) + 4 half + r % 4 of the tile against this lane's row
-            v16f Sa, Sb;
+            // S^T = K Q^T: register r of tile kt holds key 32 kt + 8 (r / 4) + 4 half + r % 4 against this lane's row
+            v16f Sa[KT], Sb[KT];
 #pragma unroll
-            for (int r = 0; r < 16; ++r) Sa[r] = Sb[r] = 0.f;
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) Sa[kt][r] = Sb[kt][r] = 0.f;
 #pragma unroll
             for (int ks = 0; ks < D / 16; ++ks) {
-                bf16x8 kf[3], qf[3];
+                bf16x8 qf[3];
 #pragma unroll
-                for (int p = 0; p < 3; ++p) {
-                    kf[p] = __builtin_bit_cast(bf16x8, *(const v4u *)&Ks[p][c][ks * 16 + half * 8]);
-                    qf[p] = __builtin_bit_cast(bf16x8, qp[ks][p]);
-                }
+                for (int p = 0; p < 3; ++p) qf[p] = __builtin_bit_cast(bf16x8, qp[ks][p]);
 #pragma unroll
-                for (int q = 0; q < 6; q += 2) {
-                    Sa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[PA_[q]], qf[PB_[q]], Sa, 0, 0, 0);
-                    Sb = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[PA_[q + 1]], qf[PB_[q + 1]], Sb, 0, 0, 0);
+                for (int kt = 0; kt < KT; ++kt) {
+                    bf16x8 kf[3];
+#pragma unroll
+                    for (int p = 0; p < 3; ++p)
+                        kf[p] = __builtin_bit_cast(bf16x8, *(const v4u *)&Ks[p][32 * kt + c][ks * 16 + half * 8]);
+#pragma unroll
+                    for (int q = 0; q < 6; q += 2) {
+                        Sa[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[PA_[q]], qf[PB_[q]], Sa[kt], 0, 0, 0);
+                        Sb[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[PA_[q + 1]], qf[PB_[q + 1]], Sb[kt], 0, 0, 0);
+                    }
                 }
             }
 
-            // softmax of this lane's row, in the lane: 16 of the tile's 32 keys here, 16 in lane ^ 32
-            float sc[16];
+            // softmax of this lane's row, in the lane: half of the trip's keys here, half in lane ^ 32
+            float sc[16 * KT];
             float m_tile = -INFINITY;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int j = j0 + 8 * (r >> 2) + 4 * half + (r & 3);
-                const bool valid = j < L && (!a.causal || j <= my_pos);
-                sc[r] = valid ? Sa[r] + Sb[r] : -INFINITY;
-                m_tile = fmaxf(m_tile, sc[r]);
-            }
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int j = j0 + 32 * kt + 8 * (r >> 2) + 4 * half + (r & 3);
+                    const bool valid = j < L && (!a.causal || j <= my_pos);
+                    sc[16 * kt + r] = valid ? Sa[kt][r] + Sb[kt][r] : -INFINITY;
+                    m_tile = fmaxf(m_tile, sc[16 * kt + r]);
+                }
             m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
             const float m_new = fmaxf(m_run, m_tile);
             const float m_ref = m_new > -INFINITY ? m_new : 0.f;  // nothing visible yet: every weight below is exp2(-inf) = 0
@@ -191,7 +202,7 @@ __global__ __launch_bounds__(FA_THREADS) void attn_prefill_bf16x3_kernel(AttnPre
             m_run = m_new;
             float psum = 0.f;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
+            for (int r = 0; r < 16 * KT; ++r) {
                 sc[r] = fast_exp2(sc[r] - m_ref);
                 psum += sc[r];
             }
@@ -201,10 +212,10 @@ __global__ __launch_bounds__(FA_THREADS) void attn_prefill_bf16x3_kernel(AttnPre
 #pragma unroll
                 for (int r = 0; r < 16; ++r) O[t][r] *= alpha;
 
-            // O^T += V^T P^T: P^T is this lane's 16 weights, already where the B operand wants them
+            // O^T += V^T P^T: P^T is this lane's weights, already where the B operand wants them
             // (registers 8 ks .. 8 ks + 7 are the keys at positions 16 ks + 8 half .. + 7 of V^T)
 #pragma unroll
-            for (int ks = 0; ks < FA_KEYS / 16; ++ks) {
+            for (int ks = 0; ks < KEYS / 16; ++ks) {
                 bf16x8 pf[3];
                 {
                     v2u lo[3], hi[3];
@@ -249,7 +260,7 @@ static int launch_fa_d(lumen_ctx *ctx, const AttnPrefillArgs &a) {
     const int nrep = a.hq / a.hkv;
     dim3 block(FA_THREADS);
 #define LAUNCH_FA(NR)                                                                                    \
-    hipLaunchKernelGGL((attn_prefill_bf16x3_kernel<D, NR>), dim3((a.s + FA_ROWS / NR - 1) / (FA_ROWS / NR), a.hkv, a.b), \
+    hipLaunchKernelGGL((attn_prefill_bf16x3_kernel<D, NR, (D == 64 ? 2 : 1)>), dim3((a.s + FA_ROWS / NR - 1) / (FA_ROWS / NR), a.hkv, a.b), \
                        block, 0, ctx->stream, a)
     switch (nrep) {
         case 1: LAUNCH_FA(1); break;
@@ -259,7 +270,7 @@ static int launch_fa_d(lumen_ctx *ctx, const AttnPrefillArgs &a) {
         default: {  // any other group size: one query head per grid row, its KV head = head / n_rep
             AttnPrefillArgs b = a;
             b.kv_div = nrep;
-            hipLaunchKernelGGL((attn_prefill_bf16x3_kernel<D, 1>), dim3((a.s + FA_ROWS - 1) / FA_ROWS, a.hq, a.b), block, 0,
+            hipLaunchKernelGGL((attn_prefill_bf16x3_kernel<D, 1, (D == 64 ? 2 : 1)>), dim3((a.s + FA_ROWS - 1) / FA_ROWS, a.hq, a.b), block, 0,
                                ctx->stream, b);
         }
     }
