@@ -313,17 +313,20 @@ def prefill_bench(args):
     for name, a in synth.iter_params(cfg, seed=0):
         model.set_param(name, a)
     ids = synth.make_tokens(S, cfg["vocab_size"], seed=0)
+    # five passes in a row: the first sizes the workspaces and the GPU clock settles over the first three
+    # (they run about 10 % slower); the figure is the mean of the last two
     passes = []
-    for _ in range(3):
+    for _ in range(5):
         model.reset_kv_caches()
         model.ctx.timer_start()
         model.forward(ids, all_rows=False)
         passes.append(model.ctx.timer_stop())
-    out = {"metric": "prompt tokens/s", "value": round(S / passes[-1] * 1e3, 1), "unit": "tokens/s", "n_gpus": 1,
-           "dtype": "f32", "data": "synthetic",
+    ms = 0.5 * (passes[-1] + passes[-2])
+    out = {"metric": "prompt tokens/s", "value": round(S / ms * 1e3, 1), "unit": "tokens/s", "n_gpus": 1,
+           "dtype": "f32", "data": "synthetic", "warmup": 3, "steps": 2,
            "config": {"workload": "TinyLlama-1.1B-shaped Llama fp32 random-init seed 0, batch 1, one prompt pass of %d "
                                   "random ids into an empty cache of %d rows" % (S, cfg["max_seq_len"])}}
-    out.update(prefill_report(cfg, S, passes[-1]))
+    out.update(prefill_report(cfg, S, ms))
     out["passes_ms"] = [round(x, 3) for x in passes]
     print(json.dumps(out))
 

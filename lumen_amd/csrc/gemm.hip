@@ -12,10 +12,12 @@
 // 2.6x the f32 matrix rate for f32 weights, 5.3x for bf16 weights; measured against an fp64
 // product the error is the same as with the f32 instruction (2e-7 .. 2e-6 of the largest element).
 //
-// When the tile grid alone cannot fill the chip (prompt of a few hundred tokens against a 2048-row
-// weight) the K range is split over gridDim.z; each split writes its partial tile to a workspace
-// and a second kernel adds the splits in index order and applies the epilogue, so the result does
-// not depend on scheduling.
+// Two tile shapes: 128x128 (two workgroups per compute unit) for prompts of up to about a thousand
+// rows, 256x256 (one workgroup per compute unit, 4x4 register tiles) above.  When the tile grid alone
+// cannot fill the chip (prompt of a few hundred tokens against a 2048-row weight, or 128 large tiles
+// on 256 compute units) the K range is split over gridDim.z; each split writes its partial tile to
+// a workspace and a second kernel adds the splits in index order and applies the epilogue, so the
+// result does not depend on scheduling.
 #include "internal.h"
 
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -200,6 +202,180 @@ __global__ __launch_bounds__(256) void gemm_bf16x3_kernel(GemmArgs a) {
     store_tile<EPI, PARTIAL>(a, acc, bm, bn, wm, wn, lane);
 }
 
+// Large products (thousands of prompt rows against thousands of weight rows): 256x256 output tile, 4
+// wavefronts x (4x4) tiles of 32x32 -- all 256 accumulator registers of a wavefront -- over 16-deep
+// slices.  A 4x4 register tile reads half the LDS bytes per matrix instruction of the 2x2 one, which is
+// what bounds the 128x128 kernel, and meets one barrier per 96 matrix instructions instead of two per 48.
+// One workgroup per compute unit: the split of slice s+1 into the other half of a double-buffered LDS
+// and the loads of slice s+2 stand in the same block as the matrix instructions of slice s, which
+// shadow them.  LDS rows are the 16 bf16 of a slice (32 bytes): operand reads and staging writes of a
+// wavefront are contiguous, so no swizzle is needed.
+#define GB_M 256
+#define GB_N 256
+#define GB_K 16
+
+template <int EPI, bool PARTIAL>
+__device__ __forceinline__ void store_big_tile(const GemmArgs &a, const v16f (&acc)[4][4], int bm, int bn, int wm, int wn,
+                                               int lane) {
+    const int M = a.M, N = a.N;
+    float *part = PARTIAL ? a.part + (size_t)blockIdx.z * M * N : nullptr;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = bm + wm * 128 + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+                const int col = bn + wn * 128 + j * 32 + (lane & 31);
+                const float v = acc[i][j][r];
+                if (PARTIAL) {
+                    if (row < M && col < N) part[(size_t)row * N + col] = v;
+                } else if (EPI == EPI_SWIGLU) {
+                    const float up = __shfl_xor(v, 1, 64);
+                    if (!(col & 1) && row < M && col < N) a.C[(size_t)row * (N >> 1) + (col >> 1)] = silu_g(v) * up;
+                } else if (row < M && col < N) {
+                    const size_t o = (size_t)row * N + col;
+                    a.C[o] = (EPI == EPI_RESIDUAL) ? a.residual[o] + v : v;
+                }
+            }
+}
+
+template <bool WBF16, int EPI, bool PARTIAL>
+__global__ __launch_bounds__(256, 1) void gemm_bf16x3_big_kernel(GemmArgs a) {
+    constexpr int PW = WBF16 ? 1 : 3;
+    constexpr int AST = 4;                // 16-byte pieces of A per thread per slice: 256 rows x 16 k / 256 threads
+    constexpr int WST = WBF16 ? 2 : 4;
+    __shared__ __align__(16) uint16_t As[2][3][GB_M][GB_K];
+    __shared__ __align__(16) uint16_t Ws[2][PW][GB_N][GB_K];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int bm = blockIdx.y * GB_M, bn = blockIdx.x * GB_N;
+    const int M = a.M, N = a.N, K = a.K;
+    const float *A = a.A;
+    // this workgroup's share of K: whole slices, [kb, ke)
+    const int slices = K / GB_K;
+    const int per = (slices + (int)gridDim.z - 1) / (int)gridDim.z;
+    const int kb = min((int)blockIdx.z * per, slices) * GB_K;
+    const int ke = min(K, kb + per * GB_K);
+
+    v16f acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    v4f va[AST];
+    v4u vw[WST];
+    // A and f32 W: piece i of this thread is row (tid + 256 i) / 4, k offset 4 * ((tid + 256 i) % 4);
+    // bf16 W: row (tid + 256 i) / 2, k offset 8 * ((tid + 256 i) % 2).  No branches: K is a multiple of
+    // the slice, rows past the end are clamped to the last one (their products are never stored).
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < AST; ++i) {
+            const int idx = tid + i * 256;
+            const int row = min(bm + (idx >> 2), M - 1), k4 = (idx & 3) * 4;
+            va[i] = *(const v4f *)(A + (size_t)row * K + k0 + k4);
+        }
+#pragma unroll
+        for (int i = 0; i < WST; ++i) {
+            const int idx = tid + i * 256;
+            const int row = min(bn + (WBF16 ? idx >> 1 : idx >> 2), N - 1), kk = WBF16 ? (idx & 1) * 8 : (idx & 3) * 4;
+            if (WBF16) vw[i] = *(const v4u *)((const uint16_t *)a.W + (size_t)row * K + k0 + kk);
+            else vw[i] = *(const v4u *)((const float *)a.W + (size_t)row * K + k0 + kk);
+        }
+    };
+    // piece i of the fetched slice, split into LDS half b
+    auto stage_piece = [&](int b, int i) {
+        const int idx = tid + i * 256;
+        v2u pl[3];
+        split3(va[i], pl);
+#pragma unroll
+        for (int p = 0; p < 3; ++p) *(v2u *)&As[b][p][idx >> 2][(idx & 3) * 4] = pl[p];
+        if (WBF16) {
+            if (i < WST) *(v4u *)&Ws[b][0][idx >> 1][(idx & 1) * 8] = vw[i < WST ? i : 0];
+        } else {
+            split3((v4f){__uint_as_float(vw[i].x), __uint_as_float(vw[i].y), __uint_as_float(vw[i].z),
+                         __uint_as_float(vw[i].w)}, pl);
+#pragma unroll
+            for (int p = 0; p < PW; ++p) *(v2u *)&Ws[b][p][idx >> 2][(idx & 3) * 4] = pl[p];
+        }
+    };
+    const int c = lane & 31, g8 = (lane >> 5) * 8;
+    // The matrix instructions of the slice in LDS half b.  With with_stage, piece j of the next slice is
+    // split into the other half one bf16 plane at a time, a plane after every four matrix instructions of
+    // column tile j, so that the vector ALU works in their shadow.
+    auto mma = [&](int b, bool with_stage) {
+        bf16x8 af[4][3];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int p = 0; p < 3; ++p)
+                af[i][p] = __builtin_bit_cast(bf16x8, *(const v4u *)&As[b][p][wm * 128 + i * 32 + c][g8]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            bf16x8 wf[PW];
+#pragma unroll
+            for (int p = 0; p < PW; ++p)
+                wf[p] = __builtin_bit_cast(bf16x8, *(const v4u *)&Ws[b][p][wn * 128 + j * 32 + c][g8]);
+            constexpr int NPROD = WBF16 ? 3 : 6;
+            constexpr int PA_[6] = {2, 0, 1, 1, 0, 0}, PW_[6] = {0, 2, 1, 0, 1, 0};
+            const int idx = tid + j * 256;
+            float ra[4] = {va[j].x, va[j].y, va[j].z, va[j].w};
+            float rw[4] = {__uint_as_float(vw[WBF16 ? 0 : j].x), __uint_as_float(vw[WBF16 ? 0 : j].y),
+                           __uint_as_float(vw[WBF16 ? 0 : j].z), __uint_as_float(vw[WBF16 ? 0 : j].w)};
+#pragma unroll
+            for (int q = 0; q < NPROD; ++q) {
+                const int xa = WBF16 ? 2 - q : PA_[q], xw = WBF16 ? 0 : PW_[q];
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i][xa], wf[xw], acc[i][j], 0, 0, 0);
+                if (with_stage) {
+                    const int p = q % 3;
+                    float *src = q < 3 ? ra : rw;
+                    uint16_t *dst = q < 3 ? &As[b ^ 1][p][idx >> 2][(idx & 3) * 4] : &Ws[b ^ 1][p][idx >> 2][(idx & 3) * 4];
+                    *(v2u *)dst = (v2u){pack_hi(src[1], src[0]), pack_hi(src[3], src[2])};
+                    if (p < 2) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) src[e] -= __uint_as_float(__float_as_uint(src[e]) & 0xffff0000u);
+                    }
+                    if (WBF16 && q == 0 && j < WST) *(v4u *)&Ws[b ^ 1][0][idx >> 1][(idx & 1) * 8] = vw[j < WST ? j : 0];
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one matrix instruction,
+                        __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);  // three vector ALU instructions in its shadow
+                    }
+                    __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);      // the plane's LDS write
+                }
+            }
+        }
+    };
+
+    // slice s is multiplied from LDS half s & 1 while slice s+1 is split into the other half (last read
+    // before the barrier that ended the previous trip) and slice s+2 travels from memory
+    if (kb < ke) {
+        fetch(kb);
+#pragma unroll
+        for (int i = 0; i < AST; ++i) stage_piece(0, i);
+        if (kb + GB_K < ke) fetch(kb + GB_K);
+        __syncthreads();
+        int k0 = kb, b = 0;
+        for (; k0 + 2 * GB_K < ke; k0 += GB_K, b ^= 1) {
+            mma(b, true);
+            fetch(k0 + 2 * GB_K);
+            __syncthreads();
+        }
+        if (k0 + GB_K < ke) {
+            mma(b, true);
+            __syncthreads();
+            b ^= 1;
+        }
+        mma(b, false);
+    }
+    store_big_tile<EPI, PARTIAL>(a, acc, bm, bn, wm, wn, lane);
+}
+
 // Adds the K splits of every output element in split order and applies the epilogue.
 template <int EPI>
 __global__ __launch_bounds__(256) void gemm_reduce_kernel(GemmArgs a, int splits) {
@@ -253,6 +429,19 @@ static void launch_gemm_epi(const GemmArgs &a, dim3 grid, hipStream_t s) {
     }
 }
 
+template <bool BF16>
+static void launch_gemm_big(const GemmArgs &a, dim3 grid, hipStream_t s) {
+    if (grid.z > 1) {
+        hipLaunchKernelGGL((gemm_bf16x3_big_kernel<BF16, EPI_STORE, true>), grid, dim3(256), 0, s, a);
+        return;
+    }
+    switch (a.epi) {
+        case EPI_STORE: hipLaunchKernelGGL((gemm_bf16x3_big_kernel<BF16, EPI_STORE, false>), grid, dim3(256), 0, s, a); break;
+        case EPI_RESIDUAL: hipLaunchKernelGGL((gemm_bf16x3_big_kernel<BF16, EPI_RESIDUAL, false>), grid, dim3(256), 0, s, a); break;
+        default: hipLaunchKernelGGL((gemm_bf16x3_big_kernel<BF16, EPI_SWIGLU, false>), grid, dim3(256), 0, s, a); break;
+    }
+}
+
 static void launch_gemm_reduce(const GemmArgs &a, int splits, int blocks, hipStream_t s) {
     switch (a.epi) {
         case EPI_STORE: hipLaunchKernelGGL(gemm_reduce_kernel<EPI_STORE>, dim3(blocks), dim3(256), 0, s, a, splits); break;
@@ -275,6 +464,30 @@ static int gemm_splits(const lumen_ctx *ctx, const GemmArgs &a) {
     return s < 1 ? 1 : (int)s;
 }
 
+// K splits (1 to 4) for the 256x256 kernel, or 0 where the 128x128 kernel is to run.  The large tile
+// pays from about a thousand rows of A on, when its workgroups -- one per compute unit at a time --
+// come in nearly whole rounds: the smallest split that fills 90 % of its last round, else the best
+// of them if that fills 80 %.  A split keeps at least 512 of K and the partial tiles within the
+// workspace limit.
+static int gemm_big_splits(const lumen_ctx *ctx, const GemmArgs &a) {
+    if (a.M < 1024 || a.K % GB_K != 0) return 0;
+    const long tiles = (long)((a.N + GB_N - 1) / GB_N) * ((a.M + GB_M - 1) / GB_M);
+    const long cus = ctx->num_cus;
+    int best = 0;
+    double best_fill = 0.0;
+    for (int s = 1; s <= 4; ++s) {
+        if (s > 1 && (a.K / s < 512 || (size_t)s * a.M * a.N * sizeof(float) > ((size_t)256 << 20))) break;
+        const long w = tiles * s, rounds = (w + cus - 1) / cus;
+        const double fill = (double)w / (double)(rounds * cus);
+        if (fill >= 0.9) return s;
+        if (fill > best_fill) {
+            best_fill = fill;
+            best = s;
+        }
+    }
+    return best_fill >= 0.8 ? best : 0;
+}
+
 int launch_gemm(lumen_ctx *ctx, const GemmArgs &a) {
     if (a.M <= 0 || a.N <= 0) return LUMEN_OK;
     const bool aligned = (((uintptr_t)a.A | (uintptr_t)a.W) & 15) == 0;
@@ -292,7 +505,9 @@ int launch_gemm(lumen_ctx *ctx, const GemmArgs &a) {
     }
     if (a.epi == EPI_SWIGLU && (a.N & 1)) LUMEN_FAIL(LUMEN_ERR_SHAPE, "SwiGLU epilogue needs an even column count, got %d", a.N);
     GemmArgs g = a;
-    const int splits = gemm_splits(ctx, a);
+    int splits = gemm_big_splits(ctx, a);
+    const bool big = splits > 0;
+    if (!big) splits = gemm_splits(ctx, a);
     if (splits > 1) {
         const size_t need = (size_t)splits * a.M * a.N * sizeof(float);
         if (ctx->gemm_ws_bytes < need) {
@@ -306,8 +521,15 @@ int launch_gemm(lumen_ctx *ctx, const GemmArgs &a) {
         g.part = ctx->gemm_ws;
     }
     dim3 grid((a.N + BN - 1) / BN, (a.M + BM - 1) / BM, splits);
-    if (a.w_bf16) launch_gemm_epi<true>(g, grid, ctx->stream);
-    else launch_gemm_epi<false>(g, grid, ctx->stream);
+    if (big) {
+        dim3 bgrid((a.N + GB_N - 1) / GB_N, (a.M + GB_M - 1) / GB_M, splits);
+        if (a.w_bf16) launch_gemm_big<true>(g, bgrid, ctx->stream);
+        else launch_gemm_big<false>(g, bgrid, ctx->stream);
+    } else if (a.w_bf16) {
+        launch_gemm_epi<true>(g, grid, ctx->stream);
+    } else {
+        launch_gemm_epi<false>(g, grid, ctx->stream);
+    }
     LUMEN_CHECK_LAUNCH();
     if (splits > 1) {
         size_t blocks = ((size_t)a.M * a.N + 255) / 256;

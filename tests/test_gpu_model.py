@@ -335,3 +335,18 @@ def test_llama2_7b_shape_bf16_weights_prefill_512_decode():
     cfg.pop("weight_dtype")
     gpu, ora = _stream_build(cfg, seed=5, bf16=True)
     _prefill_decode_check(gpu, ora, cfg["vocab_size"], 512, 8, 2e-2, seed=5)
+
+
+@pytest.mark.slow
+@pytest.mark.parametrize("bf16,tol", [(False, 1e-4), (True, 2e-2)])
+def test_wide_model_prompt_of_4000_rows_on_the_large_gemm_tiles(bf16, tol):
+    """A prompt of 4000 rows against projections 3328 and 3840 rows wide: q|k|v and o_proj then run on the
+    256x256 GEMM tiles without a K split, i.e. with the plain store and the residual add in the tile
+    epilogue (TinyLlama's own widths split K there and add in a second pass), with f32 and with bf16-stored
+    weights.  One layer, 52 query heads on 4 KV heads."""
+    cfg = dict(vocab_size=256, hidden_size=3328, intermediate_size=256, num_hidden_layers=1,
+               num_attention_heads=52, num_key_value_heads=4, rms_norm_eps=1e-5, max_seq_len=4096,
+               rope_theta=10000.0)
+    gpu, ora = _stream_build(cfg, seed=6, bf16=bf16)
+    _prefill_decode_check(gpu, ora, cfg["vocab_size"], 4000, 2, tol, seed=6)
+

@@ -119,6 +119,36 @@ def test_gemm_bf16_weights():
     assert max_rel(C, lo.gemm(A, lo.bf16_to_f32(bits))) <= 1e-5
 
 
+@pytest.mark.parametrize("M,N,K,bf16", [
+    (1030, 13000, 528, False),   # 5 x 51 large tiles, no K split; ragged rows and columns, an odd number of slices
+    (1100, 2816, 2048, False),   # 55 large tiles: K split in four, partial tiles added in a second pass
+    (1024, 7424, 1040, True),    # bf16-stored weight, K split in two unequal shares (33 and 32 slices)
+    (1500, 10496, 272, True),    # bf16-stored weight, no K split, 17 slices
+])
+def test_gemm_with_a_thousand_rows_and_more(M, N, K, bf16):
+    """From 1024 rows of A on the product may run on 256x256 tiles (one workgroup per compute unit, K split up to
+    four ways): same values as the fp64 product to 1e-5 of the largest element, and every row equal to the
+    vector-matrix product of that row alone (src/ops/matmul.rs:42-69 against :70-92) within the same bound."""
+    A = f32(RNG.normal(0, 1, (M, K)))
+    W = f32(RNG.normal(0, 0.02, (N, K)))
+    if bf16:
+        bits = lo.f32_to_bf16(W)
+        W = lo.bf16_to_f32(bits)
+        C = ops.matmul(dev(A[None]), dev(bits)).data()[0]
+    else:
+        C = ops.matmul(dev(A[None]), dev(W)).data()[0]
+    assert C.shape == (M, N) and np.isfinite(C).all()
+    ref = A.astype(np.float64) @ W.astype(np.float64).T
+    assert max_rel(C, ref) <= 1e-5
+    # per element, against the size of its own terms: an f32 dot product of this length is good to a few 1e-7
+    size = np.abs(A).astype(np.float64) @ np.abs(W).astype(np.float64).T
+    assert (np.abs(C - ref) / size).max() <= 1e-6
+    Wd = dev(bits) if bf16 else dev(W)
+    for row in (0, 255, 256, M - 1):
+        y = ops.matmul(dev(A[row][None]), Wd).data()[0]
+        assert max_rel(C[row], y) <= 1e-5
+
+
 @pytest.mark.parametrize("rows,dim,eps", [(1, 2048, 1e-5), (7, 100, 1e-6), (128, 2048, 1e-5), (3, 1, 1e-5)])
 def test_rmsnorm(rows, dim, eps):
     x = f32(RNG.normal(0, 2, (rows, dim)))
