@@ -55,15 +55,6 @@ __device__ __forceinline__ void fa_split4(const v4f x, v2u (&part)[3]) {
         }
     }
 }
-// one value -> its three parts
-__device__ __forceinline__ void fa_split1(float x, uint16_t (&part)[3]) {
-#pragma unroll
-    for (int p = 0; p < 3; ++p) {
-        part[p] = (uint16_t)(__float_as_uint(x) >> 16);
-        if (p < 2) x -= __uint_as_float(__float_as_uint(x) & 0xffff0000u);
-    }
-}
-
 // KT: key tiles of 32 per trip of the loop (2 for head_dim 64: one barrier pair, one row maximum and one rescale of
 // O per 64 keys; 1 for head_dim 128, whose K and V tiles fill LDS twice as fast).
 template <int D, int NREP, int KT>
@@ -119,6 +110,14 @@ __global__ __launch_bounds__(FA_THREADS, (D == 64 ? 2 : 1)) void attn_prefill_bf
         for (int r = 0; r < 16; ++r) O[t][r] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;  // of this lane's row; l over this lane's half of the keys
 
+    // V^T is staged with bits 2 and 3 of the key index exchanged: the 8 keys a lane holds of S^T (4 + 4,
+    // eight apart) then sit next to each other for the 16-byte operand read.  A thread takes 4 elements
+    // (v_k4 ..) of the 4 keys that land on positions 4 v_g .. 4 v_g + 3 -- consecutive keys from v_key on --
+    // so that one element of the four keys is one 8-byte LDS write.
+    static_assert(PIECES == 4, "a thread stages four keys of V");
+    constexpr int NG = KEYS / 4;  // groups of four key positions
+    const int v_g = (tid >> 2) % NG, v_k4 = ((tid / (4 * NG)) * 4 + (tid & 3)) * 4;
+    const int v_key = 4 * ((v_g & ~3) | ((v_g & 1) << 1) | ((v_g >> 1) & 1));
     v4f kreg[PIECES], vreg[PIECES];
     auto fetch = [&](int j0) {
 #pragma unroll
@@ -127,7 +126,7 @@ __global__ __launch_bounds__(FA_THREADS, (D == 64 ? 2 : 1)) void attn_prefill_bf
             const int key = idx / (D / 4), k4 = (idx % (D / 4)) * 4;
             const int j = min(j0 + key, L - 1);  // keys past L are masked below
             kreg[p] = *(const v4f *)(Kc + (size_t)j * D + k4);
-            vreg[p] = *(const v4f *)(Vc + (size_t)j * D + k4);
+            vreg[p] = *(const v4f *)(Vc + (size_t)min(j0 + v_key + p, L - 1) * D + v_k4);
         }
     };
 
@@ -142,17 +141,13 @@ __global__ __launch_bounds__(FA_THREADS, (D == 64 ? 2 : 1)) void attn_prefill_bf
             fa_split4(kreg[p], kp);
 #pragma unroll
             for (int q = 0; q < 3; ++q) *(v2u *)&Ks[q][key][k4] = kp[q];
-            // V^T, with bits 2 and 3 of the key index exchanged: the 8 keys a lane holds of S^T
-            // (4 + 4, eight apart) then sit next to each other for the 16-byte operand read
-            const int kpos = (key & ~12) | ((key & 4) << 1) | ((key & 8) >> 1);
-            const float ve[4] = {vreg[p].x, vreg[p].y, vreg[p].z, vreg[p].w};
+        }
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                uint16_t vp[3];
-                fa_split1(ve[e], vp);
+        for (int e = 0; e < 4; ++e) {
+            v2u vp[3];
+            fa_split4((v4f){vreg[0][e], vreg[1][e], vreg[2][e], vreg[3][e]}, vp);
 #pragma unroll
-                for (int q = 0; q < 3; ++q) Vt[q][k4 + e][kpos] = vp[q];
-            }
+            for (int q = 0; q < 3; ++q) *(v2u *)&Vt[q][v_k4 + e][4 * v_g] = vp[q];
         }
         __syncthreads();
         if (j0 + KEYS < kmax) fetch(j0 + KEYS);  // in flight during the matrix instructions below
