@@ -101,6 +101,8 @@ __global__ __launch_bounds__(FA_THREADS, (D == 64 ? 2 : 1)) void attn_prefill_bf
     const int kmax = a.causal ? min(L, a.past_len + q_last + 1) : L;
     const int wave_i_last = min(q0 + (wave * 32 + 31) / NREP, a.s - 1);
     const int wave_kmax = a.causal ? min(L, a.past_len + wave_i_last + 1) : L;
+    // keys [0, wave_kfull) are visible to every row of this wavefront: no mask needed below it
+    const int wave_kfull = a.causal ? min(L, a.past_len + q0 + (wave * 32) / NREP + 1) : L;
 
     // O^T: register r of tile t belongs to element 32 t + 8 (r / 4) + 4 half + r % 4 of this lane's row
     v16f O[DT];
@@ -181,15 +183,25 @@ __global__ __launch_bounds__(FA_THREADS, (D == 64 ? 2 : 1)) void attn_prefill_bf
             // softmax of this lane's row, in the lane: half of the trip's keys here, half in lane ^ 32
             float sc[16 * KT];
             float m_tile = -INFINITY;
+            if (j0 + KEYS <= wave_kfull) {  // uniform per wavefront: every key of the trip is visible to every row
 #pragma unroll
-            for (int kt = 0; kt < KT; ++kt)
+                for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int j = j0 + 32 * kt + 8 * (r >> 2) + 4 * half + (r & 3);
-                    const bool valid = j < L && (!a.causal || j <= my_pos);
-                    sc[16 * kt + r] = valid ? Sa[kt][r] + Sb[kt][r] : -INFINITY;
-                    m_tile = fmaxf(m_tile, sc[16 * kt + r]);
-                }
+                    for (int r = 0; r < 16; ++r) {
+                        sc[16 * kt + r] = Sa[kt][r] + Sb[kt][r];
+                        m_tile = fmaxf(m_tile, sc[16 * kt + r]);
+                    }
+            } else {
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int j = j0 + 32 * kt + 8 * (r >> 2) + 4 * half + (r & 3);
+                        const bool valid = j < L && (!a.causal || j <= my_pos);
+                        sc[16 * kt + r] = valid ? Sa[kt][r] + Sb[kt][r] : -INFINITY;
+                        m_tile = fmaxf(m_tile, sc[16 * kt + r]);
+                    }
+            }
             m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
             const float m_new = fmaxf(m_run, m_tile);
             const float m_ref = m_new > -INFINITY ? m_new : 0.f;  // nothing visible yet: every weight below is exp2(-inf) = 0
