@@ -79,7 +79,10 @@ int lumen_download(lumen_ctx *ctx, void *dst_host, const void *src_dev, size_t b
  * memory-bound GEMV (:42-69), M > 1 the MFMA GEMM (:70-92). */
 int lumen_matmul_f32(lumen_ctx *ctx, const float *A_dev, const float *W_dev, float *C_dev,
                      int M, int N, int K_a, int K_w);
-/* the two branches on their own */
+/* the two branches on their own.  The GEMM splits K over workgroups when its tile grid
+ * alone would not fill the chip; the partial tiles go to a workspace of the ctx (256 MiB at
+ * most) that grows, with a stream synchronisation and a hipMalloc, the first time a call
+ * needs more of it.  Results do not depend on scheduling (splits are added in index order). */
 int lumen_gemv_f32(lumen_ctx *ctx, const float *W_dev, const float *x_dev, float *y_dev, int N, int K);
 int lumen_gemm_f32(lumen_ctx *ctx, const float *A_dev, const float *W_dev, float *C_dev,
                    int M, int N, int K);
