@@ -178,10 +178,19 @@ __device__ __forceinline__ bool attn_decode_short(const AttnDecodeArgs &a, int r
     }
     wave_merge_publish<D, 1>(st, sm, sl, sacc);
     __syncthreads();
+    float *part0 = a.part + ((size_t)bb * a.hq + hq) * a.nsplit * (D + 2);  // slice 0 of this head
     for (int dd = threadIdx.x; dd < D; dd += THREADS) {
         float mm, ls, cx;
         wave_fold<D, 1, WAVES>(sm, sl, sacc, 0, dd, mm, ls, cx);
-        a.out[((size_t)bb * a.hq + hq) * D + dd] = cx * (1.0f / (ls + 1e-9f));  // self_attention.rs:287-290
+        if (a.defer_merge) {  // the consumer divides
+            part0[dd] = cx;
+            if (dd == 0) {
+                part0[D] = mm;
+                part0[D + 1] = ls;
+            }
+        } else {
+            a.out[((size_t)bb * a.hq + hq) * D + dd] = cx * (1.0f / (ls + 1e-9f));  // self_attention.rs:287-290
+        }
     }
     return true;
 }
@@ -327,7 +336,7 @@ __device__ __forceinline__ bool attn_decode_slice(const AttnDecodeArgs &a, int r
     for (int dd = t; dd < D; dd += THREADS) {
         float mm, ls, cx;
         wave_fold<D, 1, WAVES>(sm, sl, sacc, 0, dd, mm, ls, cx);
-        if (nact == 1) {
+        if (nact == 1 && !a.defer_merge) {
             out_head[dd] = cx * (1.0f / (ls + 1e-9f));  // self_attention.rs:287-290
         } else {
             float *pp = part_head + (size_t)slice * (D + 2);
@@ -338,7 +347,7 @@ __device__ __forceinline__ bool attn_decode_slice(const AttnDecodeArgs &a, int r
             }
         }
     }
-    if (nact == 1) return true;
+    if (nact == 1 || a.defer_merge) return true;  // one slice, or the consumer folds them
     // The barrier makes every wavefront wait for its own stores before thread 0 signals.
     __syncthreads();
     if (t == 0) {
@@ -473,6 +482,9 @@ int attn_decode_nsplit(int max_seq, int d) {
 
 size_t attn_decode_part_floats(int b, int hq, int d, int nsplit) { return (size_t)b * hq * nsplit * (d + 2); }
 
+int attn_decode_trip_rows(int d) { return 16384 / d; }
+int attn_decode_short_rows(int d) { return 2 * attn_decode_trip_rows(d) < ATTN_SHORT_ROWS ? 2 * attn_decode_trip_rows(d) : ATTN_SHORT_ROWS; }
+
 template <int D>
 static int launch_decode_d(lumen_ctx *ctx, const AttnDecodeArgs &a) {
     constexpr int WAVES = DecodeWaves<D>::value;
@@ -501,6 +513,8 @@ static int launch_decode_d(lumen_ctx *ctx, const AttnDecodeArgs &a) {
 
 int launch_attn_decode(lumen_ctx *ctx, const AttnDecodeArgs &a) {
     if (a.hkv <= 0 || a.hq % a.hkv) LUMEN_FAIL(LUMEN_ERR_SHAPE, "heads %d not a multiple of kv heads %d", a.hq, a.hkv);
+    if (a.defer_merge && (!a.pre_rotated || a.max_seq > a.nsplit * attn_decode_trip_rows(a.d)))
+        LUMEN_FAIL(LUMEN_ERR_INVALID, "decode attention: a deferred merge needs a rotated q and one-trip slices");
     switch (a.d) {
         case 16: return launch_decode_d<16>(ctx, a);
         case 32: return launch_decode_d<32>(ctx, a);

@@ -93,6 +93,57 @@ __device__ __forceinline__ void stage_x(float *xs, const float *__restrict__ x, 
     __syncthreads();
 }
 
+// Stages the decode attention output from the attention kernel's partial states: head h, element d is
+// sum_s w_s ctx_s[d] / (sum_s w_s l_s + 1e-9) with w_s = exp2(m_s - max m) over the slices in use
+// (self_attention.rs:287-290 after the merge of the slices' online-softmax states).  A thread's loads
+// are independent of each other: one trip to memory after the position is known.  Slices not in use
+// hold whatever an earlier step left there: they are never read (the index is clamped to the last one
+// in use and its weight forced to zero).  All threads of the workgroup must call it.
+#define GEMV_FOLD_MAX_SLICES 16
+typedef float v2f __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void stage_attn_fold(float *xs, const GemvArgs &a, int K, int kpad) {
+    const int tid = threadIdx.x, nthreads = blockDim.x;
+    const int D = a.attn_d, S = a.attn_nslices, stride = D + 2;
+    const int rows = *a.attn_pos + 1;
+    int nact = 1;
+    if (rows > a.attn_short_rows) nact = min(S, (rows + a.attn_trip - 1) / a.attn_trip);
+    for (int k = tid * 4; k < kpad; k += nthreads * 4) {
+        v4f v = {0.f, 0.f, 0.f, 0.f};
+        if (k < K) {
+            const float *ph = a.attn_part + (size_t)(k / D) * S * stride;
+            const int d = k % D;
+            float m[GEMV_FOLD_MAX_SLICES], l[GEMV_FOLD_MAX_SLICES];
+            v2f c0[GEMV_FOLD_MAX_SLICES], c1[GEMV_FOLD_MAX_SLICES];
+#pragma unroll
+            for (int s = 0; s < GEMV_FOLD_MAX_SLICES; ++s) {
+                const float *pp = ph + (size_t)min(s, nact - 1) * stride;
+                m[s] = pp[D];
+                l[s] = pp[D + 1];
+                c0[s] = *(const v2f *)(pp + d);  // rows of D + 2 floats: 8-byte aligned
+                c1[s] = *(const v2f *)(pp + d + 2);
+            }
+            float M = -INFINITY;
+#pragma unroll
+            for (int s = 0; s < GEMV_FOLD_MAX_SLICES; ++s)
+                if (s < nact) M = fmaxf(M, m[s]);
+            float L = 0.f;
+#pragma unroll
+            for (int s = 0; s < GEMV_FOLD_MAX_SLICES; ++s) {
+                const float w = (s < nact && m[s] > -INFINITY) ? __builtin_amdgcn_exp2f(m[s] - M) : 0.f;
+                L = fmaf(l[s], w, L);
+                v.x = fmaf(c0[s].x, w, v.x);
+                v.y = fmaf(c0[s].y, w, v.y);
+                v.z = fmaf(c1[s].x, w, v.z);
+                v.w = fmaf(c1[s].y, w, v.w);
+            }
+            const float inv = 1.0f / (L + 1e-9f);
+            v.x *= inv; v.y *= inv; v.z *= inv; v.w *= inv;
+        }
+        *(v4f *)(xs + k) = v;
+    }
+    __syncthreads();
+}
+
 template <bool BF16, int R, int PRO, int EPI>
 __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(GemvArgs a) {
     extern __shared__ __align__(16) float xs[];
@@ -178,7 +229,8 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(GemvArgs a) {
         }
     };
     preload(gw);
-    stage_x<PRO>(xs, a.x + (a.x_sel ? sel_off : 0), a.norm_w, a.eps, K, kpad);
+    if (PRO == PRO_ATTN_FOLD) stage_attn_fold(xs, a, K, kpad);
+    else stage_x<PRO>(xs, a.x + (a.x_sel ? sel_off : 0), a.norm_w, a.eps, K, kpad);
     float best = -INFINITY;
     int best_idx = 0x7fffffff;
 
@@ -383,7 +435,9 @@ static void launch_epi(const GemvArgs &a, dim3 grid, int threads, size_t lds, hi
 
 template <bool BF16, int R>
 static void launch_pro(const GemvArgs &a, dim3 grid, int threads, size_t lds, hipStream_t s) {
-    if (a.pro == PRO_RMSNORM)
+    if (a.pro == PRO_ATTN_FOLD)  // o_proj only (launch_gemv checks): one row per unit, residual epilogue
+        hipLaunchKernelGGL((gemv_kernel<BF16, 1, PRO_ATTN_FOLD, EPI_RESIDUAL>), grid, dim3(threads), lds, s, a);
+    else if (a.pro == PRO_RMSNORM)
         launch_epi<BF16, R, PRO_RMSNORM>(a, grid, threads, lds, s);
     else
         launch_epi<BF16, R, PRO_NONE>(a, grid, threads, lds, s);
@@ -398,7 +452,7 @@ int launch_gemv(lumen_ctx *ctx, const GemvArgs &a) {
     const int piece = 64 * vec * (8 / R);  // x is staged zero-padded to whole pieces
     const int kpad = (a.K + piece - 1) / piece * piece;
     const size_t lds = (size_t)kpad * sizeof(float);
-    const bool aligned = (((uintptr_t)a.W | (uintptr_t)a.x) & 15) == 0 &&
+    const bool aligned = (((uintptr_t)a.W | (uintptr_t)a.x) & 15) == 0 && (((uintptr_t)a.attn_part) & 7) == 0 &&
                          (a.pro != PRO_RMSNORM || ((uintptr_t)a.norm_w & 15) == 0);
     const bool fast = (a.K % vec == 0) && aligned && lds <= 64 * 1024;
     if (!fast) {
@@ -413,6 +467,12 @@ int launch_gemv(lumen_ctx *ctx, const GemvArgs &a) {
             hipLaunchKernelGGL(gemv_generic_kernel<false>, dim3(blocks), dim3(GEMV_THREADS), 0, ctx->stream, a);
         LUMEN_CHECK_LAUNCH();
         return LUMEN_OK;
+    }
+    if (a.pro == PRO_ATTN_FOLD) {
+        if (a.epi != EPI_RESIDUAL || R != 1 || !a.attn_part || !a.attn_pos || a.attn_d <= 0 || a.attn_d % 4 ||
+            a.K % a.attn_d || a.attn_nslices < 1 || a.attn_nslices > GEMV_FOLD_MAX_SLICES)
+            LUMEN_FAIL(LUMEN_ERR_INVALID, "GEMV over attention partials: one row per unit, residual epilogue, at most %d slices (got %d)",
+                       GEMV_FOLD_MAX_SLICES, a.attn_nslices);
     }
     if ((a.epi == EPI_SWIGLU || a.epi == EPI_ROPE_QKV) && (a.N & 1))
         LUMEN_FAIL(LUMEN_ERR_SHAPE, "paired-row epilogue needs an even row count, got %d", a.N);

@@ -71,7 +71,7 @@ struct lumen_kv_cache {
 // ---------------------------------------------------------------- launchers
 // Every launcher validates nothing: callers check shapes first.
 
-enum GemvPro { PRO_NONE = 0, PRO_RMSNORM = 1 };
+enum GemvPro { PRO_NONE = 0, PRO_RMSNORM = 1, PRO_ATTN_FOLD = 2 };
 enum GemvEpi { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2, EPI_ARGMAX = 3, EPI_ROPE_QKV = 4 };
 
 struct GemvArgs {
@@ -102,6 +102,12 @@ struct GemvArgs {
     const int *pos;
     float *k_cache, *v_cache;  // [hkv, max_seq, D]
     int hq, hkv, D, max_seq;
+    // PRO_ATTN_FOLD: x is the decode attention output [attn_hq * attn_d], still in the kernel's partial
+    // states attn_part [attn_hq][attn_nslices][attn_d + 2] (ctx, m, l).  With *attn_pos + 1 cached rows,
+    // slice 0 alone is in use up to attn_short_rows, else one slice per attn_trip rows.
+    const float *attn_part;
+    const int *attn_pos;
+    int attn_nslices, attn_d, attn_trip, attn_short_rows;
 };
 int launch_gemv(lumen_ctx *ctx, const GemvArgs &a);
 int gemv_max_blocks(const lumen_ctx *ctx);
@@ -150,6 +156,10 @@ struct AttnDecodeArgs {
     int nsplit;         // slices a long cache is cut into (attn_decode_nsplit)
     int pre_rotated;    // q is already rotated and row pos of the cache already written (fused QKV GEMV)
     int expect_short;   // hint: the cache is short (a few hundred rows); a wrong hint only costs time
+    // Leave the merge of a long cache's slices to the consumer: every workgroup stores its partial state
+    // (ctx[D], m, l) in `part` -- the short form in slice 0 -- and `out` is not written.  The o_proj GEMV
+    // folds the partials while it stages its input (PRO_ATTN_FOLD).  Needs pre_rotated and one-trip slices.
+    int defer_merge;
 };
 int launch_attn_decode(lumen_ctx *ctx, const AttnDecodeArgs &a);
 
@@ -176,5 +186,8 @@ int launch_attn_prefill_mfma(lumen_ctx *ctx, const AttnPrefillArgs &a);
 
 int attn_decode_nsplit(int max_seq, int d);
 size_t attn_decode_part_floats(int b, int hq, int d, int nsplit);
+// rows of one slice of a long cache, and the longest cache the one-workgroup-per-head form takes
+int attn_decode_trip_rows(int d);
+int attn_decode_short_rows(int d);
 
 void rope_tables_host(std::vector<float> &cos_t, std::vector<float> &sin_t, int dim, int max_seq, float theta);

@@ -228,7 +228,9 @@ def test_decode_modes_agree_with_each_other_and_the_oracle(cfg, bf16, n_prompt):
     (dict(num_attention_heads=8, num_key_value_heads=2, max_seq_len=600, qk_norm=True, head_dim=64), 507),  # norm in the kernel
     (dict(hidden_size=384, num_attention_heads=6, num_key_value_heads=2, max_seq_len=600, intermediate_size=1056), 508),  # groups of three heads
     (dict(hidden_size=128, num_attention_heads=2, num_key_value_heads=1, max_seq_len=4096, intermediate_size=352), 3900),  # 16 slices, all in use
-], ids=["d64-nrep8", "d64-nrep4", "d128-nrep2", "d64-qknorm", "d64-nrep3", "d64-long-4096"])
+    (dict(num_attention_heads=8, num_key_value_heads=2, max_seq_len=4096), 505),  # 16 slices offered, 1 to 3 in use: merged by o_proj
+    (dict(num_attention_heads=8, num_key_value_heads=2, max_seq_len=4096), 3),    # the same model from an almost empty cache
+], ids=["d64-nrep8", "d64-nrep4", "d128-nrep2", "d64-qknorm", "d64-nrep3", "d64-long-4096", "d64-4096-cross", "d64-4096-start"])
 def test_decode_across_the_short_to_split_attention_boundary(cfg_extra, n_prompt):
     """Decode attention changes form where the cache passes 512 rows (256 for head_dim 128): steps on both sides of
     the boundary, and the step that crosses it, agree with the checker."""
