@@ -44,7 +44,7 @@ struct lumen_llama {
     float *part = nullptr;
     int *counters = nullptr;
     int nsplit = 1;     // slices of a long cache in the decode attention kernel
-    bool defer_merge = false;  // the o_proj GEMV, not the attention kernel, merges the slices of a long cache
+    bool defer_merge = false;  // the o_proj GEMV, not the attention kernel, may merge the slices of a long cache
     int pk_nsplit = 1;  // the same for the persistent kernel (its own slicing: 64 rows per slice, 64 at most)
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
@@ -180,11 +180,11 @@ extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg,
     M_TRY(dmalloc_t(m, &m->d_pos, 4));
     M_TRY(dmalloc_t(m, &m->tok_hist, (size_t)cfg->max_seq_len + 1));
     m->nsplit = attn_decode_nsplit(cfg->max_seq_len, D);
-    // With 16 slices (caches of 2049-4096 rows at head_dim 64) the o_proj GEMV folds the slices' partial
-    // states while it stages its input: an atomic and a second round of loads fewer inside the attention
-    // kernel.  With more slices the partials would outweigh what the GEMV workgroups can re-read; with
-    // fewer the in-kernel merge is short.  q/k norm models rotate inside the attention kernel: not covered.
-    m->defer_merge = m->nsplit == 16 && !cfg->qk_norm && cfg->max_seq_len <= m->nsplit * attn_decode_trip_rows(D);
+    // Where a cache is cut into 2 to 16 slices the o_proj GEMV can fold the slices' partial states while it
+    // stages its input: an atomic and a second round of loads fewer inside the attention kernel.  With more
+    // slices the partials would outweigh what the GEMV workgroups can re-read.  q/k norm models rotate
+    // inside the attention kernel: not covered.  Used on the long side of the short-cache boundary only.
+    m->defer_merge = m->nsplit >= 2 && m->nsplit <= 16 && !cfg->qk_norm && cfg->max_seq_len <= m->nsplit * attn_decode_trip_rows(D);
     m->pk_nsplit = cfg->max_seq_len / 64 < 1 ? 1 : (cfg->max_seq_len / 64 > 64 ? 64 : cfg->max_seq_len / 64);
     M_TRY(dmalloc_t(m, &m->part, attn_decode_part_floats(1, Hq, D, m->nsplit > m->pk_nsplit ? m->nsplit : m->pk_nsplit)));
     M_TRY(dmalloc_t(m, &m->counters, (size_t)Hq));
@@ -450,7 +450,9 @@ static int enqueue_decode_step(lumen_llama *m, StepProbe *pr = nullptr) {
         a.scale = m->scale; a.q_norm_w = w.q_norm; a.k_norm_w = w.k_norm; a.norm_eps = c.rms_norm_eps;
         a.part = m->part; a.counters = m->counters; a.nsplit = m->nsplit; a.pre_rotated = fuse_rope;
         a.expect_short = expect_short_cache(m);
-        a.defer_merge = m->defer_merge;
+        // (a graph is captured anew when the hint changes sides, so the choice is the same for every launch of a step)
+        const bool defer = m->defer_merge && !a.expect_short;
+        a.defer_merge = defer;
         pr->before(KC_ATTN);
         LUMEN_TRY(launch_attn_decode(ctx, a));
         pr->after();
@@ -458,7 +460,7 @@ static int enqueue_decode_step(lumen_llama *m, StepProbe *pr = nullptr) {
         g = {};
         g.W = w.wo; g.x = m->attn; g.y = m->h; g.N = H; g.K = m->qd; g.w_bf16 = m->bf16;
         g.pro = PRO_NONE; g.epi = EPI_RESIDUAL; g.residual = m->x;
-        if (m->defer_merge) {
+        if (defer) {
             g.pro = PRO_ATTN_FOLD; g.attn_part = m->part; g.attn_pos = m->d_pos; g.attn_nslices = m->nsplit; g.attn_d = m->D;
             g.attn_trip = attn_decode_trip_rows(m->D); g.attn_short_rows = attn_decode_short_rows(m->D);
         }
