@@ -35,6 +35,9 @@ def main():
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--prompt", type=int, default=128)
+    ap.add_argument("--max-seq", type=int, default=2048,
+                    help="rows of the static KV cache (2048: the headline configuration; 4096 with --prompt 3968 "
+                         "--steps 32 is the long-context configuration)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--mode", choices=["graph", "eager"], default="graph",
                     help="how decode steps are issued: a HIP graph replay per token (default) or kernel by kernel "
@@ -64,7 +67,7 @@ def main():
     from lumen_amd import synth
     from lumen_amd.models import LlamaModel
 
-    cfg = dict(synth.TINYLLAMA_1B)
+    cfg = dict(synth.TINYLLAMA_1B, max_seq_len=args.max_seq)
     need = args.prompt + args.warmup + 3 * args.steps + 8
     if need > cfg["max_seq_len"]:
         sys.exit("bench.py: prompt + warmup + 3*steps = %d exceeds max_seq_len %d" % (need, cfg["max_seq_len"]))
@@ -136,6 +139,10 @@ def main():
             kernels[name] = {"avg_us": round(1e3 * (s_ms / n - event_overhead_ms), 3),
                              "launches_per_step": n // args.steps}
 
+    # decode attention: K and V rows of every KV head, read once per launch (mean cache length of the timed region)
+    at_ms, at_n = prof["attn_decode"]
+    at_avg_ms = at_ms / max(at_n, 1) - event_overhead_ms
+    at_bytes = 2.0 * cfg["num_key_value_heads"] * mean_len * 64 * 4
     out = {
         "metric": "batch-1 decode tokens/s", "value": round(tok_s, 2), "unit": "tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
@@ -153,6 +160,9 @@ def main():
         "step_roofline": {"bytes_per_token": step_bytes, "achieved_GBps": round(step_bytes / (ms_per_step * 1e-3) / 1e9, 1),
                           "frac_of_8TBps": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                           "roofline_tokens_per_s": round(HBM_PEAK_GBS * 1e9 / step_bytes, 1)},
+        "attention": {"kernel": "attn_decode_kernel<64, 8, 8, true>", "kv_bytes_per_launch": at_bytes,
+                      "avg_launch_us": round(at_avg_ms * 1e3, 3), "achieved_GBps": round(at_bytes / (at_avg_ms * 1e-3) / 1e9, 1),
+                      "frac_of_8TBps": round(at_bytes / (at_avg_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
         "kernels": kernels,
         "prefill": dict(prefill_report(cfg, args.prompt, prefill_ms), passes_ms=[round(x, 3) for x in prefill_all_ms]),
         "decode_mode": args.mode, "eager_ms_per_step": round(eager_ms / args.steps, 5),
