@@ -214,9 +214,9 @@ __global__ __launch_bounds__(256) void gemm_bf16x3_kernel(GemmArgs a) {
 //          is what bounds gemm_bf16x3_kernel.  For thousands of prompt rows.
 //   F = 2: 128x128, two or three workgroups per compute unit: the tile grid and K splits of
 //          gemm_bf16x3_kernel, for shorter prompts with f32 weights.
-#define GB_M 256
+#define GB_M 256  // the F = 4 tile
 #define GB_N 256
-#define GB_K 16
+#define GB_K 16   // slice depth of the pipelined kernel
 
 template <int EPI, bool PARTIAL, int F>
 __device__ __forceinline__ void store_wave_tiles(const GemmArgs &a, const v16f (&acc)[F][F], int bm, int bn, int wm, int wn,
