@@ -461,18 +461,30 @@ static void launch_gemm_reduce(const GemmArgs &a, int splits, int blocks, hipStr
     }
 }
 
-// K splits for a tile grid that does not fill the chip: enough workgroups for two per compute
-// unit, at least four 32-deep slices each, partial tiles within the workspace limit.
+// K splits for a 128x128 tile grid that does not fill the chip.  A compute unit works its workgroups off
+// one after the other as far as the matrix pipes are concerned, so what counts is the largest number of
+// workgroups any compute unit gets times the length of one: ceil(tiles * s / CUs) * (slices / s + a
+// fixed cost per workgroup for its first loads and its partial tile).  88 tiles of 128 slices: s = 6
+// makes 528 workgroups -- three for 16 of the compute units -- where s = 5 makes 440, two at most.
+// At least 128 of K per split, 16 splits at most, partial tiles within the workspace limit.
 static int gemm_splits(const lumen_ctx *ctx, const GemmArgs &a) {
     const long tiles = (long)((a.N + BN - 1) / BN) * ((a.M + BM - 1) / BM);
-    const long want = 2L * ctx->num_cus;
-    if (tiles * 4 >= want * 3) return 1;  // three quarters of the slots filled: a split would cost more in partial tiles than it gains
-    long s = (want + tiles - 1) / tiles;
-    const long max_by_k = a.K / (4 * BK);
-    if (s > max_by_k) s = max_by_k;
-    if (s > 16) s = 16;
-    while (s > 1 && (size_t)s * a.M * a.N * sizeof(float) > ((size_t)256 << 20)) --s;
-    return s < 1 ? 1 : (int)s;
+    const long cus = ctx->num_cus;
+    if (tiles * 4 >= 2 * cus * 3) return 1;  // three quarters of two per compute unit: a split would cost more in partial tiles than it gains
+    const long slices = (a.K + GB_K - 1) / GB_K;
+    const long fixed = 6;  // per workgroup, in slices
+    long best = 1, best_cost = 0;
+    for (long s = 1; s <= 16; ++s) {
+        if (s > 1 && (a.K / s < 4 * BK || (size_t)s * a.M * a.N * sizeof(float) > ((size_t)256 << 20))) break;
+        const long per_cu = (tiles * s + cus - 1) / cus;
+        // a workgroup alone on its compute unit has nobody to overlap its barriers and first loads with
+        const long cost = per_cu * ((slices + s - 1) / s + fixed) * (per_cu == 1 ? 4 : 3);
+        if (s == 1 || cost < best_cost) {  // ties: the fewer partial tiles
+            best = s;
+            best_cost = cost;
+        }
+    }
+    return (int)best;
 }
 
 // K splits (1 to 4) for the 256x256 kernel, or 0 where the 128x128 kernel is to run.  The large tile
