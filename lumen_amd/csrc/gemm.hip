@@ -502,13 +502,19 @@ static int gemm_big_splits(const lumen_ctx *ctx, const GemmArgs &a) {
         if (s > 1 && (a.K / s < 512 || (size_t)s * a.M * a.N * sizeof(float) > ((size_t)256 << 20))) break;
         const long w = tiles * s, rounds = (w + cus - 1) / cus;
         const double fill = (double)w / (double)(rounds * cus);
-        if (fill >= 0.9) return s;
         if (fill > best_fill) {
             best_fill = fill;
             best = s;
         }
+        if (fill >= 0.9) break;
     }
-    return best_fill >= 0.8 ? best : 0;
+    if (best_fill < 0.8) return 0;
+    // A split writes and re-reads s partial copies of C.  Where the 128x128 grid fills the chip two and a
+    // half times over on its own (1024 x 11264: 704 tiles) that costs more than the large tile gains
+    // (336 against 270 us there).
+    const long tiles128 = (long)((a.N + BN - 1) / BN) * ((a.M + BM - 1) / BM);
+    if (best > 1 && tiles128 * 2 >= cus * 5) return 0;
+    return best;
 }
 
 int launch_gemm(lumen_ctx *ctx, const GemmArgs &a) {
