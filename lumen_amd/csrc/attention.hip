@@ -406,8 +406,23 @@ __device__ __forceinline__ bool attn_decode_slice(const AttnDecodeArgs &a, int r
 // Grid: x = n_rep * nslices workgroups per KV head, y = KV head, z = batch.  NREP_T: the group size
 // n_rep where it is one of the common ones (index arithmetic with constants), 0 for any other.
 template <int D, int NREP_T, int WAVES, bool PRE>
-__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void attn_decode_kernel(AttnDecodeArgs a) {
+__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void attn_decode_kernel(
+    float *k_cache_hot, float *v_cache_hot, const int *pos_dev_hot, const float *q_hot, int max_seq_hot, int hkv_hot,
+    int start_short, int grid_x, int pos_host_hot, int hq_hot, AttnDecodeArgs a_mem) {
     typedef AttnGeom<D, WAVES> G;
+    // The leading scalar arguments repeat the fields that the first trip of row loads depends on, and
+    // start_short is the form to try first (decided by the launcher from the position, or from the hint
+    // where the position sits in device memory): they are preloaded into scalar registers (see the
+    // Makefile), so those loads go out without waiting for a read of the argument block.
+    AttnDecodeArgs a = a_mem;
+    a.k_cache = k_cache_hot;
+    a.v_cache = v_cache_hot;
+    a.pos_dev = pos_dev_hot;
+    a.max_seq = max_seq_hot;
+    a.hkv = hkv_hot;
+    a.pos_host = pos_host_hot;
+    a.q = q_hot;
+    a.hq = hq_hot;
     __shared__ __align__(16) float q_rot[D];
     __shared__ __align__(16) float k_new[D];
     __shared__ __align__(16) float v_new[D];
@@ -425,11 +440,11 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
     // head the heads of a group are placed 8 apart, four to an XCD, so that a group's K/V rows are
     // fetched into two L2s instead of eight (that placement is for groups of eight heads).
     int r = split;
-    if (NREP == 8 && gridDim.x >= 32 && (gridDim.x & 7) == 0) r = (split & 7) < 2 && split < 32 ? (split >> 3) + 4 * (split & 7) : NREP;
+    if (NREP == 8 && grid_x >= 32 && (grid_x & 7) == 0) r = (split & 7) < 2 && split < 32 ? (split >> 3) + 4 * (split & 7) : NREP;
     // Long form: workgroup `split` takes query head rr over slice `slice`.  With 8 or more slices
     // the heads of one (KV head, slice) sit 8 workgroups apart -- on one XCD -- so the slice's rows
     // reach that XCD's L2 once for all of them.
-    const int nslices = (int)gridDim.x / NREP;  // a power of two
+    const int nslices = grid_x / NREP;  // a power of two
     int slice, rr;
     if (nslices >= 8) {
         slice = (split & 7) | ((split / (8 * NREP)) << 3);
@@ -447,7 +462,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
     // other one if the hint was wrong.  One call site per form: two would let the compiler keep the
     // first one's loaded rows alive for the second across everything in between.
     int pos_new = a.pos_dev ? -1 : a.pos_host;  // == past_len, the new token's position
-    bool want_short = pos_new >= 0 ? pos_new + 1 <= SHORT_ROWS : a.expect_short != 0;
+    bool want_short = start_short != 0;
 #pragma unroll 1
     for (int attempt = 0; attempt < 2; ++attempt) {
         if (want_short) {
@@ -490,14 +505,17 @@ static int launch_decode_d(lumen_ctx *ctx, const AttnDecodeArgs &a) {
     constexpr int WAVES = DecodeWaves<D>::value;
     const int nrep = a.hq / a.hkv;
     dim3 grid(nrep * a.nsplit, a.hkv, a.b);
+    // the form the kernel tries first: known from the position, or the caller's hint
+    const int start_short = a.pos_dev ? (a.expect_short != 0) : (a.pos_host + 1 <= attn_decode_short_rows(D));
     if ((size_t)a.max_seq * D * sizeof(float) >= ((size_t)1 << 32))  // 32-bit byte offsets inside a head
         LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "decode attention: a KV head of %d rows x %d exceeds 4 GiB", a.max_seq, D);
+#define DECODE_HOT a.k_cache, a.v_cache, a.pos_dev, a.q, a.max_seq, a.hkv, start_short, (int)grid.x, a.pos_host, a.hq
 #define LAUNCH_DECODE(NR)                                                                                          \
     do {                                                                                                           \
         if (a.pre_rotated)                                                                                         \
-            hipLaunchKernelGGL((attn_decode_kernel<D, NR, WAVES, true>), grid, dim3(WAVES * 64), 0, ctx->stream, a);  \
+            hipLaunchKernelGGL((attn_decode_kernel<D, NR, WAVES, true>), grid, dim3(WAVES * 64), 0, ctx->stream, DECODE_HOT, a);  \
         else                                                                                                       \
-            hipLaunchKernelGGL((attn_decode_kernel<D, NR, WAVES, false>), grid, dim3(WAVES * 64), 0, ctx->stream, a); \
+            hipLaunchKernelGGL((attn_decode_kernel<D, NR, WAVES, false>), grid, dim3(WAVES * 64), 0, ctx->stream, DECODE_HOT, a); \
     } while (0)
     switch (nrep) {
         case 1: LAUNCH_DECODE(1); break;
@@ -507,6 +525,7 @@ static int launch_decode_d(lumen_ctx *ctx, const AttnDecodeArgs &a) {
         default: LAUNCH_DECODE(0); break;
     }
 #undef LAUNCH_DECODE
+#undef DECODE_HOT
     LUMEN_CHECK_LAUNCH();
     return LUMEN_OK;
 }

@@ -16,7 +16,7 @@ typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 
 #define GEMV_THREADS 256                  // default workgroup: 4 wavefronts
 #define GEMV_WAVES (GEMV_THREADS / 64)
-#define GEMV_MAX_WAVES 8                  // the kernel takes its size from blockDim.x, up to this
+#define GEMV_MAX_WAVES 8                  // the launcher picks 4 to 8 wavefronts per workgroup
 
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
@@ -62,9 +62,9 @@ __device__ __forceinline__ float dot16(const v4u raw, const float *xs) {
 // of the workgroup must call it.
 template <int PRO>
 __device__ __forceinline__ void stage_x(float *xs, const float *__restrict__ x, const float *__restrict__ g,
-                                        float eps, int K, int kpad) {
+                                        float eps, int K, int kpad, int nwaves) {
     __shared__ float red[GEMV_MAX_WAVES];
-    const int tid = threadIdx.x, nthreads = blockDim.x, nwaves = nthreads >> 6;
+    const int tid = threadIdx.x, nthreads = nwaves * 64;
     float ss = 0.f;
     for (int k = tid * 4; k < kpad; k += nthreads * 4) {
         v4f v = {0.f, 0.f, 0.f, 0.f};
@@ -101,8 +101,8 @@ __device__ __forceinline__ void stage_x(float *xs, const float *__restrict__ x, 
 // in use and its weight forced to zero).  All threads of the workgroup must call it.
 #define GEMV_FOLD_MAX_SLICES 16
 typedef float v2f __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ void stage_attn_fold(float *xs, const GemvArgs &a, int K, int kpad) {
-    const int tid = threadIdx.x, nthreads = blockDim.x;
+__device__ __forceinline__ void stage_attn_fold(float *xs, const GemvArgs &a, int K, int kpad, int nwaves) {
+    const int tid = threadIdx.x, nthreads = nwaves * 64;
     const int D = a.attn_d, S = a.attn_nslices, stride = D + 2;
     const int rows = *a.attn_pos + 1;
     int nact = 1;
@@ -145,28 +145,31 @@ __device__ __forceinline__ void stage_attn_fold(float *xs, const GemvArgs &a, in
 }
 
 template <bool BF16, int R, int PRO, int EPI>
-__global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(GemvArgs a) {
+__global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W_hot, int N_hot, int K_hot, int D_hot,
+                                                                  int nblocks, int nwaves, GemvArgs a) {
+    // The leading scalar arguments repeat what the first weight loads need (a.W, a.N, a.K, a.D, the grid
+    // and workgroup size): the file is compiled with kernel-argument preloading, so they are in scalar
+    // registers when a wavefront starts and its first loads do not wait for a read of the argument block.
     extern __shared__ __align__(16) float xs[];
     constexpr int VEC = BF16 ? 8 : 4;          // elements per 16-byte load
     constexpr int SWEEP = 64 * VEC;            // elements one wavefront covers per load
     constexpr int U = 8 / R;                   // loads in flight per lane per row
     constexpr int PIECE = SWEEP * U;           // elements of a row one piece covers
     constexpr int ESZ = BF16 ? 2 : 4;
-    const int K = a.K, N = a.N;
+    const int K = K_hot, N = N_hot, D = D_hot;
     const int kpad = (K + PIECE - 1) / PIECE * PIECE;  // xs is zero from K to kpad
 
     const int lane = threadIdx.x & 63;
-    const int nwaves = blockDim.x >> 6;
     const int gw = blockIdx.x * nwaves + (threadIdx.x >> 6);
-    const int nw = gridDim.x * nwaves;
+    const int nw = nblocks * nwaves;
     const int nunits = (N + R - 1) / R;
-    const char *Wb = (const char *)a.W;
+    const char *Wb = (const char *)W_hot;
     const size_t row_bytes = (size_t)K * ESZ;
-    const int half_d = a.D >> 1;
+    const int half_d = D >> 1;
 
     // row r of unit u: consecutive rows, or the RoPE pair (j, j + D/2) of one head
     auto unit_row = [&](int u, int r) {
-        if (EPI == EPI_ROPE_QKV) return (u / half_d) * a.D + (u % half_d) + r * half_d;
+        if (EPI == EPI_ROPE_QKV) return (u / half_d) * D + (u % half_d) + r * half_d;
         return u * R + r;
     };
 
@@ -220,8 +223,8 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(GemvArgs a) {
     auto preload = [&](int un) {
         if (EPI == EPI_ROPE_QKV && un < nunits) {
             const int j = un % half_d;
-            pre0 = a.cos_t[(size_t)pos * a.D + j];
-            pre1 = a.sin_t[(size_t)pos * a.D + j];
+            pre0 = a.cos_t[(size_t)pos * D + j];
+            pre1 = a.sin_t[(size_t)pos * D + j];
         }
         if (EPI == EPI_RESIDUAL) {
             if (un * R < N) pre0 = residual[un * R];
@@ -229,8 +232,8 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(GemvArgs a) {
         }
     };
     preload(gw);
-    if (PRO == PRO_ATTN_FOLD) stage_attn_fold(xs, a, K, kpad);
-    else stage_x<PRO>(xs, a.x + (a.x_sel ? sel_off : 0), a.norm_w, a.eps, K, kpad);
+    if (PRO == PRO_ATTN_FOLD) stage_attn_fold(xs, a, K, kpad, nwaves);
+    else stage_x<PRO>(xs, a.x + (a.x_sel ? sel_off : 0), a.norm_w, a.eps, K, kpad, nwaves);
     float best = -INFINITY;
     int best_idx = 0x7fffffff;
 
@@ -276,14 +279,14 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(GemvArgs a) {
                         o2 = x1 * sn + x2 * c;
                     }
                     if (head < a.hq) {
-                        a.y[head * a.D + j] = o1;
-                        a.y[head * a.D + j + half_d] = o2;
+                        a.y[head * D + j] = o1;
+                        a.y[head * D + j + half_d] = o2;
                     } else if (head < a.hq + a.hkv) {
-                        float *dst = a.k_cache + ((size_t)(head - a.hq) * a.max_seq + pos) * a.D;
+                        float *dst = a.k_cache + ((size_t)(head - a.hq) * a.max_seq + pos) * D;
                         dst[j] = o1;
                         dst[j + half_d] = o2;
                     } else {
-                        float *dst = a.v_cache + ((size_t)(head - a.hq - a.hkv) * a.max_seq + pos) * a.D;
+                        float *dst = a.v_cache + ((size_t)(head - a.hq - a.hkv) * a.max_seq + pos) * D;
                         dst[j] = x1;
                         dst[j + half_d] = x2;
                     }
@@ -344,14 +347,14 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(GemvArgs a) {
         __syncthreads();  // thread 0's stores are complete past this barrier
         if (threadIdx.x == 0) {
             const int old = __hip_atomic_fetch_add(a.amax_counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            am_last = (old == (int)gridDim.x - 1);
+            am_last = (old == nblocks - 1);
             if (am_last) __hip_atomic_store(a.amax_counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         __syncthreads();
         if (!am_last) return;
         float bv = -INFINITY;
         int bi = 0x7fffffff;
-        for (int i = threadIdx.x; i < (int)gridDim.x; i += (int)blockDim.x) {
+        for (int i = threadIdx.x; i < nblocks; i += nwaves * 64) {
             const float v = __hip_atomic_load(a.amax_val + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             const int ix = __hip_atomic_load(a.amax_idx + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if (v > bv || (v == bv && ix < bi)) {
@@ -416,19 +419,19 @@ template <bool BF16, int R, int PRO>
 static void launch_epi(const GemvArgs &a, dim3 grid, int threads, size_t lds, hipStream_t s) {
     switch (a.epi) {
         case EPI_STORE:
-            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_STORE>), grid, dim3(threads), lds, s, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_STORE>), grid, dim3(threads), lds, s, a.W, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
             break;
         case EPI_RESIDUAL:
-            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_RESIDUAL>), grid, dim3(threads), lds, s, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_RESIDUAL>), grid, dim3(threads), lds, s, a.W, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
             break;
         case EPI_ARGMAX:
-            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_ARGMAX>), grid, dim3(threads), lds, s, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_ARGMAX>), grid, dim3(threads), lds, s, a.W, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
             break;
         case EPI_ROPE_QKV:
-            hipLaunchKernelGGL((gemv_kernel<BF16, 2, PRO, EPI_ROPE_QKV>), grid, dim3(threads), lds, s, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, 2, PRO, EPI_ROPE_QKV>), grid, dim3(threads), lds, s, a.W, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
             break;
         default:
-            hipLaunchKernelGGL((gemv_kernel<BF16, 2, PRO, EPI_SWIGLU>), grid, dim3(threads), lds, s, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, 2, PRO, EPI_SWIGLU>), grid, dim3(threads), lds, s, a.W, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
             break;
     }
 }
@@ -436,7 +439,7 @@ static void launch_epi(const GemvArgs &a, dim3 grid, int threads, size_t lds, hi
 template <bool BF16, int R>
 static void launch_pro(const GemvArgs &a, dim3 grid, int threads, size_t lds, hipStream_t s) {
     if (a.pro == PRO_ATTN_FOLD)  // o_proj only (launch_gemv checks): one row per unit, residual epilogue
-        hipLaunchKernelGGL((gemv_kernel<BF16, 1, PRO_ATTN_FOLD, EPI_RESIDUAL>), grid, dim3(threads), lds, s, a);
+        hipLaunchKernelGGL((gemv_kernel<BF16, 1, PRO_ATTN_FOLD, EPI_RESIDUAL>), grid, dim3(threads), lds, s, a.W, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
     else if (a.pro == PRO_RMSNORM)
         launch_epi<BF16, R, PRO_RMSNORM>(a, grid, threads, lds, s);
     else
