@@ -12,6 +12,7 @@ from lumen_amd import _lib, synth
 from lumen_amd.autograd import no_grad
 from lumen_amd.models import LayeredLlamaModel, LlamaModel
 from oracle import lumen_oracle as lo
+from tests import golden_util
 from tests.gpu_util import max_rel
 
 pytestmark = pytest.mark.gpu
@@ -72,6 +73,23 @@ def test_prefill_then_teacher_forced_decode(cfg, tol, bf16):
             n = n_prompt + n_dec
             assert max_rel(k[:, :, :n], ora.cache_k(layer)[:, :, :n]) <= tol
             assert max_rel(v[:, :, :n], ora.cache_v(layer)[:, :, :n]) <= tol
+
+
+@pytest.mark.parametrize("name", golden_util.CASES)
+def test_against_committed_golden_logits(name):
+    """Prefill then decode against the committed fp64 logits of an independent implementation of the model
+    (tests/golden): same 1e-4 bound as against the oracle."""
+    cfg, params, ids, ref = golden_util.load_case(name)
+    n, n_prompt = len(ids), 13
+    gpu = LlamaModel(cfg)
+    for pname, a in params.items():
+        gpu.set_param(pname, a)
+    got = gpu.forward(ids[:n_prompt], all_rows=True)
+    assert max_rel(got, ref[:n_prompt]) <= 1e-4
+    for t in range(n_prompt, n):
+        g = gpu.forward(ids[t:t + 1], all_rows=False)
+        assert max_rel(g, ref[t]) <= 1e-4, (t, max_rel(g, ref[t]))
+        check_argmax(g, ref[t].astype(np.float32), 1e-4)
 
 
 def test_last_row_only_prefill_equals_all_rows_and_incremental_prefill():

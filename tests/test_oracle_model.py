@@ -11,6 +11,7 @@ import torch
 
 from lumen_amd import synth
 from oracle import lumen_oracle as lo
+from tests import golden_util
 
 transformers = pytest.importorskip("transformers")
 
@@ -40,6 +41,23 @@ def hf_model(cfg, params):
     missing, unexpected = model.load_state_dict(sd, strict=False)
     assert not [m for m in missing if "rotary" not in m] and not unexpected, (missing, unexpected)
     return model.double().eval()
+
+
+@pytest.mark.parametrize("name", golden_util.CASES)
+def test_forward_matches_committed_golden_logits(name):
+    """The same comparison against the committed fp64 vectors (no transformers needed at test time)."""
+    cfg, params, ids, ref = golden_util.load_case(name)
+    n, n_prompt = len(ids), 13
+    m = lo.Llama(cfg, params)
+    rc, logits = m.forward(ids[:n_prompt])
+    assert rc == lo.LO_OK
+    scale = np.abs(ref).max()
+    assert np.abs(logits - ref[:n_prompt]).max() <= 2e-5 * scale
+    for t in range(n_prompt, n):
+        rc, lg = m.forward(ids[t:t + 1])
+        assert rc == lo.LO_OK
+        assert np.abs(lg[0] - ref[t]).max() <= 2e-5 * scale
+        assert lo.argmax(lg[0]) == int(ref[t].argmax())
 
 
 @pytest.mark.parametrize("cfg", [TINY, TINY_QWEN], ids=["llama", "qwen3"])
