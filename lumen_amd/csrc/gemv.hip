@@ -99,7 +99,6 @@ __device__ __forceinline__ void stage_x(float *xs, const float *__restrict__ x, 
 // are independent of each other: one trip to memory after the position is known.  Slices not in use
 // hold whatever an earlier step left there: they are never read (the index is clamped to the last one
 // in use and its weight forced to zero).  All threads of the workgroup must call it.
-#define GEMV_FOLD_MAX_SLICES 16
 typedef float v2f __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ void stage_attn_fold(float *xs, const GemvArgs &a, int K, int kpad, int nwaves) {
     const int tid = threadIdx.x, nthreads = nwaves * 64;
@@ -446,6 +445,37 @@ static void launch_pro(const GemvArgs &a, dim3 grid, int threads, size_t lds, hi
         launch_epi<BF16, R, PRO_NONE>(a, grid, threads, lds, s);
 }
 
+// Grid of the fused kernel for an [N, K] product: workgroups and threads per workgroup.
+int gemv_grid(const lumen_ctx *ctx, int N, int K, int w_bf16, int epi, int *threads_out) {
+    const int vec = w_bf16 ? 8 : 4;
+    const int R = (epi == EPI_SWIGLU || epi == EPI_ROPE_QKV || N >= 8192) ? 2 : 1;
+    const int piece = 64 * vec * (8 / R);
+    const int kpad = (K + piece - 1) / piece * piece;
+    const size_t lds = (size_t)kpad * sizeof(float);
+    const int nunits = (N + R - 1) / R;
+    // Wavefronts per workgroup: when the units divide into exactly one workgroup of 5 to 8 wavefronts
+    // per compute unit, take that shape -- every compute unit gets the same share and stages x once
+    // (q|k|v of a 2048-wide model: 1280 pairs = 256 x 5; its o_proj and down: 2048 rows = 256 x 8).
+    int waves = GEMV_WAVES;
+    if (nunits % ctx->num_cus == 0) {
+        const int w = nunits / ctx->num_cus;
+        if (w > GEMV_WAVES && w <= GEMV_MAX_WAVES) waves = w;
+    }
+    const int threads = waves * 64;
+    int blocks = (nunits + waves - 1) / waves;
+    // one wave of workgroups: at most 4 per compute unit, fewer when their staged x would not fit the
+    // compute unit's 160 KiB of LDS side by side (a second, partial wave of workgroups costs more
+    // than longer row loops: 4.0 -> 4.7 TB/s at K = 11008 with bf16 weights)
+    int per_cu = (int)((size_t)(160 * 1024) / (lds + 256));
+    const int max_per_cu = 16 / waves > 1 ? 16 / waves : 1;  // 16 wavefronts per compute unit
+    if (per_cu > max_per_cu) per_cu = max_per_cu;
+    if (per_cu < 1) per_cu = 1;
+    const int cap = ctx->num_cus * per_cu;
+    if (blocks > cap) blocks = cap;
+    if (threads_out) *threads_out = threads;
+    return blocks;
+}
+
 int gemv_max_blocks(const lumen_ctx *ctx) { return ctx->num_cus * 4; }
 
 int launch_gemv(lumen_ctx *ctx, const GemvArgs &a) {
@@ -479,26 +509,8 @@ int launch_gemv(lumen_ctx *ctx, const GemvArgs &a) {
     }
     if ((a.epi == EPI_SWIGLU || a.epi == EPI_ROPE_QKV) && (a.N & 1))
         LUMEN_FAIL(LUMEN_ERR_SHAPE, "paired-row epilogue needs an even row count, got %d", a.N);
-    const int nunits = (a.N + R - 1) / R;
-    // Wavefronts per workgroup: when the units divide into exactly one workgroup of 5 to 8 wavefronts
-    // per compute unit, take that shape -- every compute unit gets the same share and stages x once
-    // (q|k|v of a 2048-wide model: 1280 pairs = 256 x 5; its o_proj and down: 2048 rows = 256 x 8).
-    int waves = GEMV_WAVES;
-    if (nunits % ctx->num_cus == 0) {
-        const int w = nunits / ctx->num_cus;
-        if (w > GEMV_WAVES && w <= GEMV_MAX_WAVES) waves = w;
-    }
-    const int threads = waves * 64;
-    int blocks = (nunits + waves - 1) / waves;
-    // one wave of workgroups: at most 4 per compute unit, fewer when their staged x would not fit the
-    // compute unit's 160 KiB of LDS side by side (a second, partial wave of workgroups costs more
-    // than longer row loops: 4.0 -> 4.7 TB/s at K = 11008 with bf16 weights)
-    int per_cu = (int)((size_t)(160 * 1024) / (lds + 256));
-    const int max_per_cu = 16 / waves > 1 ? 16 / waves : 1;  // 16 wavefronts per compute unit
-    if (per_cu > max_per_cu) per_cu = max_per_cu;
-    if (per_cu < 1) per_cu = 1;
-    const int cap = ctx->num_cus * per_cu;
-    if (blocks > cap) blocks = cap;
+    int threads = 0;
+    const int blocks = gemv_grid(ctx, a.N, a.K, a.w_bf16, a.epi, &threads);
     dim3 grid(blocks);
     if (a.w_bf16) {
         if (R == 2) launch_pro<true, 2>(a, grid, threads, lds, ctx->stream);

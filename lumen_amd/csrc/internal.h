@@ -109,8 +109,11 @@ struct GemvArgs {
     const int *attn_pos;
     int attn_nslices, attn_d, attn_trip, attn_short_rows;
 };
+#define GEMV_FOLD_MAX_SLICES 16  // PRO_ATTN_FOLD reads this many slice states per element, whatever the count in use
 int launch_gemv(lumen_ctx *ctx, const GemvArgs &a);
 int gemv_max_blocks(const lumen_ctx *ctx);
+// grid of the fused GEMV kernel for an [N, K] product (workgroups; threads per workgroup in *threads_out)
+int gemv_grid(const lumen_ctx *ctx, int N, int K, int w_bf16, int epi, int *threads_out);
 
 struct GemmArgs {
     const float *A;   // [M, K]

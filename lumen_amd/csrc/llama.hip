@@ -184,7 +184,14 @@ extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg,
     // stages its input: an atomic and a second round of loads fewer inside the attention kernel.  With more
     // slices the partials would outweigh what the GEMV workgroups can re-read.  q/k norm models rotate
     // inside the attention kernel: not covered.  Used on the long side of the short-cache boundary only.
-    m->defer_merge = m->nsplit >= 2 && m->nsplit <= 16 && !cfg->qk_norm && cfg->max_seq_len <= m->nsplit * attn_decode_trip_rows(D);
+    // Leaving the merge of the slices to the o_proj GEMV makes every one of its workgroups read every
+    // slice's state of every element out of L2: it pays while that stays a few tens of MB (33 MB for a
+    // 2048-wide model: 1.13 -> 1.09 ms per token at 4000 rows; 268 MB for a 4096-wide one with 32 KV
+    // heads, where o_proj went from 8 to 24 us)
+    const size_t fold_bytes = (size_t)gemv_grid(ctx, H, m->qd, m->bf16, EPI_RESIDUAL, nullptr) * (size_t)m->qd *
+                              GEMV_FOLD_MAX_SLICES * sizeof(float);
+    m->defer_merge = m->nsplit >= 2 && m->nsplit <= GEMV_FOLD_MAX_SLICES && !cfg->qk_norm &&
+                     cfg->max_seq_len <= m->nsplit * attn_decode_trip_rows(D) && fold_bytes <= ((size_t)64 << 20);
     m->pk_nsplit = cfg->max_seq_len / 64 < 1 ? 1 : (cfg->max_seq_len / 64 > 64 ? 64 : cfg->max_seq_len / 64);
     M_TRY(dmalloc_t(m, &m->part, attn_decode_part_floats(1, Hq, D, m->nsplit > m->pk_nsplit ? m->nsplit : m->pk_nsplit)));
     M_TRY(dmalloc_t(m, &m->counters, (size_t)Hq));
