@@ -60,17 +60,33 @@ __device__ __forceinline__ float dot16(const v4u raw, const float *xs) {
 // into LDS, zero-padded to kpad.  x is read from memory once: the raw values go to LDS while the
 // sum of squares is taken, then every thread scales the elements it staged itself.  All threads
 // of the workgroup must call it.
-template <int PRO>
+template <int PRO, int XB>
 __device__ __forceinline__ void stage_x(float *xs, const float *__restrict__ x, const float *__restrict__ g,
                                         float eps, int K, int kpad, int nwaves) {
     __shared__ float red[GEMV_MAX_WAVES];
     const int tid = threadIdx.x, nthreads = nwaves * 64;
     float ss = 0.f;
-    for (int k = tid * 4; k < kpad; k += nthreads * 4) {
-        v4f v = {0.f, 0.f, 0.f, 0.f};
-        if (k < K) v = *(const v4f *)(x + k);
-        ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
-        *(v4f *)(xs + k) = v;
+    // XB loads per thread are requested before the first one is waited for: taken one by one, each is a
+    // trip to memory of its own (eleven in a row for K = 11008 with 256 threads).  The launcher asks for
+    // XB = 4 where a thread has more than two pieces to stage; the registers this takes cost the
+    // K = 2048 kernels more than the trips (gate|up 16.1 -> 16.8 us), so those keep XB = 1.
+    
+    for (int k0 = tid * 4; k0 < kpad; k0 += nthreads * 4 * XB) {
+        v4f v[XB];
+#pragma unroll
+        for (int i = 0; i < XB; ++i) {
+            const int k = k0 + i * nthreads * 4;
+            v[i] = v4f{0.f, 0.f, 0.f, 0.f};
+            if (k < K) v[i] = *(const v4f *)(x + k);
+        }
+#pragma unroll
+        for (int i = 0; i < XB; ++i) {
+            const int k = k0 + i * nthreads * 4;
+            if (k < kpad) {
+                ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+                *(v4f *)(xs + k) = v[i];
+            }
+        }
     }
     if (PRO == PRO_RMSNORM) {
         ss = wave_sum(ss);
@@ -143,7 +159,7 @@ __device__ __forceinline__ void stage_attn_fold(float *xs, const GemvArgs &a, in
     __syncthreads();
 }
 
-template <bool BF16, int R, int PRO, int EPI>
+template <bool BF16, int R, int PRO, int EPI, int XB>
 __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W_hot, int N_hot, int K_hot, int D_hot,
                                                                   int nblocks, int nwaves, GemvArgs a) {
     // The leading scalar arguments repeat what the first weight loads need (a.W, a.N, a.K, a.D, the grid
@@ -232,7 +248,7 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W
     };
     preload(gw);
     if (PRO == PRO_ATTN_FOLD) stage_attn_fold(xs, a, K, kpad, nwaves);
-    else stage_x<PRO>(xs, a.x + (a.x_sel ? sel_off : 0), a.norm_w, a.eps, K, kpad, nwaves);
+    else stage_x<PRO, XB>(xs, a.x + (a.x_sel ? sel_off : 0), a.norm_w, a.eps, K, kpad, nwaves);
     float best = -INFINITY;
     int best_idx = 0x7fffffff;
 
@@ -414,35 +430,35 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_generic_kernel(GemvArgs a) 
     }
 }
 
-template <bool BF16, int R, int PRO>
+template <bool BF16, int R, int PRO, int XB>
 static void launch_epi(const GemvArgs &a, dim3 grid, int threads, size_t lds, hipStream_t s) {
     switch (a.epi) {
         case EPI_STORE:
-            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_STORE>), grid, dim3(threads), lds, s, a.W, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_STORE, XB>), grid, dim3(threads), lds, s, a.W, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
             break;
         case EPI_RESIDUAL:
-            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_RESIDUAL>), grid, dim3(threads), lds, s, a.W, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_RESIDUAL, XB>), grid, dim3(threads), lds, s, a.W, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
             break;
         case EPI_ARGMAX:
-            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_ARGMAX>), grid, dim3(threads), lds, s, a.W, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_ARGMAX, XB>), grid, dim3(threads), lds, s, a.W, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
             break;
         case EPI_ROPE_QKV:
-            hipLaunchKernelGGL((gemv_kernel<BF16, 2, PRO, EPI_ROPE_QKV>), grid, dim3(threads), lds, s, a.W, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, 2, PRO, EPI_ROPE_QKV, XB>), grid, dim3(threads), lds, s, a.W, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
             break;
         default:
-            hipLaunchKernelGGL((gemv_kernel<BF16, 2, PRO, EPI_SWIGLU>), grid, dim3(threads), lds, s, a.W, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, 2, PRO, EPI_SWIGLU, XB>), grid, dim3(threads), lds, s, a.W, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
             break;
     }
 }
 
-template <bool BF16, int R>
+template <bool BF16, int R, int XB>
 static void launch_pro(const GemvArgs &a, dim3 grid, int threads, size_t lds, hipStream_t s) {
     if (a.pro == PRO_ATTN_FOLD)  // o_proj only (launch_gemv checks): one row per unit, residual epilogue
-        hipLaunchKernelGGL((gemv_kernel<BF16, 1, PRO_ATTN_FOLD, EPI_RESIDUAL>), grid, dim3(threads), lds, s, a.W, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
+        hipLaunchKernelGGL((gemv_kernel<BF16, 1, PRO_ATTN_FOLD, EPI_RESIDUAL, XB>), grid, dim3(threads), lds, s, a.W, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
     else if (a.pro == PRO_RMSNORM)
-        launch_epi<BF16, R, PRO_RMSNORM>(a, grid, threads, lds, s);
+        launch_epi<BF16, R, PRO_RMSNORM, XB>(a, grid, threads, lds, s);
     else
-        launch_epi<BF16, R, PRO_NONE>(a, grid, threads, lds, s);
+        launch_epi<BF16, R, PRO_NONE, XB>(a, grid, threads, lds, s);
 }
 
 // Grid of the fused kernel for an [N, K] product: workgroups and threads per workgroup.
@@ -512,13 +528,21 @@ int launch_gemv(lumen_ctx *ctx, const GemvArgs &a) {
     int threads = 0;
     const int blocks = gemv_grid(ctx, a.N, a.K, a.w_bf16, a.epi, &threads);
     dim3 grid(blocks);
+    // pieces of x a thread stages: batched loads from three on (see stage_x)
+    const bool batch_x = (kpad + threads * 4 - 1) / (threads * 4) > 2;
+#define LAUNCH_GEMV(BF, RR)                                                    \
+    do {                                                                       \
+        if (batch_x) launch_pro<BF, RR, 4>(a, grid, threads, lds, ctx->stream); \
+        else launch_pro<BF, RR, 1>(a, grid, threads, lds, ctx->stream);        \
+    } while (0)
     if (a.w_bf16) {
-        if (R == 2) launch_pro<true, 2>(a, grid, threads, lds, ctx->stream);
-        else launch_pro<true, 1>(a, grid, threads, lds, ctx->stream);
+        if (R == 2) LAUNCH_GEMV(true, 2);
+        else LAUNCH_GEMV(true, 1);
     } else {
-        if (R == 2) launch_pro<false, 2>(a, grid, threads, lds, ctx->stream);
-        else launch_pro<false, 1>(a, grid, threads, lds, ctx->stream);
+        if (R == 2) LAUNCH_GEMV(false, 2);
+        else LAUNCH_GEMV(false, 1);
     }
+#undef LAUNCH_GEMV
     LUMEN_CHECK_LAUNCH();
     return LUMEN_OK;
 }
