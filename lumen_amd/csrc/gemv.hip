@@ -109,6 +109,85 @@ __device__ __forceinline__ void stage_x(float *xs, const float *__restrict__ x, 
     __syncthreads();
 }
 
+// Latency-bound launches (every wavefront has a single unit whose loads all go out at once): the first
+// GEMV_EARLY pieces of x of a thread -- and of the norm gains -- are requested BEFORE the weights.  Loads
+// return in the order they were issued, so x queued behind the weights would arrive after them, and the
+// staging, the sum of squares and the gains (two dependent trips more in the plain loop) would all sit
+// between the arrival of the weights and the first multiply.  Requested first, they are staged while the
+// weights are still on their way.
+#define GEMV_EARLY 2
+template <int PRO>
+__device__ __forceinline__ void request_early(v4f (&xe)[GEMV_EARLY], v4f (&ge)[GEMV_EARLY], const float *__restrict__ x,
+                                              const float *__restrict__ g, int K, int nthreads) {
+#pragma unroll
+    for (int i = 0; i < GEMV_EARLY; ++i) {
+        const int k = ((int)threadIdx.x + i * nthreads) * 4;
+        xe[i] = v4f{0.f, 0.f, 0.f, 0.f};
+        ge[i] = v4f{0.f, 0.f, 0.f, 0.f};
+        if (k < K) {
+            xe[i] = *(const v4f *)(x + k);
+            if (PRO == PRO_RMSNORM) ge[i] = *(const v4f *)(g + k);
+        }
+    }
+}
+
+// stage_x for a launch whose first GEMV_EARLY pieces per thread were requested by request_early; pieces
+// beyond those (none for the shapes the launcher sends here) take the plain loops.
+template <int PRO>
+__device__ __forceinline__ void stage_x_early(float *xs, const float *__restrict__ x, const float *__restrict__ g,
+                                              float eps, int K, int kpad, int nwaves, const v4f (&xe)[GEMV_EARLY],
+                                              const v4f (&ge)[GEMV_EARLY]) {
+    __shared__ float red_e[GEMV_MAX_WAVES];
+    const int tid = threadIdx.x, nthreads = nwaves * 64;
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < GEMV_EARLY; ++i) {
+        const int k = (tid + i * nthreads) * 4;
+        if (k < kpad) {
+            ss += xe[i].x * xe[i].x + xe[i].y * xe[i].y + xe[i].z * xe[i].z + xe[i].w * xe[i].w;
+            if (PRO != PRO_RMSNORM) *(v4f *)(xs + k) = xe[i];
+        }
+    }
+    for (int k = (tid + GEMV_EARLY * nthreads) * 4; k < kpad; k += nthreads * 4) {
+        v4f v = {0.f, 0.f, 0.f, 0.f};
+        if (k < K) v = *(const v4f *)(x + k);
+        ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+        *(v4f *)(xs + k) = v;
+    }
+    if (PRO == PRO_RMSNORM) {
+        // the early pieces stay in registers until the sum of squares is known and go to LDS scaled
+        ss = wave_sum(ss);
+        if ((tid & 63) == 0) red_e[tid >> 6] = ss;
+        __syncthreads();
+        float tot = 0.f;
+        for (int w = 0; w < nwaves; ++w) tot += red_e[w];
+        const float rms = sqrtf(tot / (float)K + eps);
+        const float inv = 1.0f / rms;
+#pragma unroll
+        for (int i = 0; i < GEMV_EARLY; ++i) {
+            const int k = (tid + i * nthreads) * 4;
+            if (k < kpad) {
+                v4f v = xe[i];
+                v.x = v.x * inv * ge[i].x;
+                v.y = v.y * inv * ge[i].y;
+                v.z = v.z * inv * ge[i].z;
+                v.w = v.w * inv * ge[i].w;
+                *(v4f *)(xs + k) = v;
+            }
+        }
+        for (int k = (tid + GEMV_EARLY * nthreads) * 4; k < K; k += nthreads * 4) {
+            v4f v = *(const v4f *)(xs + k);
+            const v4f gg = *(const v4f *)(g + k);
+            v.x = v.x * inv * gg.x;
+            v.y = v.y * inv * gg.y;
+            v.z = v.z * inv * gg.z;
+            v.w = v.w * inv * gg.w;
+            *(v4f *)(xs + k) = v;
+        }
+    }
+    __syncthreads();
+}
+
 // Stages the decode attention output from the attention kernel's partial states: head h, element d is
 // sum_s w_s ctx_s[d] / (sum_s w_s l_s + 1e-9) with w_s = exp2(m_s - max m) over the slices in use
 // (self_attention.rs:287-290 after the merge of the slices' online-softmax states).  A thread's loads
@@ -160,11 +239,15 @@ __device__ __forceinline__ void stage_attn_fold(float *xs, const GemvArgs &a, in
 }
 
 template <bool BF16, int R, int PRO, int EPI, int XB>
-__global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W_hot, int N_hot, int K_hot, int D_hot,
-                                                                  int nblocks, int nwaves, GemvArgs a) {
-    // The leading scalar arguments repeat what the first weight loads need (a.W, a.N, a.K, a.D, the grid
-    // and workgroup size): the file is compiled with kernel-argument preloading, so they are in scalar
-    // registers when a wavefront starts and its first loads do not wait for a read of the argument block.
+__global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W_hot, const float *x_hot,
+                                                                  const float *norm_w_hot, const int *row_sel_hot,
+                                                                  int N_hot, int K_hot, int D_hot, int nblocks,
+                                                                  int nwaves, GemvArgs a) {
+    // The leading scalar arguments repeat what the first loads need (a.W, a.x, a.norm_w, a.row_sel, a.N,
+    // a.K, a.D, the grid and workgroup size): the file is compiled with kernel-argument preloading, so they
+    // are in scalar registers when a wavefront starts and its first loads do not wait for a read of the
+    // argument block.  XB: how x is staged -- 1 piece at a time, 4 at a time, or 0: requested ahead of the
+    // weights (request_early).
     extern __shared__ __align__(16) float xs[];
     constexpr int VEC = BF16 ? 8 : 4;          // elements per 16-byte load
     constexpr int SWEEP = 64 * VEC;            // elements one wavefront covers per load
@@ -219,6 +302,12 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W
         }
     };
 
+    constexpr bool EARLY = XB == 0 && PRO != PRO_ATTN_FOLD;
+    v4f xe[GEMV_EARLY], ge[GEMV_EARLY];
+    // (with a row selector -- the first layer's gather -- the address of x needs a trip to memory itself:
+    // then the weights go first)
+    if (EARLY && !row_sel_hot) request_early<PRO>(xe, ge, x_hot, norm_w_hot, K, nwaves * 64);
+
     // the first weights of this wavefront start streaming before x is staged: they do not depend on it
     v4u rawA[R][U], rawB[R][U];
     load_piece(min(lu, nunits - 1), lk, rawA);
@@ -228,7 +317,13 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W
         advance_load();
     }
 
-    const long sel_off = a.row_sel ? (long)(*a.row_sel) * a.row_stride : 0;
+    long sel_off = 0;
+    const float *xin = x_hot;
+    if (row_sel_hot) {
+        sel_off = (long)(*row_sel_hot) * a.row_stride;
+        if (a.x_sel) xin += sel_off;
+        if (EARLY) request_early<PRO>(xe, ge, xin, norm_w_hot, K, nwaves * 64);
+    }
     const float *residual = a.residual + (a.residual_sel ? sel_off : 0);
     // What a unit's epilogue needs from memory is requested a unit ahead -- the first one here,
     // before x is staged -- so that no load sits between the last multiply and the store:
@@ -248,7 +343,8 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W
     };
     preload(gw);
     if (PRO == PRO_ATTN_FOLD) stage_attn_fold(xs, a, K, kpad, nwaves);
-    else stage_x<PRO, XB>(xs, a.x + (a.x_sel ? sel_off : 0), a.norm_w, a.eps, K, kpad, nwaves);
+    else if (EARLY) stage_x_early<PRO>(xs, xin, norm_w_hot, a.eps, K, kpad, nwaves, xe, ge);
+    else stage_x<PRO, (XB > 0 ? XB : 1)>(xs, xin, norm_w_hot, a.eps, K, kpad, nwaves);
     float best = -INFINITY;
     int best_idx = 0x7fffffff;
 
@@ -434,19 +530,19 @@ template <bool BF16, int R, int PRO, int XB>
 static void launch_epi(const GemvArgs &a, dim3 grid, int threads, size_t lds, hipStream_t s) {
     switch (a.epi) {
         case EPI_STORE:
-            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_STORE, XB>), grid, dim3(threads), lds, s, a.W, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_STORE, XB>), grid, dim3(threads), lds, s, a.W, a.x, a.norm_w, a.row_sel, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
             break;
         case EPI_RESIDUAL:
-            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_RESIDUAL, XB>), grid, dim3(threads), lds, s, a.W, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_RESIDUAL, XB>), grid, dim3(threads), lds, s, a.W, a.x, a.norm_w, a.row_sel, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
             break;
         case EPI_ARGMAX:
-            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_ARGMAX, XB>), grid, dim3(threads), lds, s, a.W, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_ARGMAX, XB>), grid, dim3(threads), lds, s, a.W, a.x, a.norm_w, a.row_sel, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
             break;
         case EPI_ROPE_QKV:
-            hipLaunchKernelGGL((gemv_kernel<BF16, 2, PRO, EPI_ROPE_QKV, XB>), grid, dim3(threads), lds, s, a.W, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, 2, PRO, EPI_ROPE_QKV, XB>), grid, dim3(threads), lds, s, a.W, a.x, a.norm_w, a.row_sel, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
             break;
         default:
-            hipLaunchKernelGGL((gemv_kernel<BF16, 2, PRO, EPI_SWIGLU, XB>), grid, dim3(threads), lds, s, a.W, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, 2, PRO, EPI_SWIGLU, XB>), grid, dim3(threads), lds, s, a.W, a.x, a.norm_w, a.row_sel, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
             break;
     }
 }
@@ -454,7 +550,7 @@ static void launch_epi(const GemvArgs &a, dim3 grid, int threads, size_t lds, hi
 template <bool BF16, int R, int XB>
 static void launch_pro(const GemvArgs &a, dim3 grid, int threads, size_t lds, hipStream_t s) {
     if (a.pro == PRO_ATTN_FOLD)  // o_proj only (launch_gemv checks): one row per unit, residual epilogue
-        hipLaunchKernelGGL((gemv_kernel<BF16, 1, PRO_ATTN_FOLD, EPI_RESIDUAL, XB>), grid, dim3(threads), lds, s, a.W, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
+        hipLaunchKernelGGL((gemv_kernel<BF16, 1, PRO_ATTN_FOLD, EPI_RESIDUAL, XB>), grid, dim3(threads), lds, s, a.W, a.x, a.norm_w, a.row_sel, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
     else if (a.pro == PRO_RMSNORM)
         launch_epi<BF16, R, PRO_RMSNORM, XB>(a, grid, threads, lds, s);
     else
@@ -528,12 +624,20 @@ int launch_gemv(lumen_ctx *ctx, const GemvArgs &a) {
     int threads = 0;
     const int blocks = gemv_grid(ctx, a.N, a.K, a.w_bf16, a.epi, &threads);
     dim3 grid(blocks);
-    // pieces of x a thread stages: batched loads from three on (see stage_x)
-    const bool batch_x = (kpad + threads * 4 - 1) / (threads * 4) > 2;
-#define LAUNCH_GEMV(BF, RR)                                                    \
-    do {                                                                       \
-        if (batch_x) launch_pro<BF, RR, 4>(a, grid, threads, lds, ctx->stream); \
-        else launch_pro<BF, RR, 1>(a, grid, threads, lds, ctx->stream);        \
+    // How x is staged (see stage_x, request_early): ahead of the weights where every wavefront has a
+    // single unit of at most two pieces -- all of its loads go out at once and the prologue is what the
+    // multiplies wait for -- and a thread stages at most GEMV_EARLY pieces; else in the loop, four pieces
+    // at a time from three pieces per thread on.
+    const int x_pieces = (kpad + threads * 4 - 1) / (threads * 4);
+    const int nunits = (a.N + R - 1) / R;
+    const bool early_x = a.pro != PRO_ATTN_FOLD && x_pieces <= GEMV_EARLY && kpad / piece <= 2 &&
+                         nunits <= blocks * (threads / 64);
+    const bool batch_x = x_pieces > 2;
+#define LAUNCH_GEMV(BF, RR)                                                         \
+    do {                                                                            \
+        if (early_x) launch_pro<BF, RR, 0>(a, grid, threads, lds, ctx->stream);      \
+        else if (batch_x) launch_pro<BF, RR, 4>(a, grid, threads, lds, ctx->stream); \
+        else launch_pro<BF, RR, 1>(a, grid, threads, lds, ctx->stream);             \
     } while (0)
     if (a.w_bf16) {
         if (R == 2) LAUNCH_GEMV(true, 2);
