@@ -301,8 +301,6 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W
     // pieces (2 x 8 loads per lane) are kept in flight: while one is multiplied the next one is
     // already on its way and the one after is requested as soon as its registers are free.
     const int np = kpad / PIECE;
-    const int my_units = (nunits > gw) ? (nunits - gw + nw - 1) / nw : 0;
-    const int T = my_units * np;
     int lu = gw, lk = 0;  // unit / element offset of the next piece to load
     auto advance_load = [&]() {
         lk += PIECE;
@@ -322,10 +320,14 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W
     v4u rawA[R][U], rawB[R][U];
     load_piece(min(lu, nunits - 1), lk, rawA);
     advance_load();
-    if (T > 1) {
+    // a second piece exists: the unit has one, or the wavefront a second unit (the count of pieces, which
+    // takes a division, is left until both requests are out)
+    if ((kpad > PIECE && gw < nunits) || gw + nw < nunits) {
         load_piece(lu, lk, rawB);
         advance_load();
     }
+    const int my_units = (nunits > gw) ? (nunits - gw + nw - 1) / nw : 0;
+    const int T = my_units * np;
 
     long sel_off = 0;
     const float *xin = x_hot;
