@@ -595,7 +595,12 @@ int gemv_grid(const lumen_ctx *ctx, int N, int K, int w_bf16, int epi, int *thre
     if (per_cu > max_per_cu) per_cu = max_per_cu;
     if (per_cu < 1) per_cu = 1;
     const int cap = ctx->num_cus * per_cu;
-    if (blocks > cap) blocks = cap;
+    if (blocks > cap) {
+        // every wavefront the same number of units: with the grid simply cut at the cap some wavefronts
+        // would take one unit more than the others, and those late, dependent requests are the kernel's tail
+        const int per_wave = (nunits + cap * waves - 1) / (cap * waves);
+        blocks = (nunits + waves * per_wave - 1) / (waves * per_wave);
+    }
     if (threads_out) *threads_out = threads;
     return blocks;
 }
