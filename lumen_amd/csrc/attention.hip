@@ -21,6 +21,7 @@
 //    causal prefix.
 #include "internal.h"
 #include "attn_device.h"
+#include "wave_reduce.h"
 
 #define ATT_WAVES 4
 #define ATT_THREADS (ATT_WAVES * 64)
@@ -125,8 +126,7 @@ __device__ __forceinline__ bool attn_decode_short(const AttnDecodeArgs &a, int r
                 }
                 if (g) {  // per-head RMSNorm before the rotation
                     float sq = x1 * x1 + x2 * x2;
-#pragma unroll
-                    for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o, 64);
+                    sq = wave_sum(sq);
                     const float inv = 1.0f / sqrtf(sq / (float)D + a.norm_eps);
                     x1 = x1 * inv * g1;
                     x2 = x2 * inv * g2;
@@ -282,8 +282,7 @@ __device__ __forceinline__ bool attn_decode_slice(const AttnDecodeArgs &a, int r
             }
             if (g) {  // per-head RMSNorm before the rotation
                 float sq = x1 * x1 + x2 * x2;
-#pragma unroll
-                for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o, 64);
+                sq = wave_sum(sq);
                 const float inv = 1.0f / sqrtf(sq / (float)D + a.norm_eps);
                 x1 = x1 * inv * g1;
                 x2 = x2 * inv * g2;
@@ -373,13 +372,9 @@ __device__ __forceinline__ bool attn_decode_slice(const AttnDecodeArgs &a, int r
             m = -INFINITY;
             l = 0.f;
         }
-        float M = m;
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o, 64));
+        const float M = wave_max(m);
         const float w = (m > -INFINITY) ? fast_exp2(m - M) : 0.f;
-        float L = l * w;
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) L += __shfl_xor(L, o, 64);
+        const float L = wave_sum(l * w);
         w_lds[lane] = w;
         if (lane == 0) w_lds[64] = 1.0f / (L + 1e-9f);
     }

@@ -1,16 +1,12 @@
 // Small HBM-bound kernels of the path: RMSNorm, SiLU / add / mul / SwiGLU,
 // embedding gather, greedy argmax and the tensor form of RoPE.
 #include "internal.h"
+#include "wave_reduce.h"
 
 #include <cmath>
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ float wave_sum_e(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
-}
 
 // ------------------------------------------------------------------ RMSNorm
 // One workgroup per row: sum of squares, rms = sqrt(ss/dim + eps), out = (x * inv) * w.
@@ -26,7 +22,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float *__restrict__ 
         const float v = xr[i];
         ss = fmaf(v, v, ss);
     }
-    ss = wave_sum_e(ss);
+    ss = wave_sum(ss);
     if ((tid & 63) == 0) red[tid >> 6] = ss;
     __syncthreads();
     const float tot = (red[0] + red[1]) + (red[2] + red[3]);

@@ -10,6 +10,7 @@
 // wavefront's rows are walked in pieces of 8 independent 16-byte loads per
 // lane and two pieces are kept in flight (16 loads per lane).
 #include "internal.h"
+#include "wave_reduce.h"
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
@@ -17,22 +18,6 @@ typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 #define GEMV_THREADS 256                  // default workgroup: 4 wavefronts
 #define GEMV_WAVES (GEMV_THREADS / 64)
 #define GEMV_MAX_WAVES 8                  // the launcher picks 4 to 8 wavefronts per workgroup
-
-// Sum over the 64 lanes, the same value in every lane: four DPP rotate-and-add steps leave each row of 16
-// lanes with its total, the four row totals are read through scalar registers.  (Six rounds of
-// ds_bpermute -- what __shfl_xor compiles to -- cost ~0.25 us at the very end of every wavefront.)
-__device__ __forceinline__ float wave_sum(float v) {
-    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false));  // row_ror:8
-    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xf, 0xf, false));  // row_ror:4
-    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xf, 0xf, false));  // row_ror:2
-    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xf, 0xf, false));  // row_ror:1
-    const int b = __float_as_int(v);
-    const float r0 = __int_as_float(__builtin_amdgcn_readlane(b, 0));
-    const float r1 = __int_as_float(__builtin_amdgcn_readlane(b, 16));
-    const float r2 = __int_as_float(__builtin_amdgcn_readlane(b, 32));
-    const float r3 = __int_as_float(__builtin_amdgcn_readlane(b, 48));
-    return (r0 + r1) + (r2 + r3);
-}
 
 __device__ __forceinline__ float silu_f(float g) {
     // x * (1 / (1 + exp(-x))), src/layers/activation.rs:143-146
