@@ -387,11 +387,39 @@ __global__ __launch_bounds__(256, (F == 4 ? 1 : 2)) void gemm_bf16x3_tile_kernel
     store_wave_tiles<EPI, PARTIAL, F>(a, acc, bm, bn, wm, wn, lane);
 }
 
+#define GEMM_MAX_SPLITS 16
 // Adds the K splits of every output element in split order and applies the epilogue.
 template <int EPI>
 __global__ __launch_bounds__(256) void gemm_reduce_kernel(GemmArgs a, int splits) {
     const size_t MN = (size_t)a.M * a.N;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
+    if ((MN & 3) == 0 && splits <= GEMM_MAX_SPLITS && ((((uintptr_t)a.C | (uintptr_t)a.residual | (uintptr_t)a.part) & 15) == 0)) {
+        // four elements per thread; the partials of all splits are requested before the first is added (one
+        // trip to memory instead of one per split), then added in split order as in the scalar loop below
+        typedef float v4 __attribute__((ext_vector_type(4)));
+        for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < MN / 4; q += stride) {
+            v4 pv[GEMM_MAX_SPLITS];
+#pragma unroll
+            for (int s = 0; s < GEMM_MAX_SPLITS; ++s)
+                if (s < splits) pv[s] = *(const v4 *)(a.part + (size_t)s * MN + 4 * q);
+            v4 r4 = {0.f, 0.f, 0.f, 0.f};
+            if (EPI == EPI_RESIDUAL) r4 = *(const v4 *)(a.residual + 4 * q);
+            v4 v = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < GEMM_MAX_SPLITS; ++s)
+                if (s < splits) v += pv[s];
+            if (EPI == EPI_SWIGLU) {
+                // row-major [M, N/2]: pairs 2q, 2q + 1 of the flattened [M, N]
+                a.C[2 * q] = silu_g(v.x) * v.y;
+                a.C[2 * q + 1] = silu_g(v.z) * v.w;
+            } else if (EPI == EPI_RESIDUAL) {
+                *(v4 *)(a.C + 4 * q) = r4 + v;
+            } else {
+                *(v4 *)(a.C + 4 * q) = v;
+            }
+        }
+        return;
+    }
     if (EPI == EPI_SWIGLU) {
         for (size_t p = (size_t)blockIdx.x * blockDim.x + threadIdx.x; p < MN / 2; p += stride) {
             float g = 0.f, u = 0.f;
