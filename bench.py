@@ -151,7 +151,7 @@ def main():
                                "greedy decode, static KV cache max_seq_len %d" % (args.prompt, cfg["max_seq_len"]),
                    "layers": cfg["num_hidden_layers"], "hidden": H, "heads": "32q/4kv", "head_dim": 64,
                    "intermediate": I, "vocab": cfg["vocab_size"], "kv_len_during_timing": [len0, len0 + args.steps]},
-        "roofline": {"bound": "hbm", "kernel": "gemv_kernel<false, 2, 1, 2> (RMSNorm + gate|up GEMV [11264,2048] + SwiGLU)",
+        "roofline": {"bound": "hbm", "kernel": "gemv_kernel<false, 2, 1, 2, 1> (RMSNorm + gate|up GEMV [11264,2048] + SwiGLU)",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic(),
                      "bytes_per_launch": gu_bytes, "avg_launch_us": round(gu_avg_ms * 1e3, 3),
