@@ -233,7 +233,7 @@ __device__ __forceinline__ void stage_attn_fold(float *xs, const GemvArgs &a, in
     __syncthreads();
 }
 
-template <bool BF16, int R, int PRO, int EPI, int XB>
+template <bool BF16, int R, int PRO, int EPI, int XB, bool KA>
 __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W_hot, const float *x_hot,
                                                                   const float *norm_w_hot, const int *row_sel_hot,
                                                                   int N_hot, int K_hot, int D_hot, int nblocks,
@@ -276,7 +276,9 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W
             const char *rp = Wb + (size_t)row * row_bytes;
 #pragma unroll
             for (int uu = 0; uu < U; ++uu) {
-                const int kk = min(k0 + uu * SWEEP + lane * VEC, K - VEC);
+                // KA: K is a whole number of pieces, no position lies past the end of the row -- the eight
+                // addresses are then one base plus constant offsets
+                const int kk = KA ? k0 + uu * SWEEP + lane * VEC : min(k0 + uu * SWEEP + lane * VEC, K - VEC);
                 raw[r][uu] = __builtin_nontemporal_load((const v4u *)(rp + (size_t)kk * ESZ));
             }
         }
@@ -523,35 +525,35 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_generic_kernel(GemvArgs a) 
     }
 }
 
-template <bool BF16, int R, int PRO, int XB>
+template <bool BF16, int R, int PRO, int XB, bool KA>
 static void launch_epi(const GemvArgs &a, dim3 grid, int threads, size_t lds, hipStream_t s) {
     switch (a.epi) {
         case EPI_STORE:
-            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_STORE, XB>), grid, dim3(threads), lds, s, a.W, a.x, a.norm_w, a.row_sel, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_STORE, XB, KA>), grid, dim3(threads), lds, s, a.W, a.x, a.norm_w, a.row_sel, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
             break;
         case EPI_RESIDUAL:
-            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_RESIDUAL, XB>), grid, dim3(threads), lds, s, a.W, a.x, a.norm_w, a.row_sel, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_RESIDUAL, XB, KA>), grid, dim3(threads), lds, s, a.W, a.x, a.norm_w, a.row_sel, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
             break;
         case EPI_ARGMAX:
-            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_ARGMAX, XB>), grid, dim3(threads), lds, s, a.W, a.x, a.norm_w, a.row_sel, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, R, PRO, EPI_ARGMAX, XB, KA>), grid, dim3(threads), lds, s, a.W, a.x, a.norm_w, a.row_sel, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
             break;
         case EPI_ROPE_QKV:
-            hipLaunchKernelGGL((gemv_kernel<BF16, 2, PRO, EPI_ROPE_QKV, XB>), grid, dim3(threads), lds, s, a.W, a.x, a.norm_w, a.row_sel, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, 2, PRO, EPI_ROPE_QKV, XB, KA>), grid, dim3(threads), lds, s, a.W, a.x, a.norm_w, a.row_sel, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
             break;
         default:
-            hipLaunchKernelGGL((gemv_kernel<BF16, 2, PRO, EPI_SWIGLU, XB>), grid, dim3(threads), lds, s, a.W, a.x, a.norm_w, a.row_sel, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
+            hipLaunchKernelGGL((gemv_kernel<BF16, 2, PRO, EPI_SWIGLU, XB, KA>), grid, dim3(threads), lds, s, a.W, a.x, a.norm_w, a.row_sel, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
             break;
     }
 }
 
-template <bool BF16, int R, int XB>
+template <bool BF16, int R, int XB, bool KA>
 static void launch_pro(const GemvArgs &a, dim3 grid, int threads, size_t lds, hipStream_t s) {
     if (a.pro == PRO_ATTN_FOLD)  // o_proj only (launch_gemv checks): one row per unit, residual epilogue
-        hipLaunchKernelGGL((gemv_kernel<BF16, 1, PRO_ATTN_FOLD, EPI_RESIDUAL, XB>), grid, dim3(threads), lds, s, a.W, a.x, a.norm_w, a.row_sel, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
+        hipLaunchKernelGGL((gemv_kernel<BF16, 1, PRO_ATTN_FOLD, EPI_RESIDUAL, XB, KA>), grid, dim3(threads), lds, s, a.W, a.x, a.norm_w, a.row_sel, a.N, a.K, a.D, (int)grid.x, threads >> 6, a);
     else if (a.pro == PRO_RMSNORM)
-        launch_epi<BF16, R, PRO_RMSNORM, XB>(a, grid, threads, lds, s);
+        launch_epi<BF16, R, PRO_RMSNORM, XB, KA>(a, grid, threads, lds, s);
     else
-        launch_epi<BF16, R, PRO_NONE, XB>(a, grid, threads, lds, s);
+        launch_epi<BF16, R, PRO_NONE, XB, KA>(a, grid, threads, lds, s);
 }
 
 // Grid of the fused kernel for an [N, K] product: workgroups and threads per workgroup.
@@ -635,11 +637,17 @@ int launch_gemv(lumen_ctx *ctx, const GemvArgs &a) {
     const bool early_x = a.pro != PRO_ATTN_FOLD && x_pieces <= GEMV_EARLY && kpad / piece <= 2 &&
                          nunits <= blocks * (threads / 64);
     const bool batch_x = x_pieces > 2;
-#define LAUNCH_GEMV(BF, RR)                                                         \
-    do {                                                                            \
-        if (early_x) launch_pro<BF, RR, 0>(a, grid, threads, lds, ctx->stream);      \
-        else if (batch_x) launch_pro<BF, RR, 4>(a, grid, threads, lds, ctx->stream); \
-        else launch_pro<BF, RR, 1>(a, grid, threads, lds, ctx->stream);             \
+    const bool ka = a.K % piece == 0;  // whole pieces: no clamped load positions
+#define LAUNCH_GEMV_K(BF, RR, KAV)                                                       \
+    do {                                                                                 \
+        if (early_x) launch_pro<BF, RR, 0, KAV>(a, grid, threads, lds, ctx->stream);      \
+        else if (batch_x) launch_pro<BF, RR, 4, KAV>(a, grid, threads, lds, ctx->stream); \
+        else launch_pro<BF, RR, 1, KAV>(a, grid, threads, lds, ctx->stream);             \
+    } while (0)
+#define LAUNCH_GEMV(BF, RR)                  \
+    do {                                     \
+        if (ka) LAUNCH_GEMV_K(BF, RR, true); \
+        else LAUNCH_GEMV_K(BF, RR, false);   \
     } while (0)
     if (a.w_bf16) {
         if (R == 2) LAUNCH_GEMV(true, 2);
@@ -649,6 +657,7 @@ int launch_gemv(lumen_ctx *ctx, const GemvArgs &a) {
         else LAUNCH_GEMV(false, 1);
     }
 #undef LAUNCH_GEMV
+#undef LAUNCH_GEMV_K
     LUMEN_CHECK_LAUNCH();
     return LUMEN_OK;
 }
