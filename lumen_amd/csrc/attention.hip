@@ -347,11 +347,11 @@ __device__ __forceinline__ bool attn_decode_slice(const AttnDecodeArgs &a, int r
         }
     }
     if (nact == 1 || a.defer_merge) return true;  // one slice, or the consumer folds them
-    // The barrier makes every wavefront wait for its own stores before thread 0 signals.
+    // every wavefront's stores are ordered before thread 0's arrival by the barrier (see handover_arrive)
     __syncthreads();
     if (t == 0) {
         int *counter = a.counters + (size_t)bb * a.hq + hq;
-        const int old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int old = handover_arrive(counter);
         *s_last = (old == nact - 1);
         if (*s_last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
@@ -685,9 +685,13 @@ extern "C" int lumen_kv_cache_create(lumen_ctx *ctx, int b, int h_kv, int max_se
         LUMEN_FAIL(LUMEN_ERR_HIP, "kv_cache_create: hipMalloc of 2 x %zu bytes failed", bytes);
     }
     // zero-initialised like Array4::zeros (self_attention.rs:35-36); eager, never graph-captured
-    HIP_TRY(hipMemsetAsync(c->k, 0, bytes, ctx->stream));
-    HIP_TRY(hipMemsetAsync(c->v, 0, bytes, ctx->stream));
-    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    if (hipMemsetAsync(c->k, 0, bytes, ctx->stream) != hipSuccess || hipMemsetAsync(c->v, 0, bytes, ctx->stream) != hipSuccess ||
+        hipStreamSynchronize(ctx->stream) != hipSuccess) {
+        hipFree(c->k);
+        hipFree(c->v);
+        delete c;
+        LUMEN_FAIL(LUMEN_ERR_HIP, "kv_cache_create: clearing 2 x %zu bytes failed", bytes);
+    }
     *out = c;
     return LUMEN_OK;
 }
@@ -701,6 +705,7 @@ extern "C" int lumen_kv_cache_destroy(lumen_kv_cache *c) {
     }
     hipFree(c->part);
     hipFree(c->counters);
+    hipFree(c->q_rot);
     delete c;
     return LUMEN_OK;
 }
@@ -809,17 +814,24 @@ extern "C" int lumen_attn_prefill_f32(lumen_kv_cache *c, lumen_rope *rope, const
     if (new_len > c->max_seq)  // self_attention.rs:341-346
         LUMEN_FAIL(LUMEN_ERR_KV_OVERFLOW, "KV cache overflow: new_len=%d > max_seq=%d", new_len, c->max_seq);
     if (s == 0) return LUMEN_OK;
-    float *q_rot = nullptr;
-    HIP_TRY(hipMalloc((void **)&q_rot, sizeof(float) * (size_t)c->b * s * h * c->d));
+    // rotated queries: scratch kept on the cache, grown (with a stream synchronisation) only when a call needs more
+    const size_t q_floats = (size_t)c->b * s * h * c->d;
+    if (q_floats > c->q_rot_floats) {
+        HIP_TRY(hipStreamSynchronize(c->ctx->stream));
+        hipFree(c->q_rot);
+        c->q_rot = nullptr;
+        c->q_rot_floats = 0;
+        HIP_TRY(hipMalloc((void **)&c->q_rot, sizeof(float) * q_floats));
+        c->q_rot_floats = q_floats;
+    }
+    float *q_rot = c->q_rot;
     AttnPrefillArgs a = {};
     a.q = q; a.k = k; a.v = v; a.out = out; a.k_cache = c->k; a.v_cache = c->v;
     a.cos_t = rope->cos_dev; a.sin_t = rope->sin_dev;
     a.b = c->b; a.s = s; a.hq = h; a.hkv = c->h_kv; a.d = c->d; a.max_seq = c->max_seq; a.past_len = past_len;
     a.q_stride = h * c->d; a.k_stride = c->h_kv * c->d; a.v_stride = c->h_kv * c->d;
     a.scale = scale; a.causal = causal; a.q_rot = q_rot;
-    int rc = launch_attn_prefill(c->ctx, a);
-    hipStreamSynchronize(c->ctx->stream);
-    hipFree(q_rot);
+    const int rc = launch_attn_prefill(c->ctx, a);
     if (rc == LUMEN_OK) c->len = new_len;
     return rc;
 }

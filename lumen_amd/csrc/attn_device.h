@@ -1,6 +1,6 @@
 // Device-side building blocks of GQA attention over the static KV cache,
-// shared by the stand-alone attention kernels and the persistent decode
-// kernel.  WAVES = wavefronts per workgroup (64 lanes each).
+// shared by the decode and the row-loop prefill attention kernels.
+// WAVES = wavefronts per workgroup (64 lanes each).
 //
 // Lane mapping: a K/V row of D floats is covered by LPR = D/4 lanes holding
 // 16 bytes each, so one 64-lane load instruction fetches 64/LPR rows.  Every
@@ -9,9 +9,7 @@
 // registers.
 #pragma once
 
-#ifndef LUMEN_CPU_EMU
 #include <hip/hip_runtime.h>
-#endif
 #include <cmath>
 
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -293,109 +291,4 @@ __device__ __forceinline__ void part_store(float *p, float v) {
 }
 __device__ __forceinline__ float part_load(const float *p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// Folds the nact partial states of head-dim element (hq, dd) in slice order: out = ctx / (l + 1e-9),
-// self_attention.rs:287-290.  pp points at the head's first partial; entries are (D + 2) floats apart.
-template <int D>
-__device__ __forceinline__ float fold_slices(const float *pp, int nact, int dd) {
-    constexpr int B = 8;  // slices fetched together: 3 * B independent loads in flight, one wait
-    float M = -INFINITY, Ls = 0.f, Cx = 0.f;
-    for (int s0 = 0; s0 < nact; s0 += B) {
-        float mv[B], lv[B], cv[B];
-#pragma unroll
-        for (int j = 0; j < B; ++j) {
-            const float *e = pp + (size_t)min(s0 + j, nact - 1) * (D + 2);
-            mv[j] = part_load(e + D);
-            lv[j] = part_load(e + D + 1);
-            cv[j] = part_load(e + dd);
-        }
-#pragma unroll
-        for (int j = 0; j < B; ++j) {
-            if (s0 + j < nact && mv[j] > -INFINITY) {
-                const float mn = fmaxf(M, mv[j]);
-                const float a = fast_exp2(M - mn), b = fast_exp2(mv[j] - mn);
-                Ls = Ls * a + lv[j] * b;
-                Cx = Cx * a + cv[j] * b;
-                M = mn;
-            }
-        }
-    }
-    return Cx * (1.0f / (Ls + 1e-9f));
-}
-
-// The same fold for a whole KV group by one workgroup, with one trip to memory instead of one per
-// batch of slices: every thread first requests the context partials of its own output element
-// (up to 32 slices, held in registers), then wavefront r reads the (max, sum) pairs of head r --
-// lane s takes slice s -- and leaves the slice weights exp2(m_s - M) and 1 / (sum + 1e-9) in LDS;
-// after the barrier the partials are already there.  More than 32 slices take a second trip.
-// part_group: partials of the group's first head; heads are nsplit * (D + 2) floats apart.
-// w_lds [NREP][64], linv_lds [NREP].  All threads of the workgroup call it; nsplit <= 64.
-template <int D, int NREP, int WAVES, int B>
-__device__ __forceinline__ void fold_slices_block_b(const float *part_group, int nsplit, int nact, float *w_lds,
-                                                    float *linv_lds, float *out_group) {
-    constexpr int THREADS = WAVES * 64;
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const size_t head_stride = (size_t)nsplit * (D + 2);
-    // context partials of the first output element of this thread
-    float cv[B];
-    if (t < NREP * D) {
-        const float *pp = part_group + (t / D) * head_stride + t % D;
-#pragma unroll
-        for (int j = 0; j < B; ++j) cv[j] = part_load(pp + (size_t)min(j, nact - 1) * (D + 2));
-    }
-    for (int r = wave; r < NREP; r += WAVES) {
-        const float *pp = part_group + r * head_stride + (size_t)min(lane, nact - 1) * (D + 2);
-        float m = part_load(pp + D), l = part_load(pp + D + 1);
-        if (lane >= nact) {
-            m = -INFINITY;
-            l = 0.f;
-        }
-        float M = m;
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off, 64));
-        const float w = (m > -INFINITY) ? fast_exp2(m - M) : 0.f;
-        float L = l * w;
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) L += __shfl_xor(L, off, 64);
-        w_lds[r * 64 + lane] = w;
-        if (lane == 0) linv_lds[r] = 1.0f / (L + 1e-9f);
-    }
-    __syncthreads();
-    for (int e = t; e < NREP * D; e += THREADS) {
-        const int r = e / D, dd = e % D;
-        const float *pp = part_group + r * head_stride + dd;
-        float acc = 0.f;
-        for (int s0 = 0; s0 < nact; s0 += B) {
-            if (e != t || s0 != 0) {
-#pragma unroll
-                for (int j = 0; j < B; ++j) cv[j] = part_load(pp + (size_t)min(s0 + j, nact - 1) * (D + 2));
-            }
-#pragma unroll
-            for (int j = 0; j < B; ++j)
-                if (s0 + j < nact) acc = fmaf(cv[j], w_lds[r * 64 + s0 + j], acc);
-        }
-        out_group[r * D + dd] = acc * linv_lds[r];
-    }
-}
-
-template <int D, int NREP, int WAVES>
-__device__ __forceinline__ void fold_slices_block(const float *part_group, int nsplit, int nact, float *w_lds,
-                                                  float *linv_lds, float *out_group) {
-    if (nact <= 8) fold_slices_block_b<D, NREP, WAVES, 8>(part_group, nsplit, nact, w_lds, linv_lds, out_group);
-    else if (nact <= 16) fold_slices_block_b<D, NREP, WAVES, 16>(part_group, nsplit, nact, w_lds, linv_lds, out_group);
-    else fold_slices_block_b<D, NREP, WAVES, 32>(part_group, nsplit, nact, w_lds, linv_lds, out_group);
-}
-
-// How the cached rows [0, pos) are cut into slices for one decode step: only
-// as many slices as give each at least one full trip of rows take part, the
-// others return at once.  The new token (row `pos`) belongs to the last
-// active slice.
-template <int D, int WAVES>
-__device__ __forceinline__ void decode_slices(int pos, int nsplit, int &nact, int &chunk) {
-    typedef AttnGeom<D, WAVES> G;
-    nact = (pos + G::ROWS_PER_TRIP - 1) / G::ROWS_PER_TRIP;
-    nact = nact < 1 ? 1 : (nact > nsplit ? nsplit : nact);
-    chunk = (pos + nact - 1) / nact;
-    chunk = (chunk + G::RPI - 1) / G::RPI * G::RPI;
 }

@@ -454,9 +454,9 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W
             __hip_atomic_store(a.amax_val + blockIdx.x, best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(a.amax_idx + blockIdx.x, best_idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        __syncthreads();  // thread 0's stores are complete past this barrier
+        __syncthreads();
         if (threadIdx.x == 0) {
-            const int old = __hip_atomic_fetch_add(a.amax_counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const int old = handover_arrive(a.amax_counter);
             am_last = (old == nblocks - 1);
             if (am_last) __hip_atomic_store(a.amax_counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }

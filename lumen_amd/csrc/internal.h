@@ -66,6 +66,8 @@ struct lumen_kv_cache {
     float *part = nullptr;  // [b*h_q_max, nsplit, d + 2]
     int *counters = nullptr;
     int part_heads = 0;
+    float *q_rot = nullptr;  // rotated queries of the prefill entry point, grown on demand
+    size_t q_rot_floats = 0;
 };
 
 // ---------------------------------------------------------------- launchers

@@ -9,7 +9,6 @@
 // replayed per token; greedy generation never returns to the host between
 // tokens.
 #include "internal.h"
-#include "decode_persistent.h"
 
 #include <algorithm>
 #include <cmath>
@@ -45,17 +44,13 @@ struct lumen_llama {
     int *counters = nullptr;
     int nsplit = 1;     // slices of a long cache in the decode attention kernel
     bool defer_merge = false;  // the o_proj GEMV, not the attention kernel, may merge the slices of a long cache
-    int pk_nsplit = 1;  // the same for the persistent kernel (its own slicing: 64 rows per slice, 64 at most)
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
     int graph_expect_short = 0;            // the hint the captured attention launches carry
-    int decode_mode = LUMEN_DECODE_GRAPH;  // persistent when the shape allows, set at create
-    PkLayer *pk_layers = nullptr;          // device copy of the per-layer pointers
+    int decode_mode = LUMEN_DECODE_GRAPH;
     float *amax_val = nullptr;
     int *amax_idx = nullptr;
     int *amax_counter = nullptr;
-    unsigned *d_bar = nullptr;
-    int *d_err = nullptr;
     // prefill buffers (grown on demand, kept)
     int pf_cap = 0, pf_logit_cap = 0;
     float *p_x = nullptr, *p_h = nullptr, *p_n = nullptr, *p_qkv = nullptr, *p_qrot = nullptr, *p_attn = nullptr,
@@ -63,11 +58,6 @@ struct lumen_llama {
     int *p_ids = nullptr;
     std::vector<void *> allocs;
 };
-
-// The persistent kernel stays off the GPU until the cause of the memory fault of its first run is known.
-static const bool PERSISTENT_KERNEL_ENABLED = false;
-
-static bool persistent_ok(const lumen_llama *m);
 
 static int dmalloc(lumen_llama *m, void **p, size_t bytes) {
     HIP_TRY(hipMalloc(p, bytes ? bytes : 16));
@@ -192,8 +182,7 @@ extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg,
                               GEMV_FOLD_MAX_SLICES * sizeof(float);
     m->defer_merge = m->nsplit >= 2 && m->nsplit <= GEMV_FOLD_MAX_SLICES && !cfg->qk_norm &&
                      cfg->max_seq_len <= m->nsplit * attn_decode_trip_rows(D) && fold_bytes <= ((size_t)64 << 20);
-    m->pk_nsplit = cfg->max_seq_len / 64 < 1 ? 1 : (cfg->max_seq_len / 64 > 64 ? 64 : cfg->max_seq_len / 64);
-    M_TRY(dmalloc_t(m, &m->part, attn_decode_part_floats(1, Hq, D, m->nsplit > m->pk_nsplit ? m->nsplit : m->pk_nsplit)));
+    M_TRY(dmalloc_t(m, &m->part, attn_decode_part_floats(1, Hq, D, m->nsplit)));
     M_TRY(dmalloc_t(m, &m->counters, (size_t)Hq));
     if (hipMemsetAsync(m->counters, 0, sizeof(int) * Hq, ctx->stream) != hipSuccess ||
         hipMemsetAsync(m->d_tok, 0, 4 * sizeof(int), ctx->stream) != hipSuccess ||
@@ -203,14 +192,6 @@ extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg,
         LUMEN_FAIL(LUMEN_ERR_HIP, "llama_create: clearing decode state failed");
     }
     {
-        std::vector<PkLayer> pl(L);
-        for (int l = 0; l < L; ++l) {
-            const LayerW &w = m->layers[l];
-            pl[l] = PkLayer{w.wqkv, w.wo, w.wgu, w.wdown, w.in_norm, w.post_norm, w.q_norm, w.k_norm,
-                            m->k_slab + m->cache_stride * l, m->v_slab + m->cache_stride * l};
-        }
-        M_TRY(dmalloc_t(m, &m->pk_layers, (size_t)L));
-        M_TRY(lumen_upload(ctx, m->pk_layers, pl.data(), sizeof(PkLayer) * (size_t)L));
         const size_t nb = (size_t)std::max(gemv_max_blocks(ctx), ctx->num_cus);
         M_TRY(dmalloc_t(m, &m->amax_val, nb));
         M_TRY(dmalloc_t(m, &m->amax_idx, nb));
@@ -220,10 +201,8 @@ extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg,
             lumen_llama_destroy(m);
             LUMEN_FAIL(LUMEN_ERR_HIP, "llama_create: clearing the arg-max counter failed");
         }
-        M_TRY(dmalloc_t(m, &m->d_bar, 4));
-        M_TRY(dmalloc_t(m, &m->d_err, 4));
     }
-    m->decode_mode = (PERSISTENT_KERNEL_ENABLED && persistent_ok(m)) ? LUMEN_DECODE_PERSISTENT : LUMEN_DECODE_GRAPH;
+    m->decode_mode = LUMEN_DECODE_GRAPH;
 #undef M_TRY
     *out = m;
     return LUMEN_OK;
@@ -538,54 +517,14 @@ static hipError_t launch_step(lumen_llama *m) {
     return enqueue_decode_step(m) == LUMEN_OK ? hipSuccess : hipErrorLaunchFailure;
 }
 
-static void fill_pk_args(const lumen_llama *m, PkArgs &a) {
-    const lumen_llama_config &c = m->cfg;
-    a = PkArgs{};
-    a.layers = m->pk_layers; a.n_layers = c.num_hidden_layers;
-    a.H = c.hidden_size; a.I = c.intermediate_size; a.V = c.vocab_size; a.qd = m->qd; a.kvd = m->kvd;
-    a.hq = c.num_attention_heads; a.hkv = c.num_key_value_heads; a.D = m->D; a.max_seq = c.max_seq_len;
-    a.nsplit = m->pk_nsplit; a.eps = c.rms_norm_eps; a.scale = m->scale; a.w_bf16 = m->bf16;
-    a.embed = m->embed; a.lm_head = m->lm_head; a.final_norm = m->final_norm;
-    a.cos_t = m->cos_dev; a.sin_t = m->sin_dev;
-    a.x = m->x; a.h = m->h; a.qkv = m->qkv; a.attn = m->attn; a.act = m->act; a.logits = m->logits;
-    a.part = m->part; a.head_counters = m->counters; a.tok = m->d_tok; a.pos = m->d_pos;
-    a.bar = m->d_bar; a.err = m->d_err; a.amax_val = m->amax_val; a.amax_idx = m->amax_idx;
-}
-
-static bool persistent_ok(const lumen_llama *m) {
-    PkArgs a;
-    fill_pk_args(m, a);
-    return pk_supported(a);
-}
-
-// n decode steps in one cooperative launch; ids_dev [n] / logits_dev [n,V] optional device buffers
-static int run_persistent(lumen_llama *m, int n, int *ids_dev, float *logits_dev) {
-    PkArgs a;
-    fill_pk_args(m, a);
-    a.n_steps = n; a.ids_out = ids_dev; a.logits_out = logits_dev;
-    LUMEN_TRY(launch_decode_persistent(m->ctx, a));
-    int err = 0;
-    HIP_TRY(hipMemcpyAsync(&err, m->d_err, sizeof(int), hipMemcpyDeviceToHost, m->ctx->stream));
-    HIP_TRY(hipStreamSynchronize(m->ctx->stream));
-    if (err) {
-        LUMEN_FAIL(LUMEN_ERR_HIP, "persistent decode kernel: a grid barrier ran into its time limit "
-                                  "(workgroups not co-resident?); model state is undefined, reset it");
-    }
-    m->len += n;
-    return LUMEN_OK;
-}
-
 extern "C" int lumen_llama_set_decode_mode(lumen_llama *m, int mode) {
     if (!m) LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_set_decode_mode: null model");
     if (mode != LUMEN_DECODE_EAGER && mode != LUMEN_DECODE_GRAPH && mode != LUMEN_DECODE_PERSISTENT)
         LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_set_decode_mode: unknown mode %d", mode);
-    if (mode == LUMEN_DECODE_PERSISTENT && !persistent_ok(m))
-        LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "the persistent decode kernel needs head_dim 64 or 128 and n_rep 1, 2, 4 or 8");
-    if (mode == LUMEN_DECODE_PERSISTENT && !PERSISTENT_KERNEL_ENABLED)
+    if (mode == LUMEN_DECODE_PERSISTENT)
         LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED,
-                   "the persistent decode kernel is switched off: its first run on the GPU ended in a memory fault "
-                   "whose cause is not established (the same code is clean under Address/Thread/MemorySanitizer on "
-                   "the CPU); use LUMEN_DECODE_GRAPH");
+                   "this library holds no persistent decode kernel (a grid-wide hand-over costs more on this chip "
+                   "than the kernel boundary it would replace); use LUMEN_DECODE_GRAPH");
     m->decode_mode = mode;
     return LUMEN_OK;
 }
@@ -721,12 +660,8 @@ extern "C" int lumen_llama_forward(lumen_llama *m, const float *ids_host, int s,
     hipStream_t st = m->ctx->stream;
     HIP_TRY(hipMemcpyAsync(m->d_tok, ids.data(), sizeof(int), hipMemcpyHostToDevice, st));
     HIP_TRY(hipStreamSynchronize(st));
-    if (m->decode_mode == LUMEN_DECODE_PERSISTENT) {
-        LUMEN_TRY(run_persistent(m, 1, nullptr, nullptr));
-    } else {
-        HIP_TRY(launch_step(m));
-        m->len += 1;
-    }
+    HIP_TRY(launch_step(m));
+    m->len += 1;
     if (logits_host) return lumen_download(m->ctx, logits_host, m->logits, sizeof(float) * (size_t)m->cfg.vocab_size);
     return LUMEN_OK;
 }
@@ -744,24 +679,6 @@ extern "C" int lumen_llama_decode_greedy(lumen_llama *m, int first_id, int n, in
     const size_t V = (size_t)m->cfg.vocab_size;
     HIP_TRY(hipMemcpyAsync(m->d_tok, &first_id, sizeof(int), hipMemcpyHostToDevice, st));
     HIP_TRY(hipStreamSynchronize(st));
-    if (m->decode_mode == LUMEN_DECODE_PERSISTENT) {
-        int *ids_dev = nullptr;
-        if (ids_out) HIP_TRY(hipMalloc((void **)&ids_dev, sizeof(int) * (size_t)n));
-        float *logits_dev = nullptr;
-        if (logits_out && hipMalloc((void **)&logits_dev, sizeof(float) * V * (size_t)n) != hipSuccess) {
-            hipFree(ids_dev);
-            LUMEN_FAIL(LUMEN_ERR_HIP, "decode_greedy: no memory for %d x %zu logits", n, V);
-        }
-        int prc = run_persistent(m, n, ids_dev, logits_dev);
-        hipError_t pe = hipSuccess;
-        if (prc == LUMEN_OK && ids_dev) pe = hipMemcpy(ids_out, ids_dev, sizeof(int) * (size_t)n, hipMemcpyDeviceToHost);
-        if (prc == LUMEN_OK && pe == hipSuccess && logits_dev)
-            pe = hipMemcpy(logits_out, logits_dev, sizeof(float) * V * (size_t)n, hipMemcpyDeviceToHost);
-        hipFree(ids_dev);
-        hipFree(logits_dev);
-        if (prc == LUMEN_OK && pe != hipSuccess) LUMEN_FAIL(LUMEN_ERR_HIP, "decode_greedy: %s", hipGetErrorString(pe));
-        return prc;
-    }
     // the arg-max epilogue leaves every pick in tok_hist at the index of the position it is the token of
     const int len0 = m->len;
     int rc = LUMEN_OK;

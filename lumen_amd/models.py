@@ -151,8 +151,8 @@ class LlamaModel:
     DECODE_MODES = {"eager": _lib.DECODE_EAGER, "graph": _lib.DECODE_GRAPH, "persistent": _lib.DECODE_PERSISTENT}
 
     def set_decode_mode(self, mode):
-        """'persistent' (one cooperative kernel for all layers and steps), 'graph' (HIP graph replay
-        per token) or 'eager' (kernel by kernel)."""
+        """'graph' (HIP graph replay per token) or 'eager' (kernel by kernel); 'persistent' is refused
+        (the library holds no such kernel)."""
         check(lib.lumen_llama_set_decode_mode(self.handle, self.DECODE_MODES[mode]))
 
     @property

@@ -192,13 +192,11 @@ MHA128 = dict(vocab_size=700, hidden_size=256, intermediate_size=704, num_hidden
               num_key_value_heads=2, rms_norm_eps=1e-5, max_seq_len=300, rope_theta=10000.0)  # head_dim 128, n_rep 1
 
 
-# The persistent decode kernel is switched off in the library: its first run on the GPU ended in a
-# memory fault whose cause is not established, so it must not run on a GPU.  Its logic is covered on
-# the CPU by tests/test_cpu_emu.py (ASan build of the same device code against the oracle).
+# The library holds no persistent decode kernel (the mode constant is kept so that callers get a clear refusal).
 MODES = ("graph", "eager")
 
 
-def test_persistent_mode_is_refused_while_switched_off():
+def test_persistent_mode_is_refused():
     gpu, _, _ = build(GQA64, seed=20)
     assert gpu.decode_mode == "graph"
     with pytest.raises(_lib.LumenError) as e:
@@ -267,6 +265,86 @@ def test_decode_across_the_short_to_split_attention_boundary(cfg_extra, n_prompt
     assert gpu.kv_len == n_prompt + 14
 
 
+def _greedy_call_checked(gpu, ora, first, n, tol):
+    """ONE decode_greedy call of n steps; the checker is then fed the GPU's own picks, so every step's
+    logits are compared on identical inputs whatever a near-tie does to the sequence."""
+    picks, logits = gpu.decode_greedy(first, n, want_logits=True)
+    tok = first
+    for t in range(n):
+        _, r = ora.forward(np.array([tok]))
+        assert max_rel(logits[t], r[0]) <= tol, (t, max_rel(logits[t], r[0]))
+        check_argmax(logits[t], r[0], tol)
+        tok = int(picks[t])
+    return picks, logits
+
+
+@pytest.mark.parametrize("cfg_extra,n_prompt,same_bits", [
+    (dict(num_attention_heads=8, num_key_value_heads=2, max_seq_len=4096), 492, False),  # slices merged by o_proj when eager
+    (dict(num_attention_heads=8, num_key_value_heads=1, max_seq_len=4096), 490, False),  # n_rep 8: remapped head index
+    (dict(num_attention_heads=8, num_key_value_heads=2, max_seq_len=1100, qk_norm=True, head_dim=64), 494, True),  # norm + rotation in the kernel
+    (dict(hidden_size=256, num_attention_heads=2, num_key_value_heads=1, max_seq_len=700, intermediate_size=704), 236, False),  # head_dim 128: 256 rows
+    (dict(hidden_size=256, num_attention_heads=2, num_key_value_heads=1, max_seq_len=700, intermediate_size=704, qk_norm=True, head_dim=128), 236, True),
+], ids=["d64-nrep4-defer", "d64-nrep8-defer", "d64-qknorm", "d128", "d128-qknorm"])
+def test_one_greedy_call_replays_a_graph_across_the_attention_boundary(cfg_extra, n_prompt, same_bits):
+    """A single decode_greedy call captures its graph once, on the short side of the attention boundary (512 cached
+    rows, 256 for head_dim 128), and keeps replaying it on the long side: the captured launches then carry a stale
+    hint and the kernel hands over to the sliced form by itself.  Every step of such a call is held to the checker,
+    and to the eager launches of the same steps (whose hint is right at every step; where the eager steps leave the
+    merge of the slices to o_proj the two differ in summation order, elsewhere they are bit-equal)."""
+    cfg = dict(vocab_size=900, hidden_size=512, intermediate_size=1408, num_hidden_layers=2, rms_norm_eps=1e-5,
+               rope_theta=10000.0)
+    cfg.update(cfg_extra)
+    gpu, ora, _ = build(cfg, seed=41)
+    ids = synth.make_tokens(n_prompt, cfg["vocab_size"], seed=41)
+    n = 40
+    results = {}
+    for mode in MODES:
+        gpu.reset_kv_caches()
+        ora.reset()
+        gpu.set_decode_mode(mode)
+        got = gpu.forward(ids, all_rows=False)
+        _, ref = ora.forward(ids)
+        assert max_rel(got, ref[-1]) <= 1e-4
+        results[mode] = _greedy_call_checked(gpu, ora, lo.argmax(ref[-1]), n, 1e-4)
+        assert gpu.kv_len == n_prompt + n
+    (pg, lg), (pe, le) = results["graph"], results["eager"]
+    if same_bits:
+        assert np.array_equal(lg, le) and np.array_equal(pg, pe)
+    elif np.array_equal(pg, pe):
+        assert max_rel(lg, le) <= 1e-5
+
+
+@pytest.mark.parametrize("qk_norm", [False, True], ids=["merge-in-oproj", "merge-in-kernel"])
+def test_sliced_attention_decode_is_bit_reproducible(qk_norm):
+    """The same 64 greedy steps at ~4000 cached rows (16 slices per head, partial states handed from
+    workgroup to workgroup through memory) give the same bits every time, whether the slices are merged by
+    the attention kernel's last workgroup (q/k-norm model) or by the o_proj product."""
+    cfg = dict(vocab_size=900, hidden_size=256, intermediate_size=704, num_hidden_layers=2, rms_norm_eps=1e-5,
+               rope_theta=10000.0, num_attention_heads=4, num_key_value_heads=2, max_seq_len=4096)
+    if qk_norm:
+        cfg.update(qk_norm=True, head_dim=64)
+    gpu, ora, _ = build(cfg, seed=43)
+    ids = synth.make_tokens(3960, cfg["vocab_size"], seed=43)
+    first = None
+    for rep in range(20):
+        gpu.reset_kv_caches()
+        last = gpu.forward(ids, all_rows=False)
+        picks, logits = gpu.decode_greedy(int(np.argmax(last)), 64, want_logits=True)
+        if first is None:
+            first = (last, picks, logits)
+            _, ref = ora.forward(ids)
+            assert max_rel(last, ref[-1]) <= 1e-4
+            tok = int(np.argmax(last))
+            for t in range(64):
+                _, r = ora.forward(np.array([tok]))
+                assert max_rel(logits[t], r[0]) <= 1e-4, t
+                tok = int(picks[t])
+        else:
+            assert np.array_equal(last, first[0]), rep
+            assert np.array_equal(picks, first[1]), rep
+            assert np.array_equal(logits, first[2]), rep
+
+
 @pytest.mark.slow
 def test_tinyllama_1b_shape_prefill_128_decode_teacher_forced():
     """The headline configuration at full size: 22 layers, hidden 2048, 32/4 heads, vocab 32000,
@@ -329,21 +407,35 @@ def _prefill_decode_check(gpu, ora, vocab, n_prompt, n_dec, tol, seed):
 
 
 @pytest.mark.slow
-def test_long_context_tinyllama_shape_3968_prompt():
-    """Config 3 at full width and full context (prompt 3968, decode to the 4096 limit region) on 3 of the
-    22 layers: every kernel shape and the 62-slice attention merge are the real ones."""
+def test_long_context_tinyllama_shape_3968_prompt_decode_to_the_last_row():
+    """Config 3 at full width and full context on 3 of the 22 layers (every kernel shape and the 16-slice
+    attention merge are the real ones): prompt 3968, 12 teacher-forced steps, then ONE greedy call of 116
+    steps that fills the 4096-row cache to its last row; the step after that is refused like the
+    reference's assert (self_attention.rs:144-149)."""
     cfg = dict(synth.TINYLLAMA_1B_LONG, num_hidden_layers=3)
     gpu, ora = _stream_build(cfg, seed=3)
     _prefill_decode_check(gpu, ora, cfg["vocab_size"], 3968, 12, 1e-4, seed=3)
+    _greedy_call_checked(gpu, ora, 17, 116, 1e-4)
+    assert gpu.kv_len == ora.kv_len == cfg["max_seq_len"] == 4096
+    k, _ = gpu.cache(2)
+    assert max_rel(k[:, :, 4090:], ora.cache_k(2)[:, :, 4090:]) <= 1e-4 and np.abs(k[:, :, 4095]).max() > 0
+    for call in (lambda: gpu.forward(np.array([1]), all_rows=False), lambda: gpu.decode_greedy(1, 1)):
+        with pytest.raises(_lib.LumenError) as e:
+            call()
+        assert e.value.status == _lib.ERR_KV_OVERFLOW
+    assert gpu.kv_len == 4096
 
 
 @pytest.mark.slow
-def test_qwen3_0p6b_shape_prefill_256_decode():
-    """Config 4 shape (head_dim 128 decoupled from hidden 1024, per-head q/k RMSNorm, tied 151936-row
-    embedding, rope_theta 1e6) on 4 of the 28 layers; no reference model exists for it (oracle-extrapolated)."""
-    cfg = dict(synth.QWEN3_0P6B, num_hidden_layers=4)
+def test_qwen3_0p6b_shape_full_depth_prefill_256_decode():
+    """Config 4 at full size: 28 layers, head_dim 128 decoupled from hidden 1024, per-head q/k RMSNorm, tied
+    151936-row embedding, rope_theta 1e6; prompt 256 (the last prompt row crosses nothing: head_dim 128 changes
+    form at 256 rows, so the first decode step is the first sliced one), 8 teacher-forced steps and one greedy
+    call of 8.  No reference model exists for this shape (oracle-extrapolated)."""
+    cfg = dict(synth.QWEN3_0P6B)
     gpu, ora = _stream_build(cfg, seed=4)
-    _prefill_decode_check(gpu, ora, cfg["vocab_size"], 256, 12, 1e-4, seed=4)
+    _prefill_decode_check(gpu, ora, cfg["vocab_size"], 256, 8, 1e-4, seed=4)
+    _greedy_call_checked(gpu, ora, 23, 8, 1e-4)
 
 
 @pytest.mark.slow
