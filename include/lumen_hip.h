@@ -163,6 +163,18 @@ int lumen_kv_cache_get_view(const lumen_kv_cache *cache, int current_len, float 
 int lumen_attn_decode_f32(lumen_kv_cache *cache, lumen_rope *rope, const float *q3_dev,
                           const float *k3_dev, const float *v3_dev, float *out_dev,
                           int h, float scale, int causal);
+/* The same decode step for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments,
+ * same results, bit for bit, as lumen_attn_decode_f32, but the scratch that the slices of a long cache need
+ * (per query head and slice a partial state of head_dim + 2 floats, plus one arrival counter per query head)
+ * comes from a fixed 4 MiB array inside the library's device image instead of a hipMalloc at the first call:
+ * this entry point calls no allocator.  batch x heads > 1024, or partial states beyond the array
+ * (batch x heads x slices x (head_dim + 2) x 4 bytes > 4 MiB - 4 KiB; slices = ceil(max_seq / (16384 / head_dim))
+ * rounded up to a power of two, 64 at most) -> LUMEN_ERR_UNSUPPORTED.  All calls on one GPU share that GPU's
+ * array: calls that overlap in time on one GPU (two contexts, two streams) race; calls in stream order do not. */
+int lumen_attn_decode_static_f32(lumen_kv_cache *cache, lumen_rope *rope, const float *q3_dev,
+                                 const float *k3_dev, const float *v3_dev, float *out_dev,
+                                 int h, float scale, int causal);
 /* SelfAttention::forward prefill core, S > 1, self_attention.rs:308-419 with
  * gqa_attention_no_repeat_bshd_view :519-641 and softmax_inplace_view :643-678:
  * q [B, S, H, D], k/v [B, S, H_kv, D] un-rotated; appends S positions to the

@@ -94,6 +94,7 @@ extern "C" {
     pub fn lumen_kv_cache_update(cache: *mut lumen_kv_cache, k_dev: *const c_float, v_dev: *const c_float, s: c_int, start_pos: c_int) -> c_int;
     pub fn lumen_kv_cache_get_view(cache: *const lumen_kv_cache, current_len: c_int, k_out_dev: *mut c_float, v_out_dev: *mut c_float) -> c_int;
     pub fn lumen_attn_decode_f32(cache: *mut lumen_kv_cache, rope: *mut lumen_rope, q3_dev: *const c_float, k3_dev: *const c_float, v3_dev: *const c_float, out_dev: *mut c_float, h: c_int, scale: c_float, causal: c_int) -> c_int;
+    pub fn lumen_attn_decode_static_f32(cache: *mut lumen_kv_cache, rope: *mut lumen_rope, q3_dev: *const c_float, k3_dev: *const c_float, v3_dev: *const c_float, out_dev: *mut c_float, h: c_int, scale: c_float, causal: c_int) -> c_int;
     pub fn lumen_attn_prefill_f32(cache: *mut lumen_kv_cache, rope: *mut lumen_rope, q_dev: *const c_float, k_dev: *const c_float, v_dev: *const c_float, out_dev: *mut c_float, s: c_int, h: c_int, scale: c_float, causal: c_int) -> c_int;
     pub fn lumen_llama_create(ctx: *mut lumen_ctx, cfg: *const lumen_llama_config, out: *mut *mut lumen_llama) -> c_int;
     pub fn lumen_llama_destroy(model: *mut lumen_llama) -> c_int;

@@ -85,6 +85,7 @@ SIGNATURES = {
     "lumen_kv_cache_update": (_i, [_vp, _vp, _vp, _i, _i]),
     "lumen_kv_cache_get_view": (_i, [_vp, _i, _vp, _vp]),
     "lumen_attn_decode_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _f, _i]),
+    "lumen_attn_decode_static_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _f, _i]),
     "lumen_attn_prefill_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _i]),
     "lumen_llama_create": (_i, [_vp, C.POINTER(LlamaConfigStruct), _pp]),
     "lumen_llama_destroy": (_i, [_vp]),

@@ -778,9 +778,24 @@ static int ensure_split_scratch(lumen_kv_cache *c, int hq, int nsplit) {
     return LUMEN_OK;
 }
 
-extern "C" int lumen_attn_decode_f32(lumen_kv_cache *c, lumen_rope *rope, const float *q3, const float *k3,
-                                     const float *v3, float *out, int h, float scale, int causal) {
-    (void)causal;  // the causal test `j > past_len` never fires for S == 1 (self_attention.rs:256)
+// The decode step of SelfAttention::forward behind both entry points: checks, launch, len += 1.
+static int attn_decode_entry(lumen_kv_cache *c, lumen_rope *rope, const float *q3, const float *k3, const float *v3,
+                             float *out, int h, float scale, float *part, int *counters, int nsplit) {
+    const int past_len = c->len, new_len = past_len + 1;
+    AttnDecodeArgs a = {};
+    a.q = q3; a.k_new = k3; a.v_new = v3; a.out = out;
+    a.k_cache = c->k; a.v_cache = c->v; a.cos_t = rope->cos_dev; a.sin_t = rope->sin_dev;
+    a.pos_dev = nullptr; a.pos_host = past_len;
+    a.b = c->b; a.hq = h; a.hkv = c->h_kv; a.d = c->d; a.max_seq = c->max_seq; a.scale = scale;
+    a.q_norm_w = nullptr; a.k_norm_w = nullptr; a.norm_eps = 0.f;
+    a.part = part; a.counters = counters; a.nsplit = nsplit;
+    LUMEN_TRY(launch_attn_decode(c->ctx, a));
+    c->len = new_len;
+    return LUMEN_OK;
+}
+
+static int check_attn_decode(const lumen_kv_cache *c, const lumen_rope *rope, const float *q3, const float *k3,
+                             const float *v3, const float *out, int h) {
     if (!c || !rope || !q3 || !k3 || !v3 || !out) LUMEN_FAIL(LUMEN_ERR_INVALID, "attn_decode: null argument");
     if (rope->dim != c->d) LUMEN_FAIL(LUMEN_ERR_SHAPE, "RoPE dimension mismatch: %d vs head_dim %d", rope->dim, c->d);
     if (h <= 0 || h % c->h_kv) LUMEN_FAIL(LUMEN_ERR_SHAPE, "attn_decode: %d heads over %d kv heads", h, c->h_kv);
@@ -789,18 +804,64 @@ extern "C" int lumen_attn_decode_f32(lumen_kv_cache *c, lumen_rope *rope, const 
         LUMEN_FAIL(LUMEN_ERR_KV_OVERFLOW, "KV cache overflow: new_len=%d > max_seq=%d", new_len, c->max_seq);
     if (past_len >= rope->max_seq)  // encoding.rs:176-181
         LUMEN_FAIL(LUMEN_ERR_ROPE_RANGE, "RoPE index out of range: pos %d >= max %d", past_len, rope->max_seq);
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_attn_decode_f32(lumen_kv_cache *c, lumen_rope *rope, const float *q3, const float *k3,
+                                     const float *v3, float *out, int h, float scale, int causal) {
+    (void)causal;  // the causal test `j > past_len` never fires for S == 1 (self_attention.rs:256)
+    LUMEN_TRY(check_attn_decode(c, rope, q3, k3, v3, out, h));
     const int nsplit = attn_decode_nsplit(c->max_seq, c->d);
     LUMEN_TRY(ensure_split_scratch(c, h, nsplit));
-    AttnDecodeArgs a = {};
-    a.q = q3; a.k_new = k3; a.v_new = v3; a.out = out;
-    a.k_cache = c->k; a.v_cache = c->v; a.cos_t = rope->cos_dev; a.sin_t = rope->sin_dev;
-    a.pos_dev = nullptr; a.pos_host = past_len;
-    a.b = c->b; a.hq = h; a.hkv = c->h_kv; a.d = c->d; a.max_seq = c->max_seq; a.scale = scale;
-    a.q_norm_w = nullptr; a.k_norm_w = nullptr; a.norm_eps = 0.f;
-    a.part = c->part; a.counters = c->counters; a.nsplit = nsplit;
-    LUMEN_TRY(launch_attn_decode(c->ctx, a));
-    c->len = new_len;
+    return attn_decode_entry(c, rope, q3, k3, v3, out, h, scale, c->part, c->counters, nsplit);
+}
+
+// ------------------------------------------------ decode attention that allocates nothing
+// The slices of a long cache hand their partial states (ctx[D], m, l per query head and slice) and one arrival
+// counter per query head from workgroup to workgroup through device memory.  lumen_attn_decode_f32 keeps that
+// scratch on the cache object and allocates it at the first call; this variant takes it from a fixed array in
+// the library's own device image instead, so it never calls an allocator.  Every GPU holds its own copy of the
+// array for the life of the process; host code reaches it only through the address hipGetSymbolAddress gives on
+// that GPU (the array's name in host code is a host-side stand-in, not a device address).
+#define ATTN_STATIC_COUNTERS 1024                    // query heads x batch at most
+#define ATTN_STATIC_BYTES ((size_t)4 << 20)          // counters (first 4 KiB) + partial states
+static __device__ __align__(256) unsigned char scratch[ATTN_STATIC_BYTES];
+
+// called by lumen_ctx_create with the context's device current
+int attn_static_scratch_init(lumen_ctx *ctx) {
+    void *p = nullptr;
+    HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p || ((uintptr_t)p & 255)) LUMEN_FAIL(LUMEN_ERR_HIP, "static attention scratch: bad device address %p", p);
+    ctx->attn_static = (unsigned char *)p;
+    ctx->attn_static_bytes = ATTN_STATIC_BYTES;
     return LUMEN_OK;
+}
+
+__global__ __launch_bounds__(256) void clear_ints_kernel(int *p, int n) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) p[i] = 0;
+}
+
+extern "C" int lumen_attn_decode_static_f32(lumen_kv_cache *c, lumen_rope *rope, const float *q3, const float *k3,
+                                            const float *v3, float *out, int h, float scale, int causal) {
+    (void)causal;
+    LUMEN_TRY(check_attn_decode(c, rope, q3, k3, v3, out, h));
+    lumen_ctx *ctx = c->ctx;
+    if (!ctx->attn_static) LUMEN_FAIL(LUMEN_ERR_HIP, "attn_decode_static: the context holds no static scratch address");
+    const int nsplit = attn_decode_nsplit(c->max_seq, c->d);
+    const size_t heads = (size_t)c->b * h;
+    const size_t need = sizeof(int) * ATTN_STATIC_COUNTERS + sizeof(float) * attn_decode_part_floats(c->b, h, c->d, nsplit);
+    if (heads > ATTN_STATIC_COUNTERS || need > ctx->attn_static_bytes)
+        LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED,
+                   "attn_decode_static: batch %d x %d heads x %d slices x head_dim %d needs %zu bytes of partial states; "
+                   "the static scratch holds %zu bytes and %d heads (use lumen_attn_decode_f32)",
+                   c->b, h, nsplit, c->d, need, ctx->attn_static_bytes, ATTN_STATIC_COUNTERS);
+    int *counters = (int *)ctx->attn_static;
+    float *part = (float *)(ctx->attn_static + sizeof(int) * ATTN_STATIC_COUNTERS);
+    // the array keeps what the last call left: the arrival counters must start at zero (a fill kernel, not a
+    // memset node, so that the call may sit inside a stream capture); partial states are written before they are read
+    hipLaunchKernelGGL(clear_ints_kernel, dim3(1), dim3(256), 0, ctx->stream, counters, (int)heads);
+    LUMEN_CHECK_LAUNCH();
+    return attn_decode_entry(c, rope, q3, k3, v3, out, h, scale, part, counters, nsplit);
 }
 
 extern "C" int lumen_attn_prefill_f32(lumen_kv_cache *c, lumen_rope *rope, const float *q, const float *k,

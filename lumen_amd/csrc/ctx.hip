@@ -38,6 +38,11 @@ extern "C" int lumen_ctx_create(int device, lumen_ctx **out) {
     HIP_TRY(hipEventCreate(&c->ev0));
     HIP_TRY(hipEventCreate(&c->ev1));
     HIP_TRY(hipMalloc((void **)&c->d_scratch_int, 64 * sizeof(int)));
+    const int src = attn_static_scratch_init(c);
+    if (src != LUMEN_OK) {
+        lumen_ctx_destroy(c);
+        return src;
+    }
     *out = c;
     return LUMEN_OK;
 }

@@ -46,7 +46,11 @@ struct lumen_ctx {
     int *d_scratch_int = nullptr;  // small device scratch (argmax result etc.)
     float *gemm_ws = nullptr;      // split-K workspace of the prefill GEMM, grown on demand
     size_t gemm_ws_bytes = 0;
+    // this device's address of the fixed scratch array behind lumen_attn_decode_static_f32
+    unsigned char *attn_static = nullptr;
+    size_t attn_static_bytes = 0;
 };
+int attn_static_scratch_init(lumen_ctx *ctx);
 
 struct lumen_rope {
     lumen_ctx *ctx = nullptr;
