@@ -139,10 +139,12 @@ def main():
             kernels[name] = {"avg_us": round(1e3 * (s_ms / n - event_overhead_ms), 3),
                              "launches_per_step": n // args.steps}
 
-    # decode attention: K and V rows of every KV head, read once per launch (mean cache length of the timed region)
-    at_ms, at_n = prof["attn_decode"]
+    # decode attention: K and V rows of every KV head, read once per launch (mean cache length of the timed
+    # region); with short caches attention and o_proj are one launch, which also streams W_o [H, H]
+    fused_attn = prof["attn_oproj_fused"][1] > 0
+    at_ms, at_n = prof["attn_oproj_fused"] if fused_attn else prof["attn_decode"]
     at_avg_ms = at_ms / max(at_n, 1) - event_overhead_ms
-    at_bytes = 2.0 * cfg["num_key_value_heads"] * mean_len * 64 * 4
+    at_bytes = 2.0 * cfg["num_key_value_heads"] * mean_len * 64 * 4 + (4.0 * H * H if fused_attn else 0.0)
     out = {
         "metric": "batch-1 decode tokens/s", "value": round(tok_s, 2), "unit": "tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
@@ -160,7 +162,8 @@ def main():
         "step_roofline": {"bytes_per_token": step_bytes, "achieved_GBps": round(step_bytes / (ms_per_step * 1e-3) / 1e9, 1),
                           "frac_of_8TBps": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                           "roofline_tokens_per_s": round(HBM_PEAK_GBS * 1e9 / step_bytes, 1)},
-        "attention": {"kernel": "attn_decode_kernel<64, 8, 8, true>", "kv_bytes_per_launch": at_bytes,
+        "attention": {"kernel": "attn_oproj_kernel<64, 4, 8, false> (decode attention + o_proj)" if fused_attn
+                      else "attn_decode_kernel<64, 8, 8, true>", "bytes_per_launch": at_bytes,
                       "avg_launch_us": round(at_avg_ms * 1e3, 3), "achieved_GBps": round(at_bytes / (at_avg_ms * 1e-3) / 1e9, 1),
                       "frac_of_8TBps": round(at_bytes / (at_avg_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
         "kernels": kernels,

@@ -257,7 +257,8 @@ int lumen_llama_get_config(const lumen_llama *model, lumen_llama_config *cfg_out
 /* measurement aid (no reference counterpart): n greedy steps launched kernel by
  * kernel, every launch bracketed by HIP events on the ctx stream.  Classes:
  * 0 embedding, 1 norm+q|k|v GEMV, 2 decode attention, 3 o_proj GEMV, 4 norm+gate|up
- * GEMV, 5 down GEMV, 6 norm+lm_head GEMV, 7 argmax.  ms_sum_out / count_out [n_classes >= 8]. */
+ * GEMV, 5 down GEMV, 6 norm+lm_head GEMV, 7 argmax, 8 decode attention + o_proj in one launch
+ * (short caches).  ms_sum_out / count_out [n_classes >= 9]. */
 int lumen_llama_decode_profile(lumen_llama *model, int first_id, int n, double *ms_sum_out,
                                int *count_out, int n_classes);
 /* how S == 1 steps are issued (no reference counterpart; the results are the same):
@@ -269,6 +270,16 @@ int lumen_llama_decode_profile(lumen_llama *model, int first_id, int n, double *
 #define LUMEN_DECODE_GRAPH 1
 #define LUMEN_DECODE_PERSISTENT 2
 int lumen_llama_set_decode_mode(lumen_llama *model, int mode);
+/* While the cache is short (up to 512 rows, 256 for head_dim 128) and the shape allows (no q/k norm, head_dim 64 or
+ * 128, n_head * head_dim a multiple of 512), decode attention and the o_proj product of a layer are ONE launch:
+ * attention workgroups hand their output to resident o_proj workgroups, whose weights are already in registers,
+ * through tagged 8-byte words (no reference counterpart; same results as the two launches it replaces).  This call
+ * switches that launch off or on (enable 0 / 1) and sets its waits: spin_limit = polls after which a waiting
+ * workgroup gives up -- the call that finds a wait given up returns LUMEN_ERR_HIP, its results are invalid, every
+ * wavefront still exits -- and the pauses, in units of 256 clocks, of the o_proj workgroups before their weight
+ * requests, before their first poll and between polls.  A negative argument leaves that setting as it is.
+ * enable = 1 on a shape the launch does not cover -> LUMEN_ERR_UNSUPPORTED. */
+int lumen_llama_set_handover(lumen_llama *model, int enable, int64_t spin_limit, int pre_sleep, int poll_delay, int poll_gap);
 int lumen_llama_get_decode_mode(const lumen_llama *model, int *mode_out);
 int lumen_llama_reset(lumen_llama *model);                      /* reset_kv_caches, llama.rs:172-176 */
 int lumen_llama_kv_len(const lumen_llama *model, int *len_out);

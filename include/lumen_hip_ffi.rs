@@ -109,6 +109,7 @@ extern "C" {
     pub fn lumen_llama_get_config(model: *const lumen_llama, cfg_out: *mut lumen_llama_config) -> c_int;
     pub fn lumen_llama_decode_profile(model: *mut lumen_llama, first_id: c_int, n: c_int, ms_sum_out: *mut f64, count_out: *mut c_int, n_classes: c_int) -> c_int;
     pub fn lumen_llama_set_decode_mode(model: *mut lumen_llama, mode: c_int) -> c_int;
+    pub fn lumen_llama_set_handover(model: *mut lumen_llama, enable: c_int, spin_limit: i64, pre_sleep: c_int, poll_delay: c_int, poll_gap: c_int) -> c_int;
     pub fn lumen_llama_get_decode_mode(model: *const lumen_llama, mode_out: *mut c_int) -> c_int;
     pub fn lumen_llama_reset(model: *mut lumen_llama) -> c_int;
     pub fn lumen_llama_kv_len(model: *const lumen_llama, len_out: *mut c_int) -> c_int;

@@ -101,6 +101,7 @@ SIGNATURES = {
     "lumen_llama_decode_greedy": (_i, [_vp, _i, _i, _vp, _vp]),
     "lumen_llama_decode_profile": (_i, [_vp, _i, _i, C.POINTER(C.c_double), C.POINTER(_i), _i]),
     "lumen_llama_set_decode_mode": (_i, [_vp, _i]),
+    "lumen_llama_set_handover": (_i, [_vp, _i, C.c_int64, _i, _i, _i]),
     "lumen_llama_get_decode_mode": (_i, [_vp, C.POINTER(_i)]),
     "lumen_llama_reset": (_i, [_vp]),
     "lumen_llama_kv_len": (_i, [_vp, C.POINTER(_i)]),

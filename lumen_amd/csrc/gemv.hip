@@ -11,6 +11,7 @@
 // lane and two pieces are kept in flight (16 loads per lane).
 #include "internal.h"
 #include "wave_reduce.h"
+#include "stage_times.h"
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
@@ -252,6 +253,7 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W
     const int K = K_hot, N = N_hot, D = D_hot;
     const int kpad = (K + PIECE - 1) / PIECE * PIECE;  // xs is zero from K to kpad
 
+    STAGE_T(0);
     const int lane = threadIdx.x & 63;
     const int gw = blockIdx.x * nwaves + (threadIdx.x >> 6);
     const int nw = nblocks * nwaves;
@@ -341,9 +343,11 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W
         }
     };
     preload(gw);
+    STAGE_T(1);
     if (PRO == PRO_ATTN_FOLD) stage_attn_fold(xs, a, K, kpad, nwaves);
     else if (EARLY) stage_x_early<PRO>(xs, xin, norm_w_hot, a.eps, K, kpad, nwaves, xe, ge);
     else stage_x<PRO, (XB > 0 ? XB : 1)>(xs, xin, norm_w_hot, a.eps, K, kpad, nwaves);
+    STAGE_T(2);
     float best = -INFINITY;
     int best_idx = 0x7fffffff;
 
@@ -420,6 +424,7 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W
     };
     for (int t = 0; t < T; t += 2) {
         consume(rawA);
+        if (t == 0) STAGE_T(3);
         if (t + 2 < T) {
             load_piece(lu, lk, rawA);
             advance_load();
@@ -433,6 +438,8 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W
         }
     }
 
+    STAGE_T(4);
+    STAGE_T_STORES_DONE(5);
     if (EPI == EPI_ARGMAX) {
         // greedy pick fused into the lm_head product: per-workgroup candidates go through memory with
         // agent-scope accesses, the last workgroup to arrive folds them (lowest index wins ties)
@@ -500,6 +507,7 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W
                 if (a.tok_hist) a.tok_hist[pos + 1] = bi;  // the pick is the token of the next position
                 *a.pos_inc = pos + 1;
             }
+            if (a.step_inc) *a.step_inc += 1;
         }
     }
 }
@@ -659,6 +667,11 @@ int launch_gemv(lumen_ctx *ctx, const GemvArgs &a) {
 #undef LAUNCH_GEMV
 #undef LAUNCH_GEMV_K
     LUMEN_CHECK_LAUNCH();
+    {
+        char what[96];
+        snprintf(what, sizeof what, "gemv N=%d K=%d pro=%d epi=%d threads=%d", a.N, a.K, a.pro, a.epi, threads);
+        stage_times_report(ctx, what, blocks, "start, requests out, x staged, first piece done, rows done, stores acknowledged");
+    }
     return LUMEN_OK;
 }
 

@@ -102,6 +102,7 @@ struct GemvArgs {
     int *amax_counter; // zero between launches
     int *tok_out, *pos_inc;
     int *tok_hist;     // optional [max_seq + 1]: the pick is also stored at index *pos_inc + 1
+    unsigned *step_inc;  // optional: decode step counter, incremented together with *pos_inc
     // EPI_ROPE_QKV: rows are q|k|v heads of D; a unit is the RoPE pair (j, j + D/2) of one head.
     // q is rotated into y, k rotated and v as is go to row *pos of the KV cache.
     const float *cos_t, *sin_t;
@@ -169,8 +170,33 @@ struct AttnDecodeArgs {
     // (ctx[D], m, l) in `part` -- the short form in slice 0 -- and `out` is not written.  The o_proj GEMV
     // folds the partials while it stages its input (PRO_ATTN_FOLD).  Needs pre_rotated and one-trip slices.
     int defer_merge;
+    // the output goes out as tagged 8-byte words {value, tag} instead of plain floats (the short form inside the
+    // attention -> o_proj chain, attn_oproj.hip); null everywhere else
+    unsigned long long *out_tagged;
+    unsigned tag;
 };
 int launch_attn_decode(lumen_ctx *ctx, const AttnDecodeArgs &a);
+
+// Decode attention and the o_proj product chained inside ONE launch (attn_oproj.hip): the first hq workgroups
+// are the short-form attention (one query head each), the others the o_proj rows; the attention output travels
+// between them as tagged words.  q rotated, cache row *pos_dev written already.
+struct AttnOprojArgs {
+    AttnDecodeArgs attn;          // q, caches, pos_dev, scale, hq, hkv, d, max_seq (b = 1, pre_rotated)
+    const void *Wo;               // [N, K] f32 or bf16 bits, K = hq * d
+    const float *residual;        // [N]: y = residual + Wo attn (src/models/llama.rs:110)
+    float *y;                     // [N]
+    int N, K, w_bf16;
+    const int *row_sel;           // the residual is row *row_sel of a [rows, row_stride] table (first layer), or null
+    long row_stride;
+    unsigned long long *x_tagged; // [K] attention output on its way to the o_proj workgroups, zero at start
+    const unsigned *step_dev;     // decode step counter of the model: the tag is *step_dev * tag_mul + tag_add
+    unsigned tag_mul, tag_add;
+    int *err_dev;                 // set to 1 when a wait ran into spin_limit
+    unsigned spin_limit;          // polls before a waiting workgroup gives up
+    int pre_sleep, poll_delay, poll_gap;  // timing of the o_proj workgroups (units of 256 clocks), see attn_oproj.hip
+};
+bool attn_oproj_supported(int hq, int hkv, int d, int N, int K, int w_bf16);
+int launch_attn_oproj(lumen_ctx *ctx, const AttnOprojArgs &a);
 
 struct AttnPrefillArgs {
     const float *q;  // [B, S, Hq, D] un-rotated

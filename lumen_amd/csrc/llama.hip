@@ -44,6 +44,14 @@ struct lumen_llama {
     int *counters = nullptr;
     int nsplit = 1;     // slices of a long cache in the decode attention kernel
     bool defer_merge = false;  // the o_proj GEMV, not the attention kernel, may merge the slices of a long cache
+    // short caches: attention and o_proj chained in one launch (attn_oproj.hip); its hand-over buffer, the decode
+    // step counter its tags are made of, the flag a timed-out wait leaves, and the poll limit of a wait
+    bool chain_ao = false;
+    unsigned long long *x_tagged = nullptr;
+    unsigned *d_step = nullptr;
+    int *d_err = nullptr;
+    unsigned spin_limit = 1u << 22;
+    int chain_pre = 10, chain_delay = 16, chain_gap = 1;  // timing of the chain's o_proj workgroups (units of 256 clocks)
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
     int graph_expect_short = 0;            // the hint the captured attention launches carry
@@ -184,6 +192,17 @@ extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg,
                      cfg->max_seq_len <= m->nsplit * attn_decode_trip_rows(D) && fold_bytes <= ((size_t)64 << 20);
     M_TRY(dmalloc_t(m, &m->part, attn_decode_part_floats(1, Hq, D, m->nsplit)));
     M_TRY(dmalloc_t(m, &m->counters, (size_t)Hq));
+    // (q/k-norm models rotate inside the attention kernel: the chain wants a rotated q and a written cache row)
+    m->chain_ao = !cfg->qk_norm && attn_oproj_supported(Hq, Hkv, D, H, m->qd, m->bf16);
+    M_TRY(dmalloc_t(m, &m->x_tagged, (size_t)m->qd));
+    M_TRY(dmalloc_t(m, &m->d_step, 4));
+    M_TRY(dmalloc_t(m, &m->d_err, 4));
+    if (hipMemsetAsync(m->x_tagged, 0, sizeof(unsigned long long) * m->qd, ctx->stream) != hipSuccess ||
+        hipMemsetAsync(m->d_step, 0, 4 * sizeof(unsigned), ctx->stream) != hipSuccess ||
+        hipMemsetAsync(m->d_err, 0, 4 * sizeof(int), ctx->stream) != hipSuccess) {
+        lumen_llama_destroy(m);
+        LUMEN_FAIL(LUMEN_ERR_HIP, "llama_create: clearing the hand-over state failed");
+    }
     if (hipMemsetAsync(m->counters, 0, sizeof(int) * Hq, ctx->stream) != hipSuccess ||
         hipMemsetAsync(m->d_tok, 0, 4 * sizeof(int), ctx->stream) != hipSuccess ||
         hipMemsetAsync(m->d_pos, 0, 4 * sizeof(int), ctx->stream) != hipSuccess ||
@@ -378,7 +397,7 @@ int lumen_llama_param_list(const lumen_llama *m, std::vector<std::string> &names
 // One token through all layers; every launch reads the token id and the
 // position from device memory, so the sequence is the same for every token.
 // Kernel classes of a decode step, for per-kernel timing.
-enum { KC_EMBED = 0, KC_QKV, KC_ATTN, KC_OPROJ, KC_GATEUP, KC_DOWN, KC_LMHEAD, KC_ARGMAX, KC_COUNT };
+enum { KC_EMBED = 0, KC_QKV, KC_ATTN, KC_OPROJ, KC_GATEUP, KC_DOWN, KC_LMHEAD, KC_ARGMAX, KC_ATTN_OPROJ, KC_COUNT };
 
 struct StepProbe {  // brackets every launch with a HIP event pair when profiling
     std::vector<hipEvent_t> ev;
@@ -436,24 +455,41 @@ static int enqueue_decode_step(lumen_llama *m, StepProbe *pr = nullptr) {
         a.scale = m->scale; a.q_norm_w = w.q_norm; a.k_norm_w = w.k_norm; a.norm_eps = c.rms_norm_eps;
         a.part = m->part; a.counters = m->counters; a.nsplit = m->nsplit; a.pre_rotated = fuse_rope;
         a.expect_short = expect_short_cache(m);
-        // (a graph is captured anew when the hint changes sides, so the choice is the same for every launch of a step)
-        const bool defer = m->defer_merge && !a.expect_short;
-        a.defer_merge = defer;
-        pr->before(KC_ATTN);
-        LUMEN_TRY(launch_attn_decode(ctx, a));
-        pr->after();
-        // o_proj + residual, self_attention.rs:303, llama.rs:110
-        g = {};
-        g.W = w.wo; g.x = m->attn; g.y = m->h; g.N = H; g.K = m->qd; g.w_bf16 = m->bf16;
-        g.pro = PRO_NONE; g.epi = EPI_RESIDUAL; g.residual = m->x;
-        if (defer) {
-            g.pro = PRO_ATTN_FOLD; g.attn_part = m->part; g.attn_pos = m->d_pos; g.attn_nslices = m->nsplit; g.attn_d = m->D;
-            g.attn_trip = attn_decode_trip_rows(m->D); g.attn_short_rows = attn_decode_short_rows(m->D);
+        // (a graph is captured anew when the cache crosses the short / long boundary, so the choices below are the
+        // same for every launch of a step)
+        if (m->chain_ao && a.expect_short) {
+            // short caches: attention and o_proj + residual chained in one launch
+            AttnOprojArgs f = {};
+            f.attn = a;
+            f.attn.out_tagged = m->x_tagged;
+            f.Wo = w.wo; f.residual = m->x; f.y = m->h; f.N = H; f.K = m->qd; f.w_bf16 = m->bf16;
+            if (l == 0) { f.residual = m->embed; f.row_sel = m->d_tok; f.row_stride = H; }
+            f.x_tagged = m->x_tagged; f.step_dev = m->d_step;
+            f.tag_mul = (unsigned)c.num_hidden_layers; f.tag_add = (unsigned)l + 1u;
+            f.err_dev = m->d_err; f.spin_limit = m->spin_limit;
+            f.pre_sleep = m->chain_pre; f.poll_delay = m->chain_delay; f.poll_gap = m->chain_gap;
+            pr->before(KC_ATTN_OPROJ);
+            LUMEN_TRY(launch_attn_oproj(ctx, f));
+            pr->after();
+        } else {
+            const bool defer = m->defer_merge && !a.expect_short;
+            a.defer_merge = defer;
+            pr->before(KC_ATTN);
+            LUMEN_TRY(launch_attn_decode(ctx, a));
+            pr->after();
+            // o_proj + residual, self_attention.rs:303, llama.rs:110
+            g = {};
+            g.W = w.wo; g.x = m->attn; g.y = m->h; g.N = H; g.K = m->qd; g.w_bf16 = m->bf16;
+            g.pro = PRO_NONE; g.epi = EPI_RESIDUAL; g.residual = m->x;
+            if (defer) {
+                g.pro = PRO_ATTN_FOLD; g.attn_part = m->part; g.attn_pos = m->d_pos; g.attn_nslices = m->nsplit; g.attn_d = m->D;
+                g.attn_trip = attn_decode_trip_rows(m->D); g.attn_short_rows = attn_decode_short_rows(m->D);
+            }
+            if (l == 0) { g.residual = m->embed; g.row_sel = m->d_tok; g.row_stride = H; g.residual_sel = 1; }
+            pr->before(KC_OPROJ);
+            LUMEN_TRY(launch_gemv(ctx, g));
+            pr->after();
         }
-        if (l == 0) { g.residual = m->embed; g.row_sel = m->d_tok; g.row_stride = H; g.residual_sel = 1; }
-        pr->before(KC_OPROJ);
-        LUMEN_TRY(launch_gemv(ctx, g));
-        pr->after();
         // post_attention_layernorm + gate|up + silu*up, llama.rs:113, :60-63
         g = {};
         g.W = w.wgu; g.x = m->h; g.y = m->act; g.N = 2 * I; g.K = H; g.w_bf16 = m->bf16;
@@ -476,7 +512,7 @@ static int enqueue_decode_step(lumen_llama *m, StepProbe *pr = nullptr) {
     g.pro = PRO_RMSNORM; g.norm_w = m->final_norm; g.eps = c.rms_norm_eps;
     // the greedy pick is folded in: it becomes the next token id and the position counter advances
     g.epi = EPI_ARGMAX; g.amax_val = m->amax_val; g.amax_idx = m->amax_idx; g.amax_counter = m->amax_counter;
-    g.tok_out = m->d_tok; g.pos_inc = m->d_pos; g.tok_hist = m->tok_hist;
+    g.tok_out = m->d_tok; g.pos_inc = m->d_pos; g.tok_hist = m->tok_hist; g.step_inc = m->d_step;
     pr->before(KC_LMHEAD);
     const int rc = launch_gemv(ctx, g);
     pr->after();
@@ -529,10 +565,42 @@ extern "C" int lumen_llama_set_decode_mode(lumen_llama *m, int mode) {
     return LUMEN_OK;
 }
 
+extern "C" int lumen_llama_set_handover(lumen_llama *m, int enable, int64_t spin_limit, int pre_sleep, int poll_delay, int poll_gap) {
+    if (!m) LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_set_handover: null model");
+    if (enable > 0 && (m->cfg.qk_norm || !attn_oproj_supported(m->cfg.num_attention_heads, m->cfg.num_key_value_heads, m->D,
+                                                               m->cfg.hidden_size, m->qd, m->bf16)))
+        LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "the attention -> o_proj launch does not cover this model shape");
+    if (enable >= 0) m->chain_ao = enable > 0;
+    if (spin_limit >= 0) m->spin_limit = spin_limit > 0xffffffffLL ? 0xffffffffu : (unsigned)spin_limit;
+    if (pre_sleep >= 0) m->chain_pre = pre_sleep;
+    if (poll_delay >= 0) m->chain_delay = poll_delay;
+    if (poll_gap >= 0) m->chain_gap = poll_gap;
+    // the captured step carries the old choice
+    if (m->graph_exec) {
+        HIP_TRY(hipStreamSynchronize(m->ctx->stream));
+        hipGraphExecDestroy(m->graph_exec);
+        hipGraphDestroy(m->graph);
+        m->graph_exec = nullptr;
+        m->graph = nullptr;
+    }
+    return LUMEN_OK;
+}
+
 extern "C" int lumen_llama_get_decode_mode(const lumen_llama *m, int *mode_out) {
     if (!m || !mode_out) LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_get_decode_mode: null argument");
     *mode_out = m->decode_mode;
     return LUMEN_OK;
+}
+
+// after a synchronisation: did a wait inside the attention -> o_proj chain run into its limit?
+static int check_handover(lumen_llama *m) {
+    if (!m->chain_ao) return LUMEN_OK;
+    int err = 0;
+    HIP_TRY(hipMemcpy(&err, m->d_err, sizeof(int), hipMemcpyDeviceToHost));
+    if (!err) return LUMEN_OK;
+    HIP_TRY(hipMemset(m->d_err, 0, sizeof(int)));
+    LUMEN_FAIL(LUMEN_ERR_HIP, "decode: a workgroup gave up waiting for the attention output inside the attention -> o_proj "
+                              "launch (poll limit %u); the results of this call are invalid, reset the model", m->spin_limit);
 }
 
 static int sync_pos_to_device(lumen_llama *m) {
@@ -662,7 +730,10 @@ extern "C" int lumen_llama_forward(lumen_llama *m, const float *ids_host, int s,
     HIP_TRY(hipStreamSynchronize(st));
     HIP_TRY(launch_step(m));
     m->len += 1;
-    if (logits_host) return lumen_download(m->ctx, logits_host, m->logits, sizeof(float) * (size_t)m->cfg.vocab_size);
+    if (logits_host) {
+        LUMEN_TRY(lumen_download(m->ctx, logits_host, m->logits, sizeof(float) * (size_t)m->cfg.vocab_size));
+        return check_handover(m);
+    }
     return LUMEN_OK;
 }
 
@@ -683,6 +754,9 @@ extern "C" int lumen_llama_decode_greedy(lumen_llama *m, int first_id, int n, in
     const int len0 = m->len;
     int rc = LUMEN_OK;
     for (int t = 0; t < n && rc == LUMEN_OK; ++t) {
+        // (the graph is captured anew at the step where the cache crosses the short / long attention boundary)
+        rc = ensure_decode_graph(m);
+        if (rc != LUMEN_OK) break;
         hipError_t e = launch_step(m);
         if (e == hipSuccess && logits_out)
             e = hipMemcpyAsync(logits_out + (size_t)t * V, m->logits, sizeof(float) * V, hipMemcpyDeviceToHost, st);
@@ -697,6 +771,7 @@ extern "C" int lumen_llama_decode_greedy(lumen_llama *m, int first_id, int n, in
     if (rc == LUMEN_OK && e == hipSuccess && ids_out)
         e = hipMemcpy(ids_out, m->tok_hist + len0 + 1, sizeof(int) * (size_t)n, hipMemcpyDeviceToHost);
     if (rc == LUMEN_OK && e != hipSuccess) LUMEN_FAIL(LUMEN_ERR_HIP, "decode_greedy: %s", hipGetErrorString(e));
+    if (rc == LUMEN_OK) rc = check_handover(m);
     return rc;
 }
 

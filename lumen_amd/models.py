@@ -155,6 +155,12 @@ class LlamaModel:
         (the library holds no such kernel)."""
         check(lib.lumen_llama_set_decode_mode(self.handle, self.DECODE_MODES[mode]))
 
+    def set_handover(self, enable=-1, spin_limit=-1, pre_sleep=-1, poll_delay=-1, poll_gap=-1):
+        """The attention -> o_proj launch of short caches: off / on, and the limits and pauses of its waits
+        (negative: unchanged)."""
+        check(lib.lumen_llama_set_handover(self.handle, int(enable), int(spin_limit), int(pre_sleep), int(poll_delay),
+                                           int(poll_gap)))
+
     @property
     def decode_mode(self):
         v = C.c_int()
@@ -162,7 +168,7 @@ class LlamaModel:
         return {n: k for k, n in self.DECODE_MODES.items()}[v.value]
 
     KERNEL_CLASSES = ("embedding", "norm_qkv_gemv", "attn_decode", "oproj_gemv", "norm_gateup_gemv", "down_gemv",
-                      "norm_lmhead_gemv", "argmax")
+                      "norm_lmhead_gemv", "argmax", "attn_oproj_fused")
 
     def decode_profile(self, first_id, n):
         """n greedy steps with every launch bracketed by HIP events: {class: (ms_sum, launches)}."""

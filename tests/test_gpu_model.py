@@ -314,6 +314,64 @@ def test_one_greedy_call_replays_a_graph_across_the_attention_boundary(cfg_extra
         assert max_rel(lg, le) <= 1e-5
 
 
+CHAIN = dict(vocab_size=1200, hidden_size=512, intermediate_size=1408, num_hidden_layers=3, num_attention_heads=8,
+             num_key_value_heads=2, rms_norm_eps=1e-5, max_seq_len=700, rope_theta=10000.0)  # head_dim 64, n_rep 4
+
+
+@pytest.mark.parametrize("cfg_extra,bf16", [(dict(), False), (dict(num_key_value_heads=8), False),
+                                            (dict(hidden_size=1024, num_attention_heads=8, num_key_value_heads=4,
+                                                  intermediate_size=1024), False),
+                                            (dict(hidden_size=1024, num_attention_heads=16, num_key_value_heads=2,
+                                                  intermediate_size=1024), True)],
+                         ids=["d64-nrep4", "d64-mha", "d128-nrep2", "d64-nrep8-bf16"])
+def test_attention_oproj_launch_equals_the_two_launches_it_replaces(cfg_extra, bf16):
+    """Short caches: decode attention and o_proj run as one launch whose attention workgroups hand their output to
+    the o_proj workgroups through tagged words.  Same steps with that launch switched off (two launches): the
+    attention arithmetic is the same code, so logits agree to rounding of the o_proj sums; both are held to the
+    checker; the cache crosses a trip boundary (256 rows, 128 for head_dim 128) on the way."""
+    cfg = dict(CHAIN)
+    cfg.update(cfg_extra)
+    tol = 2e-2 if bf16 else 1e-4
+    gpu, ora, _ = build(cfg, seed=51, bf16=bf16)
+    n_prompt, n = 120, 150
+    ids = synth.make_tokens(n_prompt, cfg["vocab_size"], seed=51)
+    out = {}
+    for enable in (1, 0):
+        gpu.set_handover(enable=enable)
+        gpu.reset_kv_caches()
+        ora.reset()
+        last = gpu.forward(ids, all_rows=False)
+        _, ref = ora.forward(ids)
+        assert max_rel(last, ref[-1]) <= tol
+        out[enable] = _greedy_call_checked(gpu, ora, lo.argmax(ref[-1]), n, tol)
+        assert gpu.kv_len == n_prompt + n
+    (p1, l1), (p0, l0) = out[1], out[0]
+    if np.array_equal(p1, p0):
+        assert max_rel(l1, l0) <= 2e-6
+
+
+def test_attention_oproj_launch_gives_up_a_wait_that_cannot_end_in_time_and_says_so():
+    """Failure handling of the hand-over inside the attention -> o_proj launch, forced from the host: with a poll
+    limit of zero and no pauses the o_proj workgroups look once, before the attention can have finished, give up and
+    flag it; every wavefront exits, the call returns LUMEN_ERR_HIP, and after the defaults are back the model works."""
+    gpu, ora, _ = build(CHAIN, seed=52)
+    ids = synth.make_tokens(40, CHAIN["vocab_size"], seed=52)
+    last = gpu.forward(ids, all_rows=False)
+    gpu.set_handover(spin_limit=0, pre_sleep=0, poll_delay=0, poll_gap=0)
+    with pytest.raises(_lib.LumenError) as e:
+        gpu.decode_greedy(int(np.argmax(last)), 3)
+    assert e.value.status == _lib.ERR_HIP and "gave up waiting" in str(e.value)
+    gpu.set_handover(spin_limit=1 << 22, pre_sleep=10, poll_delay=16, poll_gap=1)
+    gpu.reset_kv_caches()
+    last = gpu.forward(ids, all_rows=False)
+    _, ref = ora.forward(ids)
+    assert max_rel(last, ref[-1]) <= 1e-4
+    _greedy_call_checked(gpu, ora, lo.argmax(ref[-1]), 12, 1e-4)
+    with pytest.raises(_lib.LumenError) as e:  # a q/k-norm model rotates inside the attention kernel: not covered
+        build(TINY_QWEN, seed=1)[0].set_handover(enable=1)
+    assert e.value.status == _lib.ERR_UNSUPPORTED
+
+
 @pytest.mark.parametrize("qk_norm", [False, True], ids=["merge-in-oproj", "merge-in-kernel"])
 def test_sliced_attention_decode_is_bit_reproducible(qk_norm):
     """The same 64 greedy steps at ~4000 cached rows (16 slices per head, partial states handed from
