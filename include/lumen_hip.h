@@ -273,12 +273,16 @@ int lumen_llama_set_decode_mode(lumen_llama *model, int mode);
 /* While the cache is short (up to 512 rows, 256 for head_dim 128) and the shape allows (no q/k norm, head_dim 64 or
  * 128, n_head * head_dim a multiple of 512), decode attention and the o_proj product of a layer are ONE launch:
  * attention workgroups hand their output to resident o_proj workgroups, whose weights are already in registers,
- * through tagged 8-byte words (no reference counterpart; same results as the two launches it replaces).  This call
- * switches that launch off or on (enable 0 / 1) and sets its waits: spin_limit = polls after which a waiting
+ * through tagged 8-byte words (no reference counterpart; same results as the two launches it replaces).  Where
+ * n_head * head_dim == hidden_size and two weight rows fit a wavefront's registers (hidden 512, 1024 or 2048 in f32, twice
+ * that in bf16) the RMSNorm + q|k|v + RoPE product joins the same launch in front, handing q and the new key /
+ * value to the attention workgroups the same way.  This call picks the form (enable 0: separate launches,
+ * 1: attention + o_proj, 2: q|k|v + attention + o_proj, the default where covered) and sets its waits: spin_limit = polls after which a waiting
  * workgroup gives up -- the call that finds a wait given up returns LUMEN_ERR_HIP, its results are invalid, every
  * wavefront still exits -- and the pauses, in units of 256 clocks, of the o_proj workgroups before their weight
- * requests, before their first poll and between polls.  A negative argument leaves that setting as it is.
- * enable = 1 on a shape the launch does not cover -> LUMEN_ERR_UNSUPPORTED. */
+ * requests, before their first poll and between polls (kept per form; the call sets those of the form in use
+ * after it).  A negative argument leaves that setting as it is.
+ * enable = 1 or 2 on a shape that form does not cover -> LUMEN_ERR_UNSUPPORTED. */
 int lumen_llama_set_handover(lumen_llama *model, int enable, int64_t spin_limit, int pre_sleep, int poll_delay, int poll_gap);
 int lumen_llama_get_decode_mode(const lumen_llama *model, int *mode_out);
 int lumen_llama_reset(lumen_llama *model);                      /* reset_kv_caches, llama.rs:172-176 */

@@ -302,7 +302,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
 #pragma unroll 1
     for (int attempt = 0; attempt < 2; ++attempt) {
         if (want_short) {
-            if (r < NREP && attn_decode_short<D, WAVES, PRE>(a, r, NREP, hk, bb, pos_new, SHORT_ROWS, q_rot, k_new, v_new, sm, sl, sacc))
+            if (r < NREP && attn_decode_short<D, WAVES, PRE ? ATTN_SRC_CACHE : ATTN_SRC_RAW>(a, r, NREP, hk, bb, pos_new, SHORT_ROWS, q_rot, k_new, v_new, sm, sl, sacc))
                 return;
             if (pos_new < 0) pos_new = *a.pos_dev;
             if (pos_new + 1 <= SHORT_ROWS) return;  // short indeed: not one of the short form's workgroups

@@ -26,7 +26,19 @@
 // that the attention's own few requests enter the memory system first; poll_delay before the first poll and poll_gap
 // between polls, because every poll of the 131072 threads is a trip to memory that the weights compete with.
 //
-// q arrives rotated and cache row `pos` is already written (both by the q|k|v product's epilogue).
+// q arrives rotated and cache row `pos` is already written (both by the q|k|v product's epilogue) -- or, QKV form,
+// that product is a third role in FRONT of the two:
+//
+//   [0, nq)       RMSNorm of the layer input + q|k|v product + RoPE, one rotation pair of rows (j, j + D/2) per
+//                 wavefront with all weights in registers (src/models/llama.rs:107, self_attention.rs:106-108,
+//                 :220-227); the rotated q, the new key and the new value leave as tagged words, key and value also
+//                 go to cache row `pos` (self_attention.rs:161-176) for the steps to come;
+//
+// the attention workgroups request their first trip of cached rows, THEN wait for their head's q and the group's
+// new row, and take that row from LDS instead of the cache.  The layer input is read by the first and (as the
+// residual) the last role; it was written by an earlier launch.  In this form the o_proj workgroups hold their
+// weight requests back (pre_sleep) until q and the new row have changed hands: every trip to memory of a hand-over
+// queues behind whatever was requested before it, and 17 MB of weights in the queue cost each trip ~2 us.
 #include "internal.h"
 #include "attn_device.h"
 #include "attn_short_device.h"
@@ -61,43 +73,18 @@ __device__ __forceinline__ float ao_dot16(const v4u raw, const float *xs) {
     return s;
 }
 
-__device__ __forceinline__ void ao_sleep(int n) {
-    for (int i = 0; i < n; ++i) __builtin_amdgcn_s_sleep(4);  // 256 clocks each
-}
-
-// This thread's EPT words of a tagged vector, polled until every one carries `tag`; false after `limit` polls.
-template <int EPT>
-__device__ __forceinline__ bool take_tagged(const unsigned long long *xp, unsigned tag, unsigned limit, int gap, float (&v)[EPT]) {
-    unsigned long long w[EPT];
-    unsigned spins = 0;
-    bool ok;
-    do {
-        ok = true;
-#pragma unroll
-        for (int e = 0; e < EPT; ++e) {
-            w[e] = tagged_load(xp + e);
-            ok = ok && (unsigned)(w[e] >> 32) == tag;
-        }
-        if (!ok) {
-            if (++spins > limit) break;  // never in a healthy launch: give up so that the wavefront exits
-            ao_sleep(gap);
-        }
-    } while (!ok);
-#pragma unroll
-    for (int e = 0; e < EPT; ++e) v[e] = __uint_as_float((unsigned)w[e]);
-    return ok;
-}
-
 // D: head_dim; NLO: 16-byte weight loads per lane and row of the o_proj product (its row length is NLO * 64 *
-// elements per load).
-template <int D, int NLO, bool BF16>
+// elements per load); QKV: with the q|k|v role in front (its rows have the same length: hidden == hq * D).
+template <int D, int NLO, bool BF16, bool QKV>
 __global__ __launch_bounds__(AO_THREADS) void attn_oproj_kernel(const void *Wo_hot, float *k_cache_hot, float *v_cache_hot,
                                                                 const float *q_hot, const int *pos_dev_hot,
                                                                 const unsigned *step_dev_hot, int max_seq_hot, int hq_hot,
-                                                                int hkv_hot, int N_hot, AttnOprojArgs a_mem) {
+                                                                int hkv_hot, int N_hot, const void *Wqkv_hot,
+                                                                const float *x_hot, const float *in_norm_hot,
+                                                                AttnOprojArgs a_mem) {
     constexpr int VEC = BF16 ? 8 : 4;
     constexpr int ESZ = BF16 ? 2 : 4;
-    constexpr int K = NLO * 64 * VEC;  // o_proj row length = hq * D
+    constexpr int K = NLO * 64 * VEC;  // o_proj row length = hq * D (QKV: also the q|k|v row length)
     constexpr int EPT = K / AO_THREADS;
     static_assert(K % AO_THREADS == 0 && EPT >= 1, "K must be a multiple of the workgroup size");
     __shared__ __align__(16) float q_rot[D];
@@ -110,8 +97,98 @@ __global__ __launch_bounds__(AO_THREADS) void attn_oproj_kernel(const void *Wo_h
     const int hq = hq_hot, hkv = hkv_hot, N = N_hot;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n_o = (N + AO_WAVES - 1) / AO_WAVES;  // o_proj workgroups
-    if ((int)blockIdx.x < hq) {
-        // ---- attention of one query head.  Workgroups are dealt round-robin over the 8 XCDs: XCD x takes the hq / 8
+    constexpr int HALF = D / 2;
+    const int nunits = QKV ? (hq + 2 * hkv) * HALF : 0;  // rotation pairs; a multiple of 8: D / 2 is
+    const int nq = nunits / AO_WAVES;                    // q|k|v workgroups
+    int blk = blockIdx.x;
+    if (QKV && blk < nq) {
+        // ---- RMSNorm + q|k|v + RoPE: one pair of rows (j, j + D/2) of one head per wavefront
+        constexpr int XP = (K / 4 + AO_THREADS - 1) / AO_THREADS;  // 16-byte pieces of x a thread stages
+        const int unit = blk * AO_WAVES + wave;
+        const int head = unit / HALF, j = unit % HALF;
+        const float *x = x_hot;
+        if (a_mem.row_sel) x += (long)(*a_mem.row_sel) * a_mem.row_stride;  // (first layer: a trip of its own)
+        // x and the gains first: what is requested first arrives first, and the norm is what the multiplies wait for
+        v4f xe[XP], ge[XP];
+#pragma unroll
+        for (int i = 0; i < XP; ++i) {
+            const int k = (tid + i * AO_THREADS) * 4;
+            xe[i] = v4f{0.f, 0.f, 0.f, 0.f};
+            ge[i] = xe[i];
+            if (k < K) {
+                xe[i] = *(const v4f *)(x + k);
+                ge[i] = *(const v4f *)(in_norm_hot + k);
+            }
+        }
+        v4u raw[2][NLO];
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            const char *rp = (const char *)Wqkv_hot + ((size_t)(head * D + j + r * HALF) * K + (size_t)lane * VEC) * ESZ;
+#pragma unroll
+            for (int i = 0; i < NLO; ++i) raw[r][i] = __builtin_nontemporal_load((const v4u *)(rp + (size_t)i * 64 * VEC * ESZ));
+        }
+        const int pos = *pos_dev_hot;
+        const unsigned tag = *step_dev_hot * a_mem.tag_mul + a_mem.tag_add;
+        const float cs = a_mem.attn.cos_t[(size_t)pos * D + j], sn = a_mem.attn.sin_t[(size_t)pos * D + j];
+        STAGE_T(1);
+        // (x * inv_rms) * g, src/layers/norm/rms_norm.rs:45-58
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < XP; ++i) ss += xe[i].x * xe[i].x + xe[i].y * xe[i].y + xe[i].z * xe[i].z + xe[i].w * xe[i].w;
+        ss = wave_sum(ss);
+        if (lane == 0) sm[wave] = ss;
+        __syncthreads();
+        float tot = 0.f;
+#pragma unroll
+        for (int w = 0; w < AO_WAVES; ++w) tot += sm[w];
+        const float inv = 1.0f / sqrtf(tot / (float)K + a_mem.norm_eps);
+#pragma unroll
+        for (int i = 0; i < XP; ++i) {
+            const int k = (tid + i * AO_THREADS) * 4;
+            if (k < K) {
+                v4f v = xe[i];
+                v.x = v.x * inv * ge[i].x;
+                v.y = v.y * inv * ge[i].y;
+                v.z = v.z * inv * ge[i].z;
+                v.w = v.w * inv * ge[i].w;
+                *(v4f *)(xs + k) = v;
+            }
+        }
+        __syncthreads();
+        STAGE_T(2);
+        float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < NLO; ++i) {
+            acc0 += ao_dot16<BF16>(raw[0][i], xs + (i * 64 + lane) * VEC);
+            acc1 += ao_dot16<BF16>(raw[1][i], xs + (i * 64 + lane) * VEC);
+        }
+        acc0 = wave_sum(acc0);
+        acc1 = wave_sum(acc1);
+        if (lane == 0) {
+            // half-split rotation at the token's position (src/layers/attention/encoding.rs:196-203)
+            float o1 = acc0, o2 = acc1;
+            if (head < hq + hkv) {
+#pragma clang fp contract(off)
+                o1 = acc0 * cs - acc1 * sn;
+                o2 = acc0 * sn + acc1 * cs;
+            }
+            unsigned long long *t = a_mem.qkv_tagged + (size_t)head * D + j;
+            tagged_store(t, o1, tag);
+            tagged_store(t + HALF, o2, tag);
+            if (head >= hq) {  // key / value of the new token: cache row pos
+                float *cache = head < hq + hkv ? k_cache_hot : v_cache_hot;
+                const int hk = head < hq + hkv ? head - hq : head - hq - hkv;
+                float *dst = cache + ((size_t)hk * max_seq_hot + pos) * D;
+                dst[j] = o1;
+                dst[j + HALF] = o2;
+            }
+        }
+        STAGE_T_STORES_DONE(3);
+        return;
+    }
+    blk -= nq;
+    if (blk < hq) {
+        // ---- attention of one query head.  Workgroup i of the grid runs on XCD i % 8: XCD x takes the hq / 8
         // consecutive heads x * hq / 8 ..., so that a KV group's rows are fetched into as few L2s as possible.
         AttnDecodeArgs a = a_mem.attn;
         a.k_cache = k_cache_hot;
@@ -122,18 +199,23 @@ __global__ __launch_bounds__(AO_THREADS) void attn_oproj_kernel(const void *Wo_h
         a.hq = hq;
         a.hkv = hkv;
         a.tag = *step_dev_hot * a_mem.tag_mul + a_mem.tag_add;
-        const int b = blockIdx.x;
-        const int h = (hq % 8 == 0) ? (b % 8) * (hq / 8) + b / 8 : b;
+        a.qkv_tagged = a_mem.qkv_tagged;
+        a.spin_limit = a_mem.spin_limit;
+        a.poll_gap = a_mem.poll_gap;
+        a.err_dev = a_mem.err_dev;
+        const int xcd = (blk + nq) & 7;
+        const int h = (hq % 8 == 0) ? xcd * (hq / 8) + (blk >> 3) : blk;
         const int nrep = hq / hkv;
         // (a cache of any length: the short form walks it trip by trip)
-        attn_decode_short<D, AO_WAVES, true>(a, h % nrep, nrep, h / nrep, 0, -1, 0x7fffffff, q_rot, k_new, v_new, sm, sl, sacc);
+        attn_decode_short<D, AO_WAVES, QKV ? ATTN_SRC_TAGGED : ATTN_SRC_CACHE>(a, h % nrep, nrep, h / nrep, 0, -1, 0x7fffffff, q_rot,
+                                                                               k_new, v_new, sm, sl, sacc);
         return;
     }
-    if ((int)blockIdx.x < hq + n_o) {
+    blk -= hq;
+    if (blk < n_o) {
         // ---- o_proj: one row per wavefront, all of its weights requested at once (rows past N: clamped, not stored)
-        const int wg = (int)blockIdx.x - hq;
-        const int row = wg * AO_WAVES + wave;
-        ao_sleep(a_mem.pre_sleep);  // (the attention's requests go first)
+        const int row = blk * AO_WAVES + wave;
+        handover_pause(a_mem.pre_sleep);  // (see the head of the file)
         v4u raw[NLO];
         {
             const char *rp = (const char *)Wo_hot + ((size_t)min(row, N - 1) * K + (size_t)lane * VEC) * ESZ;
@@ -146,7 +228,7 @@ __global__ __launch_bounds__(AO_THREADS) void attn_oproj_kernel(const void *Wo_h
         const float res = residual[min(row, N - 1)];
         STAGE_T(5);
         // the attention output: this thread's EPT words, polled until every one carries this launch's tag
-        ao_sleep(a_mem.poll_delay);
+        handover_pause(a_mem.poll_delay);
         {
             float v[EPT];
             if (!take_tagged<EPT>(a_mem.x_tagged + (size_t)tid * EPT, tag, a_mem.spin_limit, a_mem.poll_gap, v))
@@ -181,28 +263,44 @@ bool attn_oproj_supported(int hq, int hkv, int d, int N, int K, int w_bf16) {
     return nl == 2 || nl == 4 || nl == 8 || nl == 16;
 }
 
+// the q|k|v role in front: its rows are as long as o_proj's, and two of them fit a wavefront's registers
+bool qkv_attn_oproj_supported(int hq, int hkv, int d, int N, int K, int w_bf16) {
+    if (!attn_oproj_supported(hq, hkv, d, N, K, w_bf16) || N != K) return false;
+    const int nl = ao_nl(K, w_bf16);
+    return nl == 2 || nl == 4 || nl == 8;
+}
+
 int attn_oproj_workgroups(int N) { return (N + AO_WAVES - 1) / AO_WAVES; }
 
 template <int D, bool BF16>
 static int launch_ao(lumen_ctx *ctx, const AttnOprojArgs &a) {
     const int nlo = ao_nl(a.K, BF16);
-    const int n_wg = a.attn.hq + attn_oproj_workgroups(a.N);
+    const int nq = a.Wqkv ? (a.attn.hq + 2 * a.attn.hkv) * (D / 2) / AO_WAVES : 0;
+    const int n_wg = nq + a.attn.hq + attn_oproj_workgroups(a.N);
     dim3 grid(n_wg), block(AO_THREADS);
-#define AO_LAUNCH(NLO)                                                                                                 \
-    hipLaunchKernelGGL((attn_oproj_kernel<D, NLO, BF16>), grid, block, 0, ctx->stream, a.Wo, a.attn.k_cache, a.attn.v_cache, \
-                       a.attn.q, a.attn.pos_dev, a.step_dev, a.attn.max_seq, a.attn.hq, a.attn.hkv, a.N, a)
-    switch (nlo) {
-        case 2: AO_LAUNCH(2); break;
-        case 4: AO_LAUNCH(4); break;
-        case 8: AO_LAUNCH(8); break;
-        default: AO_LAUNCH(16); break;
+#define AO_LAUNCH(NLO, QKV)                                                                                                      \
+    hipLaunchKernelGGL((attn_oproj_kernel<D, NLO, BF16, QKV>), grid, block, 0, ctx->stream, a.Wo, a.attn.k_cache, a.attn.v_cache, \
+                       a.attn.q, a.attn.pos_dev, a.step_dev, a.attn.max_seq, a.attn.hq, a.attn.hkv, a.N, a.Wqkv, a.residual,     \
+                       a.in_norm_w, a)
+    if (a.Wqkv) {
+        if (nlo == 2) AO_LAUNCH(2, true);
+        else if (nlo == 4) AO_LAUNCH(4, true);
+        else AO_LAUNCH(8, true);
+    } else {
+        switch (nlo) {
+            case 2: AO_LAUNCH(2, false); break;
+            case 4: AO_LAUNCH(4, false); break;
+            case 8: AO_LAUNCH(8, false); break;
+            default: AO_LAUNCH(16, false); break;
+        }
     }
 #undef AO_LAUNCH
     LUMEN_CHECK_LAUNCH();
-    const int seg[2] = {a.attn.hq, n_wg};
-    stage_times_report(ctx, "attention | o_proj chain", n_wg,
-                       "start, (attention: rows done, merged, stored, acknowledged), o_proj: polls begin, input staged, acknowledged",
-                       seg, 2);
+    const int seg[3] = {nq, nq + a.attn.hq, n_wg};
+    stage_times_report(ctx, "(q|k|v |) attention | o_proj chain", n_wg,
+                       "start, then q|k|v: [1] requests out, [2] x staged, [3] acknowledged; attention: [1] rows done, "
+                       "[2] merged, [3] stored, [4] acknowledged; o_proj: [5] polls begin, [6] input staged, [7] acknowledged",
+                       seg + (nq ? 0 : 1), nq ? 3 : 2);
     return LUMEN_OK;
 }
 
@@ -210,8 +308,19 @@ int launch_attn_oproj(lumen_ctx *ctx, const AttnOprojArgs &a) {
     if (!attn_oproj_supported(a.attn.hq, a.attn.hkv, a.attn.d, a.N, a.K, a.w_bf16))
         LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "attention -> o_proj chain: %d/%d heads of %d, W_o [%d, %d] not covered", a.attn.hq,
                    a.attn.hkv, a.attn.d, a.N, a.K);
-    if (!a.attn.pos_dev || !a.attn.pre_rotated || a.attn.b != 1 || !a.x_tagged || !a.step_dev || !a.err_dev || !a.attn.out_tagged)
-        LUMEN_FAIL(LUMEN_ERR_INVALID, "attention -> o_proj chain: needs a rotated q, a device position, batch 1 and a hand-over buffer");
+    if (!a.attn.pos_dev || a.attn.b != 1 || !a.x_tagged || !a.step_dev || !a.err_dev || !a.attn.out_tagged)
+        LUMEN_FAIL(LUMEN_ERR_INVALID, "attention -> o_proj chain: needs a device position, batch 1 and a hand-over buffer");
+    if (a.Wqkv) {
+        if (!qkv_attn_oproj_supported(a.attn.hq, a.attn.hkv, a.attn.d, a.N, a.K, a.w_bf16))
+            LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "q|k|v -> attention -> o_proj chain: hidden %d, %d heads of %d not covered", a.N,
+                       a.attn.hq, a.attn.d);
+        if (!a.in_norm_w || !a.qkv_tagged || !a.attn.cos_t || !a.attn.sin_t || !a.residual)
+            LUMEN_FAIL(LUMEN_ERR_INVALID, "q|k|v -> attention -> o_proj chain: needs norm gains, RoPE tables and a hand-over buffer");
+        if ((((uintptr_t)a.Wqkv | (uintptr_t)a.residual | (uintptr_t)a.in_norm_w) & 15) != 0 || (a.row_sel && a.row_stride % 4))
+            LUMEN_FAIL(LUMEN_ERR_INVALID, "q|k|v -> attention -> o_proj chain: operands must be 16-byte aligned");
+    } else if (!a.attn.pre_rotated) {
+        LUMEN_FAIL(LUMEN_ERR_INVALID, "attention -> o_proj chain: needs a rotated q and the new cache row in place");
+    }
     if ((((uintptr_t)a.Wo | (uintptr_t)a.attn.q | (uintptr_t)a.attn.k_cache | (uintptr_t)a.attn.v_cache) & 15) != 0)
         LUMEN_FAIL(LUMEN_ERR_INVALID, "attention -> o_proj chain: operands must be 16-byte aligned");
     if ((size_t)a.attn.max_seq * a.attn.d * sizeof(float) >= ((size_t)1 << 32))

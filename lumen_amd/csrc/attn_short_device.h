@@ -18,6 +18,33 @@ __device__ __forceinline__ unsigned long long tagged_load(const unsigned long lo
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+__device__ __forceinline__ void handover_pause(int n) {
+    for (int i = 0; i < n; ++i) __builtin_amdgcn_s_sleep(4);  // 256 clocks each
+}
+
+// This thread's EPT words of a tagged vector, polled until every one carries `tag`; false after `limit` polls.
+template <int EPT>
+__device__ __forceinline__ bool take_tagged(const unsigned long long *xp, unsigned tag, unsigned limit, int gap, float (&v)[EPT]) {
+    unsigned long long w[EPT];
+    unsigned spins = 0;
+    bool ok;
+    do {
+        ok = true;
+#pragma unroll
+        for (int e = 0; e < EPT; ++e) {
+            w[e] = tagged_load(xp + e);
+            ok = ok && (unsigned)(w[e] >> 32) == tag;
+        }
+        if (!ok) {
+            if (++spins > limit) break;  // never in a healthy launch: give up so that the wavefront exits
+            handover_pause(gap);
+        }
+    } while (!ok);
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) v[e] = __uint_as_float((unsigned)w[e]);
+    return ok;
+}
+
 // Short contexts (up to ATTN_SHORT_ROWS cached rows; 256 for head_dim 128): one query head per
 // workgroup over ALL rows, 8 row loads per lane in flight, so that nothing has to travel between
 // workgroups -- at these lengths the hand-over of partial results through memory (an atomic and
@@ -46,20 +73,29 @@ __device__ __forceinline__ unsigned rows_mask(int first, int stride, int end) {
     return m;
 }
 
-// PRE: q is rotated and cache row pos_new written already; otherwise this workgroup normalises and
-// rotates its own query head and the group's new key itself (a few hundred flops, repeated by
-// every head of the group so that nothing has to be exchanged), the first head of the group
-// stores the new row, and every head takes that row from LDS (q_rot, k_new, v_new: D floats each).
+// Where q and the new row come from (SRC):
+//   ATTN_SRC_RAW     un-rotated projections in memory: this workgroup normalises and rotates its own query head and
+//                    the group's new key itself (a few hundred flops, repeated by every head of the group so that
+//                    nothing has to be exchanged), the first head of the group stores the new row, and every head
+//                    takes that row from LDS (q_rot, k_new, v_new: D floats each);
+//   ATTN_SRC_CACHE   q is rotated and cache row pos_new written already (an earlier launch did both);
+//   ATTN_SRC_TAGGED  rotated q, new key and new value arrive as tagged words from other workgroups of THIS launch
+//                    (which also store the row): they are polled for after the first trip of rows is requested, go to
+//                    LDS, and the new row is taken from there.
 //
 // pos_new < 0: the position is not known yet.  The first trip of rows and the query are requested
 // before it is read -- they do not depend on it: a row past the cached ones is only masked later --
 // so the position's own trip to memory is off the critical path.  Returns false, having done
 // nothing, when the position then turns out to lie past short_rows.
-template <int D, int WAVES, bool PRE>
+#define ATTN_SRC_RAW 0
+#define ATTN_SRC_CACHE 1
+#define ATTN_SRC_TAGGED 2
+template <int D, int WAVES, int SRC>
 __device__ __forceinline__ bool attn_decode_short(const AttnDecodeArgs &a, int r, int nrep, int hk, int bb, int pos_new,
                                                   int short_rows, float *q_rot, float *k_new,
                                                   float *v_new, float *sm, float *sl, float *sacc) {
     constexpr int LPR = D / 4, RPW = 64 / LPR, RPI = WAVES * RPW, UB = ShortTrip<D>::loads, THREADS = WAVES * 64;
+    constexpr bool PRE = SRC == ATTN_SRC_CACHE;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int off = wave * RPW + lane / LPR, c = lane % LPR;
     const int hq = hk * nrep + r;
@@ -86,9 +122,24 @@ __device__ __forceinline__ bool attn_decode_short(const AttnDecodeArgs &a, int r
     if (pos_new < 0) pos_new = a.pos_dev ? *a.pos_dev : a.pos_host;
     if (pos_new + 1 > short_rows) return false;
     const int pos = PRE ? pos_new + 1 : pos_new;  // rows read from the cache
-    auto get_q = [&]() {
+    auto get_q = [&]() __attribute__((always_inline)) {
         if (PRE) {
             load_q_scaled<D, 1>(q, a.q + ((size_t)bb * a.hq + hq) * D, c, a.scale);
+        } else if constexpr (SRC == ATTN_SRC_TAGGED) {
+            // wavefronts 0, 1, 2 wait for the query head, the new key and the new value (batch 1)
+            constexpr int EPL = D >= 64 ? D / 64 : 1;  // (the chain takes head_dim 64 and 128 only)
+            auto take = [&](float *dst, int vec) __attribute__((always_inline)) {
+                float v[EPL];
+                if (!take_tagged<EPL>(a.qkv_tagged + (size_t)vec * D + lane * EPL, a.tag, a.spin_limit, a.poll_gap, v))
+                    __hip_atomic_store(a.err_dev, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) dst[lane * EPL + e] = v[e];
+            };
+            if (wave == 0) take(q_rot, hq);
+            else if (wave == 1) take(k_new, a.hq + hk);
+            else if (wave == 2) take(v_new, a.hq + a.hkv + hk);
+            __syncthreads();
+            load_q_scaled<D, 1>(q, q_rot, c, a.scale);
         } else {
             // wavefront 0 takes the query head, wavefront 1 the new key, wavefront 2 copies the new value:
             // lane j holds the pair (j, j + D/2); everything they need from memory is requested at once

@@ -174,6 +174,12 @@ struct AttnDecodeArgs {
     // attention -> o_proj chain, attn_oproj.hip); null everywhere else
     unsigned long long *out_tagged;
     unsigned tag;
+    // q, the new key and the new value ARRIVE as tagged words, [hq + 2 hkv, D] rotated (the q|k|v -> attention ->
+    // o_proj chain): the cache row of the new token is not read, nothing is rotated or stored here; null everywhere else
+    const unsigned long long *qkv_tagged;
+    unsigned spin_limit;  // polls before a wait for tagged words gives up (then *err_dev = 1)
+    int poll_gap;         // pause between polls, units of 256 clocks
+    int *err_dev;
 };
 int launch_attn_decode(lumen_ctx *ctx, const AttnDecodeArgs &a);
 
@@ -194,8 +200,16 @@ struct AttnOprojArgs {
     int *err_dev;                 // set to 1 when a wait ran into spin_limit
     unsigned spin_limit;          // polls before a waiting workgroup gives up
     int pre_sleep, poll_delay, poll_gap;  // timing of the o_proj workgroups (units of 256 clocks), see attn_oproj.hip
+    // With Wqkv set the launch starts one step earlier: its first workgroups are RMSNorm + the q|k|v product + RoPE
+    // + KV append (src/models/llama.rs:107, self_attention.rs:106-108, :161-176, :220-227) on `residual` (the layer
+    // input), and q / new key / new value travel to the attention workgroups as tagged words.  Needs N == K.
+    const void *Wqkv;             // [(hq + 2 hkv) * d, N] f32 or bf16 bits, or null
+    const float *in_norm_w;       // [N] gains of the input RMSNorm
+    float norm_eps;
+    unsigned long long *qkv_tagged;  // [(hq + 2 hkv) * d]
 };
 bool attn_oproj_supported(int hq, int hkv, int d, int N, int K, int w_bf16);
+bool qkv_attn_oproj_supported(int hq, int hkv, int d, int N, int K, int w_bf16);
 int launch_attn_oproj(lumen_ctx *ctx, const AttnOprojArgs &a);
 
 struct AttnPrefillArgs {

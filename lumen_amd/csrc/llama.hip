@@ -46,12 +46,14 @@ struct lumen_llama {
     bool defer_merge = false;  // the o_proj GEMV, not the attention kernel, may merge the slices of a long cache
     // short caches: attention and o_proj chained in one launch (attn_oproj.hip); its hand-over buffer, the decode
     // step counter its tags are made of, the flag a timed-out wait leaves, and the poll limit of a wait
-    bool chain_ao = false;
-    unsigned long long *x_tagged = nullptr;
+    int chain_ao = 0;  // 0: off, 1: attention -> o_proj, 2: q|k|v -> attention -> o_proj
+    unsigned long long *x_tagged = nullptr, *qkv_tagged = nullptr;
     unsigned *d_step = nullptr;
     int *d_err = nullptr;
     unsigned spin_limit = 1u << 22;
-    int chain_pre = 10, chain_delay = 16, chain_gap = 1;  // timing of the chain's o_proj workgroups (units of 256 clocks)
+    // timing of the chain's o_proj workgroups (units of 256 clocks), per form: pause before the weight requests,
+    // before the first poll, between polls (measured optima on the 2048-wide model; see attn_oproj.hip)
+    int chain_pre[3] = {0, 10, 47}, chain_delay[3] = {0, 16, 13}, chain_gap[3] = {0, 1, 1};
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
     int graph_expect_short = 0;            // the hint the captured attention launches carry
@@ -193,11 +195,15 @@ extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg,
     M_TRY(dmalloc_t(m, &m->part, attn_decode_part_floats(1, Hq, D, m->nsplit)));
     M_TRY(dmalloc_t(m, &m->counters, (size_t)Hq));
     // (q/k-norm models rotate inside the attention kernel: the chain wants a rotated q and a written cache row)
-    m->chain_ao = !cfg->qk_norm && attn_oproj_supported(Hq, Hkv, D, H, m->qd, m->bf16);
+    m->chain_ao = (cfg->qk_norm || !attn_oproj_supported(Hq, Hkv, D, H, m->qd, m->bf16)) ? 0
+                  : qkv_attn_oproj_supported(Hq, Hkv, D, H, m->qd, m->bf16)              ? 2
+                                                                                         : 1;
     M_TRY(dmalloc_t(m, &m->x_tagged, (size_t)m->qd));
+    M_TRY(dmalloc_t(m, &m->qkv_tagged, (size_t)m->qkvd));
     M_TRY(dmalloc_t(m, &m->d_step, 4));
     M_TRY(dmalloc_t(m, &m->d_err, 4));
     if (hipMemsetAsync(m->x_tagged, 0, sizeof(unsigned long long) * m->qd, ctx->stream) != hipSuccess ||
+        hipMemsetAsync(m->qkv_tagged, 0, sizeof(unsigned long long) * m->qkvd, ctx->stream) != hipSuccess ||
         hipMemsetAsync(m->d_step, 0, 4 * sizeof(unsigned), ctx->stream) != hipSuccess ||
         hipMemsetAsync(m->d_err, 0, 4 * sizeof(int), ctx->stream) != hipSuccess) {
         lumen_llama_destroy(m);
@@ -444,9 +450,13 @@ static int enqueue_decode_step(lumen_llama *m, StepProbe *pr = nullptr) {
             g.k_cache = m->k_slab + m->cache_stride * l; g.v_cache = m->v_slab + m->cache_stride * l;
             g.hq = c.num_attention_heads; g.hkv = c.num_key_value_heads; g.D = m->D; g.max_seq = c.max_seq_len;
         }
-        pr->before(KC_QKV);
-        LUMEN_TRY(launch_gemv(ctx, g));
-        pr->after();
+        const bool chain_short = m->chain_ao && expect_short_cache(m);
+        const bool chain_qkv = chain_short && m->chain_ao > 1;
+        if (!chain_qkv) {
+            pr->before(KC_QKV);
+            LUMEN_TRY(launch_gemv(ctx, g));
+            pr->after();
+        }
         AttnDecodeArgs a = {};
         a.q = m->qkv; a.k_new = m->qkv + m->qd; a.v_new = m->qkv + m->qd + m->kvd; a.out = m->attn;
         a.k_cache = m->k_slab + m->cache_stride * l; a.v_cache = m->v_slab + m->cache_stride * l;
@@ -457,8 +467,8 @@ static int enqueue_decode_step(lumen_llama *m, StepProbe *pr = nullptr) {
         a.expect_short = expect_short_cache(m);
         // (a graph is captured anew when the cache crosses the short / long boundary, so the choices below are the
         // same for every launch of a step)
-        if (m->chain_ao && a.expect_short) {
-            // short caches: attention and o_proj + residual chained in one launch
+        if (chain_short) {
+            // short caches: (q|k|v,) attention and o_proj + residual chained in one launch
             AttnOprojArgs f = {};
             f.attn = a;
             f.attn.out_tagged = m->x_tagged;
@@ -467,7 +477,10 @@ static int enqueue_decode_step(lumen_llama *m, StepProbe *pr = nullptr) {
             f.x_tagged = m->x_tagged; f.step_dev = m->d_step;
             f.tag_mul = (unsigned)c.num_hidden_layers; f.tag_add = (unsigned)l + 1u;
             f.err_dev = m->d_err; f.spin_limit = m->spin_limit;
-            f.pre_sleep = m->chain_pre; f.poll_delay = m->chain_delay; f.poll_gap = m->chain_gap;
+            f.pre_sleep = m->chain_pre[m->chain_ao]; f.poll_delay = m->chain_delay[m->chain_ao]; f.poll_gap = m->chain_gap[m->chain_ao];
+            if (chain_qkv) {
+                f.Wqkv = w.wqkv; f.in_norm_w = w.in_norm; f.norm_eps = c.rms_norm_eps; f.qkv_tagged = m->qkv_tagged;
+            }
             pr->before(KC_ATTN_OPROJ);
             LUMEN_TRY(launch_attn_oproj(ctx, f));
             pr->after();
@@ -570,11 +583,14 @@ extern "C" int lumen_llama_set_handover(lumen_llama *m, int enable, int64_t spin
     if (enable > 0 && (m->cfg.qk_norm || !attn_oproj_supported(m->cfg.num_attention_heads, m->cfg.num_key_value_heads, m->D,
                                                                m->cfg.hidden_size, m->qd, m->bf16)))
         LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "the attention -> o_proj launch does not cover this model shape");
-    if (enable >= 0) m->chain_ao = enable > 0;
+    if (enable > 1 && !qkv_attn_oproj_supported(m->cfg.num_attention_heads, m->cfg.num_key_value_heads, m->D, m->cfg.hidden_size,
+                                                m->qd, m->bf16))
+        LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "the q|k|v -> attention -> o_proj launch does not cover this model shape");
+    if (enable >= 0) m->chain_ao = enable > 2 ? 2 : enable;
     if (spin_limit >= 0) m->spin_limit = spin_limit > 0xffffffffLL ? 0xffffffffu : (unsigned)spin_limit;
-    if (pre_sleep >= 0) m->chain_pre = pre_sleep;
-    if (poll_delay >= 0) m->chain_delay = poll_delay;
-    if (poll_gap >= 0) m->chain_gap = poll_gap;
+    if (pre_sleep >= 0) m->chain_pre[m->chain_ao] = pre_sleep;
+    if (poll_delay >= 0) m->chain_delay[m->chain_ao] = poll_delay;
+    if (poll_gap >= 0) m->chain_gap[m->chain_ao] = poll_gap;
     // the captured step carries the old choice
     if (m->graph_exec) {
         HIP_TRY(hipStreamSynchronize(m->ctx->stream));

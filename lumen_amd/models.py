@@ -156,8 +156,8 @@ class LlamaModel:
         check(lib.lumen_llama_set_decode_mode(self.handle, self.DECODE_MODES[mode]))
 
     def set_handover(self, enable=-1, spin_limit=-1, pre_sleep=-1, poll_delay=-1, poll_gap=-1):
-        """The attention -> o_proj launch of short caches: off / on, and the limits and pauses of its waits
-        (negative: unchanged)."""
+        """The chained launch of short caches: 0 separate launches, 1 attention -> o_proj, 2 q|k|v -> attention ->
+        o_proj; and the limits and pauses of its waits (negative: unchanged)."""
         check(lib.lumen_llama_set_handover(self.handle, int(enable), int(spin_limit), int(pre_sleep), int(poll_delay),
                                            int(poll_gap)))
 

@@ -322,13 +322,19 @@ CHAIN = dict(vocab_size=1200, hidden_size=512, intermediate_size=1408, num_hidde
                                             (dict(hidden_size=1024, num_attention_heads=8, num_key_value_heads=4,
                                                   intermediate_size=1024), False),
                                             (dict(hidden_size=1024, num_attention_heads=16, num_key_value_heads=2,
-                                                  intermediate_size=1024), True)],
-                         ids=["d64-nrep4", "d64-mha", "d128-nrep2", "d64-nrep8-bf16"])
-def test_attention_oproj_launch_equals_the_two_launches_it_replaces(cfg_extra, bf16):
+                                                  intermediate_size=1024), True),
+                                            (dict(hidden_size=2048, num_attention_heads=16, num_key_value_heads=4,
+                                                  intermediate_size=512, num_hidden_layers=2), False),
+                                            (dict(hidden_size=2048, num_attention_heads=32, num_key_value_heads=4,
+                                                  intermediate_size=512, num_hidden_layers=2), True)],
+                         ids=["d64-nrep4", "d64-mha", "d128-nrep2", "d64-nrep8-bf16", "d128-nrep4-h2048",
+                              "d64-nrep8-h2048-bf16"])
+def test_chained_launches_equal_the_separate_launches_they_replace(cfg_extra, bf16):
     """Short caches: decode attention and o_proj run as one launch whose attention workgroups hand their output to
-    the o_proj workgroups through tagged words.  Same steps with that launch switched off (two launches): the
-    attention arithmetic is the same code, so logits agree to rounding of the o_proj sums; both are held to the
-    checker; the cache crosses a trip boundary (256 rows, 128 for head_dim 128) on the way."""
+    the o_proj workgroups through tagged words (form 1), with the RMSNorm + q|k|v + RoPE product in front handing q
+    and the new row to the attention workgroups the same way (form 2).  Same steps with separate launches (form 0): the attention arithmetic is the same code, so
+    logits agree to rounding of the sums; every form is held to the checker; the cache crosses a trip boundary
+    (256 rows, 128 for head_dim 128) on the way."""
     cfg = dict(CHAIN)
     cfg.update(cfg_extra)
     tol = 2e-2 if bf16 else 1e-4
@@ -336,7 +342,7 @@ def test_attention_oproj_launch_equals_the_two_launches_it_replaces(cfg_extra, b
     n_prompt, n = 120, 150
     ids = synth.make_tokens(n_prompt, cfg["vocab_size"], seed=51)
     out = {}
-    for enable in (1, 0):
+    for enable in (2, 1, 0):
         gpu.set_handover(enable=enable)
         gpu.reset_kv_caches()
         ora.reset()
@@ -345,23 +351,27 @@ def test_attention_oproj_launch_equals_the_two_launches_it_replaces(cfg_extra, b
         assert max_rel(last, ref[-1]) <= tol
         out[enable] = _greedy_call_checked(gpu, ora, lo.argmax(ref[-1]), n, tol)
         assert gpu.kv_len == n_prompt + n
-    (p1, l1), (p0, l0) = out[1], out[0]
-    if np.array_equal(p1, p0):
-        assert max_rel(l1, l0) <= 2e-6
+    p0, l0 = out[0]
+    for enable in (1, 2):
+        if enable in out and np.array_equal(out[enable][0], p0):
+            assert max_rel(out[enable][1], l0) <= (2e-6 if enable == 1 else 2e-5)
 
 
 def test_attention_oproj_launch_gives_up_a_wait_that_cannot_end_in_time_and_says_so():
-    """Failure handling of the hand-over inside the attention -> o_proj launch, forced from the host: with a poll
-    limit of zero and no pauses the o_proj workgroups look once, before the attention can have finished, give up and
-    flag it; every wavefront exits, the call returns LUMEN_ERR_HIP, and after the defaults are back the model works."""
+    """Failure handling of the hand-over inside the chained launches, forced from the host: with a poll limit of
+    zero and no pauses the waiting workgroups look once, before their producers can have finished, give up and flag
+    it; every wavefront exits, the call returns LUMEN_ERR_HIP, and after the defaults are back the model works."""
     gpu, ora, _ = build(CHAIN, seed=52)
     ids = synth.make_tokens(40, CHAIN["vocab_size"], seed=52)
-    last = gpu.forward(ids, all_rows=False)
-    gpu.set_handover(spin_limit=0, pre_sleep=0, poll_delay=0, poll_gap=0)
-    with pytest.raises(_lib.LumenError) as e:
-        gpu.decode_greedy(int(np.argmax(last)), 3)
-    assert e.value.status == _lib.ERR_HIP and "gave up waiting" in str(e.value)
-    gpu.set_handover(spin_limit=1 << 22, pre_sleep=10, poll_delay=16, poll_gap=1)
+    for enable in (1, 2):
+        gpu.reset_kv_caches()
+        last = gpu.forward(ids, all_rows=False)
+        gpu.set_handover(enable=enable, spin_limit=0, pre_sleep=0, poll_delay=0, poll_gap=0)
+        with pytest.raises(_lib.LumenError) as e:
+            gpu.decode_greedy(int(np.argmax(last)), 3)
+        assert e.value.status == _lib.ERR_HIP and "gave up waiting" in str(e.value)
+    gpu.set_handover(enable=1, spin_limit=1 << 22, pre_sleep=10, poll_delay=16, poll_gap=1)
+    gpu.set_handover(enable=2, pre_sleep=47, poll_delay=13, poll_gap=1)
     gpu.reset_kv_caches()
     last = gpu.forward(ids, all_rows=False)
     _, ref = ora.forward(ids)
@@ -369,6 +379,11 @@ def test_attention_oproj_launch_gives_up_a_wait_that_cannot_end_in_time_and_says
     _greedy_call_checked(gpu, ora, lo.argmax(ref[-1]), 12, 1e-4)
     with pytest.raises(_lib.LumenError) as e:  # a q/k-norm model rotates inside the attention kernel: not covered
         build(TINY_QWEN, seed=1)[0].set_handover(enable=1)
+    assert e.value.status == _lib.ERR_UNSUPPORTED
+    wide = build(dict(CHAIN, head_dim=128, num_hidden_layers=1), seed=2)[0]  # n_head * head_dim = 2 * hidden
+    wide.set_handover(enable=1)
+    with pytest.raises(_lib.LumenError) as e:  # the q|k|v role shares the row length of o_proj
+        wide.set_handover(enable=2)
     assert e.value.status == _lib.ERR_UNSUPPORTED
 
 
