@@ -64,7 +64,7 @@ def main():
 
     import numpy as np
 
-    from lumen_amd import synth
+    from lumen_amd import _lib, synth
     from lumen_amd.models import LlamaModel
 
     cfg = dict(synth.TINYLLAMA_1B, max_seq_len=args.max_seq)
@@ -141,32 +141,49 @@ def main():
 
     # decode attention: K and V rows of every KV head, read once per launch (mean cache length of the timed
     # region); with short caches attention and o_proj are one launch, which also streams W_o [H, H]
+    # Kernel instances: the names the launchers recorded during that profile pass.  The dominant one must be what the
+    # library's own dispatch reports for [2I, H] (lumen_gemv_kernel_name reads the decision launch_gemv takes), and
+    # the committed counter figures are only quoted when they were taken on that same instance.
+    names = {k: model.profile_kernel_name(k) for k in prof if prof[k][1]}
+    gu_kernel = names["norm_gateup_gemv"]
+    picked = _lib.gemv_kernel_name(ctx.num_cus, 2 * I, H, cfg.get("weight_dtype", "f32") == "bf16", True, _lib.GEMV_EPI_SWIGLU)
+    if gu_kernel != picked:
+        raise SystemExit("bench: gate|up launched %r but the dispatch reports %r" % (gu_kernel, picked))
+    hq, hkv = cfg["num_attention_heads"], cfg["num_key_value_heads"]
+    D = cfg.get("head_dim") or H // hq
     fused_attn = prof["attn_oproj_fused"][1] > 0
     at_ms, at_n = prof["attn_oproj_fused"] if fused_attn else prof["attn_decode"]
     at_avg_ms = at_ms / max(at_n, 1) - event_overhead_ms
-    at_bytes = 2.0 * cfg["num_key_value_heads"] * mean_len * 64 * 4 + (4.0 * H * H if fused_attn else 0.0)
+    at_kernel = names["attn_oproj_fused" if fused_attn else "attn_decode"]
+    at_bytes = 2.0 * hkv * mean_len * D * 4  # K and V rows
+    at_what = "decode attention"
+    if fused_attn:
+        at_bytes += 4.0 * H * hq * D  # + W_o
+        at_what = "decode attention + o_proj"
+        if prof["norm_qkv_gemv"][1] == 0:  # + W_qkv: the q|k|v product is part of the same launch
+            at_bytes += 4.0 * (hq + 2 * hkv) * D * H
+            at_what = "RMSNorm + q|k|v + RoPE, decode attention, o_proj + residual"
     out = {
         "metric": "batch-1 decode tokens/s", "value": round(tok_s, 2), "unit": "tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "TinyLlama-1.1B-shaped Llama fp32 random-init seed 0, batch 1, prompt %d random ids, "
                                "greedy decode, static KV cache max_seq_len %d" % (args.prompt, cfg["max_seq_len"]),
-                   "layers": cfg["num_hidden_layers"], "hidden": H, "heads": "32q/4kv", "head_dim": 64,
+                   "layers": cfg["num_hidden_layers"], "hidden": H, "heads": "%dq/%dkv" % (hq, hkv), "head_dim": D,
                    "intermediate": I, "vocab": cfg["vocab_size"], "kv_len_during_timing": [len0, len0 + args.steps]},
-        "roofline": {"bound": "hbm", "kernel": "gemv_kernel<false, 2, 1, 2, 1> (RMSNorm + gate|up GEMV [11264,2048] + SwiGLU)",
+        "roofline": {"bound": "hbm", "kernel": "%s (RMSNorm + gate|up GEMV [%d,%d] + SwiGLU)" % (gu_kernel, 2 * I, H),
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic(),
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic(gu_kernel),
                      "bytes_per_launch": gu_bytes, "avg_launch_us": round(gu_avg_ms * 1e3, 3),
                      "avg_event_bracketed_us": round(gu_raw_ms * 1e3, 3),
                      "event_pair_overhead_us": round(event_overhead_ms * 1e3, 3)},
         "step_roofline": {"bytes_per_token": step_bytes, "achieved_GBps": round(step_bytes / (ms_per_step * 1e-3) / 1e9, 1),
                           "frac_of_8TBps": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                           "roofline_tokens_per_s": round(HBM_PEAK_GBS * 1e9 / step_bytes, 1)},
-        "attention": {"kernel": "attn_oproj_kernel<64, 4, 8, false> (decode attention + o_proj)" if fused_attn
-                      else "attn_decode_kernel<64, 8, 8, true>", "bytes_per_launch": at_bytes,
+        "attention": {"kernel": "%s (%s)" % (at_kernel, at_what), "bytes_per_launch": at_bytes,
                       "avg_launch_us": round(at_avg_ms * 1e3, 3), "achieved_GBps": round(at_bytes / (at_avg_ms * 1e-3) / 1e9, 1),
                       "frac_of_8TBps": round(at_bytes / (at_avg_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
-        "kernels": kernels,
+        "kernels": kernels, "kernel_instances": names,
         "prefill": dict(prefill_report(cfg, args.prompt, prefill_ms), passes_ms=[round(x, 3) for x in prefill_all_ms]),
         "decode_mode": args.mode, "eager_ms_per_step": round(eager_ms / args.steps, 5),
         "wall_s_timed_region": round(wall, 4), "setup_s": round(t_setup, 1),
@@ -197,13 +214,16 @@ def prefill_report(cfg, S, ms):
             "frac_of_mfma_bf16_peak": round(issued / MFMA_BF16_PEAK_TF, 4)}
 
 
-def measured_traffic():
+def measured_traffic(kernel):
     """HBM bytes per launch of the dominant kernel from the committed rocprofv3 --pmc runs
-    (FETCH_SIZE + WRITE_SIZE, calibrated on the copy kernel); counters cannot be read from here."""
+    (FETCH_SIZE + WRITE_SIZE, calibrated on the copy kernel); counters cannot be read from here.
+    None when those runs were taken on another kernel instance than the one launched now."""
     path = os.path.join(ROOT, "profiles", "decode_gateup_gemv_traffic.json")
     try:
         with open(path) as f:
             t = json.load(f)
+        if t["kernel"] != kernel:
+            return None
         return round(t["fetch_bytes_per_launch"] + t["write_bytes_per_launch"], 1)
     except (OSError, KeyError, ValueError):
         return None
@@ -362,7 +382,8 @@ def cpu_baseline(cfg, params, prompt, n_tokens):
     dt = time.perf_counter() - t0
     return {"value": round(n_tokens / dt, 3), "unit": "tokens/s", "cores": lo.get_threads(), "kind": "port",
             "sample": "%d greedy decode tokens after the same %d-token prompt, same weights; C restatement of "
-                      "Lumen's CPU algorithms (gcc -O3, OpenMP), Rust toolchain unavailable" % (n_tokens, len(prompt))}
+                      "Lumen's CPU algorithms (gcc -O3 -march=x86-64-v3 -ffp-contract=off, OpenMP), Rust toolchain "
+                      "unavailable" % (n_tokens, len(prompt))}
 
 
 if __name__ == "__main__":

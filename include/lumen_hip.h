@@ -63,6 +63,8 @@ int lumen_ctx_set_stream(lumen_ctx *ctx, void *hip_stream);
 int lumen_ctx_synchronize(lumen_ctx *ctx);
 /* HIP-event stopwatch on the ctx stream: start enqueues an event, stop
  * enqueues a second one, waits for it and returns the elapsed milliseconds */
+/* compute units of the context's device (what the launchers size their grids by) */
+int lumen_ctx_num_cus(const lumen_ctx *ctx, int *num_cus_out);
 int lumen_timer_start(lumen_ctx *ctx);
 int lumen_timer_stop(lumen_ctx *ctx, float *ms_out);
 
@@ -72,6 +74,8 @@ int lumen_malloc(lumen_ctx *ctx, size_t bytes, void **dev_out);
 int lumen_free(lumen_ctx *ctx, void *dev);
 int lumen_upload(lumen_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);
 int lumen_download(lumen_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes);
+/* device to device, in stream order (e.g. laying w_q | w_k | w_v out as one matrix for lumen_qkv_rope_append_f32) */
+int lumen_copy_d2d(lumen_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes);
 
 /* --------------------------------------------------------------------- ops */
 /* ops::matmul::matmul forward, src/ops/matmul.rs:10-99.  A [M, K_a] @ W[N, K_w]^T
@@ -86,6 +90,31 @@ int lumen_matmul_f32(lumen_ctx *ctx, const float *A_dev, const float *W_dev, flo
 int lumen_gemv_f32(lumen_ctx *ctx, const float *W_dev, const float *x_dev, float *y_dev, int N, int K);
 int lumen_gemm_f32(lumen_ctx *ctx, const float *A_dev, const float *W_dev, float *C_dev,
                    int M, int N, int K);
+/* The fused form of the decoder layer's leaves for one token (M == 1), one launch each: y = epilogue(W rmsnorm(x)).
+ * W [N, K] f32, or bf16 bits with w_bf16 = 1.  norm_w [K] not null: x is RMS-normalised first, (x * inv_rms) * g
+ * with eps (RMSNorm::forward, src/layers/norm/rms_norm.rs:24-62, as applied in src/models/llama.rs:107, :113, :202);
+ * norm_w null: x as it is.  Epilogues:
+ *   STORE     y [N] = W x                                        (Linear::forward, src/ops/matmul.rs:42-69)
+ *   RESIDUAL  y [N] = residual [N] + W x                         (src/models/llama.rs:110, :115)
+ *   SWIGLU    W holds gate_proj and up_proj row-interleaved (row 2i = gate_i, row 2i + 1 = up_i, N = 2 I; build it
+ *             once with lumen_interleave_rows): y [N / 2] = silu(gate) * up   (LlamaMLP::forward, llama.rs:59-65)
+ * K must be a multiple of 4 (8 for bf16) and at most 16384, operands 16-byte aligned -> else LUMEN_ERR_UNSUPPORTED.
+ * A decoder layer is five launches with these: lumen_qkv_rope_append_f32, lumen_attn_decode_prerotated_f32,
+ * RESIDUAL (o_proj), RMSNorm + SWIGLU (gate|up), RESIDUAL (down); the model-level step (lumen_llama_forward) needs
+ * three on short caches. */
+#define LUMEN_GEMV_EPI_STORE 0
+#define LUMEN_GEMV_EPI_RESIDUAL 1
+#define LUMEN_GEMV_EPI_SWIGLU 2
+#define LUMEN_GEMV_EPI_ARGMAX 3   /* model-internal (lm_head + greedy pick); named here for lumen_gemv_kernel_name */
+#define LUMEN_GEMV_EPI_ROPE_QKV 4 /* what lumen_qkv_rope_append_f32 launches */
+int lumen_gemv_fused_f32(lumen_ctx *ctx, const void *W_dev, int w_bf16, const float *x_dev, float *y_dev, int N, int K,
+                         const float *norm_w_dev, float eps, int epilogue, const float *residual_dev);
+/* out row 2i = a row i, out row 2i + 1 = b row i (rows of row_bytes bytes each, device memory, no overlap) */
+int lumen_interleave_rows(lumen_ctx *ctx, const void *a_dev, const void *b_dev, void *out_dev, int rows, size_t row_bytes);
+/* Name of the kernel instance -- template arguments as a profiler prints them -- that the fused product launches
+ * for W [N, K] on a device with num_cus compute units (MI355X: 256), aligned operands.  Host only: no GPU needed.
+ * The launcher and this function read the same decision. */
+int lumen_gemv_kernel_name(int num_cus, int N, int K, int w_bf16, int rmsnorm, int epilogue, char *buf, int buf_len);
 /* same products with W stored as bf16 bits and widened on load, f32 accumulate:
  * the device-side form of the reference's load-time upcast, src/loader.rs:50-64 */
 int lumen_gemv_bf16w(lumen_ctx *ctx, const uint16_t *W_dev, const float *x_dev, float *y_dev, int N, int K);
@@ -163,6 +192,20 @@ int lumen_kv_cache_get_view(const lumen_kv_cache *cache, int current_len, float 
 int lumen_attn_decode_f32(lumen_kv_cache *cache, lumen_rope *rope, const float *q3_dev,
                           const float *k3_dev, const float *v3_dev, float *out_dev,
                           int h, float scale, int causal);
+/* The fused decode step of SelfAttention::forward (S == 1, batch 1) as two operators.
+ * lumen_qkv_rope_append_f32: RMSNorm (norm_w null: none) + the q, k, v projections as ONE product -- Wqkv
+ * [(n_head + 2 n_kv_head) * head_dim, K] = the rows of w_q, w_k, w_v one after the other, f32 or bf16 bits -- +
+ * rotation of q and k at position cache.len + write of the rotated k and the raw v to cache row cache.len
+ * (src/layers/attention/self_attention.rs:106-108, :161-176, :220-227; input norm: src/models/llama.rs:107).
+ * q_rot_out [n_head * head_dim] is the rotated query.  The cache length does not advance.  Errors as
+ * lumen_attn_decode_f32 (KV overflow, RoPE range, shapes); the first call on a cache allocates 4 bytes.
+ * lumen_attn_decode_prerotated_f32: attention of that query over cache rows [0, cache.len] -- the appended row
+ * included -- (self_attention.rs:183-297); out [n_head * head_dim]; the cache length advances by one. */
+int lumen_qkv_rope_append_f32(lumen_kv_cache *cache, lumen_rope *rope, const void *Wqkv_dev, int w_bf16,
+                              const float *x_dev, int K, const float *norm_w_dev, float eps, float *q_rot_out_dev,
+                              int n_head);
+int lumen_attn_decode_prerotated_f32(lumen_kv_cache *cache, const float *q_rot_dev, float *out_dev, int n_head,
+                                     float scale);
 /* The same decode step for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments,
  * same results, bit for bit, as lumen_attn_decode_f32, but the scratch that the slices of a long cache need
@@ -270,6 +313,8 @@ int lumen_llama_decode_profile(lumen_llama *model, int first_id, int n, double *
 #define LUMEN_DECODE_GRAPH 1
 #define LUMEN_DECODE_PERSISTENT 2
 int lumen_llama_set_decode_mode(lumen_llama *model, int mode);
+/* name of the kernel instance the last lumen_llama_decode_profile launched for a class ("" if none) */
+int lumen_llama_profile_kernel_name(const lumen_llama *model, int kernel_class, char *buf, int buf_len);
 /* While the cache is short (up to 512 rows, 256 for head_dim 128) and the shape allows (no q/k norm, head_dim 64 or
  * 128, n_head * head_dim a multiple of 512), decode attention and the o_proj product of a layer are ONE launch:
  * attention workgroups hand their output to resident o_proj workgroups, whose weights are already in registers,

@@ -55,13 +55,18 @@ SIGNATURES = {
     "lumen_timer_stop": (_i, [_vp, C.POINTER(_f)]),
     "lumen_malloc": (_i, [_vp, C.c_size_t, _pp]),
     "lumen_free": (_i, [_vp, _vp]),
+    "lumen_ctx_num_cus": (_i, [_vp, _vp]),
     "lumen_upload": (_i, [_vp, _vp, _vp, C.c_size_t]),
     "lumen_download": (_i, [_vp, _vp, _vp, C.c_size_t]),
+    "lumen_copy_d2d": (_i, [_vp, _vp, _vp, C.c_size_t]),
     "lumen_matmul_f32": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     "lumen_gemv_f32": (_i, [_vp, _vp, _vp, _vp, _i, _i]),
     "lumen_gemv_bench": (_i, [_vp, _vp, C.c_size_t, _i, _i, _vp, _vp, _i, _i, _i, C.POINTER(_f)]),
     "lumen_gemm_f32": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i]),
     "lumen_gemv_bf16w": (_i, [_vp, _vp, _vp, _vp, _i, _i]),
+    "lumen_gemv_fused_f32": (_i, [_vp, _vp, _i, _vp, _vp, _i, _i, _vp, _f, _i, _vp]),
+    "lumen_interleave_rows": (_i, [_vp, _vp, _vp, _vp, _i, C.c_size_t]),
+    "lumen_gemv_kernel_name": (_i, [_i, _i, _i, _i, _i, _i, C.c_char_p, _i]),
     "lumen_gemm_bf16w": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i]),
     "lumen_rmsnorm_f32": (_i, [_vp, _vp, _vp, _vp, _i, _i, _f]),
     "lumen_silu_f32": (_i, [_vp, _vp, _vp, C.c_size_t]),
@@ -86,6 +91,8 @@ SIGNATURES = {
     "lumen_kv_cache_get_view": (_i, [_vp, _i, _vp, _vp]),
     "lumen_attn_decode_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _f, _i]),
     "lumen_attn_decode_static_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _f, _i]),
+    "lumen_qkv_rope_append_f32": (_i, [_vp, _vp, _vp, _i, _vp, _i, _vp, _f, _vp, _i]),
+    "lumen_attn_decode_prerotated_f32": (_i, [_vp, _vp, _vp, _i, _f]),
     "lumen_attn_prefill_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _i]),
     "lumen_llama_create": (_i, [_vp, C.POINTER(LlamaConfigStruct), _pp]),
     "lumen_llama_destroy": (_i, [_vp]),
@@ -102,6 +109,7 @@ SIGNATURES = {
     "lumen_llama_decode_profile": (_i, [_vp, _i, _i, C.POINTER(C.c_double), C.POINTER(_i), _i]),
     "lumen_llama_set_decode_mode": (_i, [_vp, _i]),
     "lumen_llama_set_handover": (_i, [_vp, _i, C.c_int64, _i, _i, _i]),
+    "lumen_llama_profile_kernel_name": (_i, [_vp, _i, C.c_char_p, _i]),
     "lumen_llama_get_decode_mode": (_i, [_vp, C.POINTER(_i)]),
     "lumen_llama_reset": (_i, [_vp]),
     "lumen_llama_kv_len": (_i, [_vp, C.POINTER(_i)]),
@@ -122,7 +130,16 @@ def load():
     return lib
 
 
+GEMV_EPI_STORE, GEMV_EPI_RESIDUAL, GEMV_EPI_SWIGLU, GEMV_EPI_ARGMAX, GEMV_EPI_ROPE_QKV = range(5)
+
 lib = load()
+
+
+def gemv_kernel_name(num_cus, n, k, w_bf16, rmsnorm, epilogue):
+    """The kernel instance the fused vector-matrix product launches for W [n, k] (host only, no GPU needed)."""
+    buf = C.create_string_buffer(160)
+    check(lib.lumen_gemv_kernel_name(int(num_cus), int(n), int(k), int(bool(w_bf16)), int(bool(rmsnorm)), int(epilogue), buf, 160))
+    return buf.value.decode()
 
 
 def check(status):

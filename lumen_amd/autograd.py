@@ -27,6 +27,12 @@ class Context:
         check(lib.lumen_ctx_create(device, C.byref(h)))
         self.handle = h
 
+    @property
+    def num_cus(self):
+        v = C.c_int()
+        check(lib.lumen_ctx_num_cus(self.handle, C.byref(v)))
+        return v.value
+
     def synchronize(self):
         check(lib.lumen_ctx_synchronize(self.handle))
 

@@ -363,6 +363,8 @@ static int launch_decode_d(lumen_ctx *ctx, const AttnDecodeArgs &a) {
 #undef LAUNCH_DECODE
 #undef DECODE_HOT
     LUMEN_CHECK_LAUNCH();
+    note_kernel(ctx, "attn_decode_kernel<%d, %d, %d, %s>", D, (nrep == 1 || nrep == 2 || nrep == 4 || nrep == 8) ? nrep : 0, WAVES,
+                a.pre_rotated ? "true" : "false");
     return LUMEN_OK;
 }
 
@@ -547,6 +549,7 @@ extern "C" int lumen_kv_cache_destroy(lumen_kv_cache *c) {
     hipFree(c->part);
     hipFree(c->counters);
     hipFree(c->q_rot);
+    hipFree(c->d_pos);
     delete c;
     return LUMEN_OK;
 }
@@ -655,6 +658,56 @@ extern "C" int lumen_attn_decode_f32(lumen_kv_cache *c, lumen_rope *rope, const 
     const int nsplit = attn_decode_nsplit(c->max_seq, c->d);
     LUMEN_TRY(ensure_split_scratch(c, h, nsplit));
     return attn_decode_entry(c, rope, q3, k3, v3, out, h, scale, c->part, c->counters, nsplit);
+}
+
+// ------------------------------------------------ the fused decode step of SelfAttention::forward, as two operators
+__global__ void set_int_kernel(int *p, int v) { *p = v; }
+
+// RMSNorm + q|k|v product + RoPE + cache append in one launch: what self_attention.rs:106-108 (projections),
+// :161-176 (new row into the cache) and :220-227 (rotation of q) do for S == 1, with the input norm of
+// llama.rs:107 on the way in.  W [(h + 2 h_kv) * d, K]: the rows of w_q, w_k, w_v one after the other.
+// q comes back rotated; the cache length does NOT advance (lumen_attn_decode_prerotated_f32 does that).
+extern "C" int lumen_qkv_rope_append_f32(lumen_kv_cache *c, lumen_rope *rope, const void *Wqkv, int w_bf16, const float *x,
+                                         int K, const float *norm_w, float eps, float *q_rot_out, int h) {
+    if (!c || !rope || !Wqkv || !x || !q_rot_out) LUMEN_FAIL(LUMEN_ERR_INVALID, "qkv_rope_append: null argument");
+    if (c->b != 1) LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "qkv_rope_append: batch 1 only (cache batch %d)", c->b);
+    if (rope->dim != c->d) LUMEN_FAIL(LUMEN_ERR_SHAPE, "RoPE dimension mismatch: %d vs head_dim %d", rope->dim, c->d);
+    if (h <= 0 || h % c->h_kv) LUMEN_FAIL(LUMEN_ERR_SHAPE, "qkv_rope_append: %d heads over %d kv heads", h, c->h_kv);
+    if (c->d % 2 || K <= 0) LUMEN_FAIL(LUMEN_ERR_SHAPE, "qkv_rope_append: head_dim %d, K %d", c->d, K);
+    if (c->len + 1 > c->max_seq)  // self_attention.rs:144-149
+        LUMEN_FAIL(LUMEN_ERR_KV_OVERFLOW, "KV cache overflow: new_len=%d > max_seq=%d", c->len + 1, c->max_seq);
+    if (c->len >= rope->max_seq)  // encoding.rs:176-181
+        LUMEN_FAIL(LUMEN_ERR_ROPE_RANGE, "RoPE index out of range: pos %d >= max %d", c->len, rope->max_seq);
+    lumen_ctx *ctx = c->ctx;
+    HIP_TRY(hipSetDevice(ctx->device));
+    if (!c->d_pos) HIP_TRY(hipMalloc(&c->d_pos, sizeof(int)));
+    hipLaunchKernelGGL(set_int_kernel, dim3(1), dim3(1), 0, ctx->stream, c->d_pos, c->len);
+    LUMEN_CHECK_LAUNCH();
+    GemvArgs g = {};
+    g.W = Wqkv; g.x = x; g.y = q_rot_out; g.N = (h + 2 * c->h_kv) * c->d; g.K = K; g.w_bf16 = w_bf16 ? 1 : 0;
+    g.pro = norm_w ? PRO_RMSNORM : PRO_NONE; g.norm_w = norm_w; g.eps = eps;
+    g.epi = EPI_ROPE_QKV; g.cos_t = rope->cos_dev; g.sin_t = rope->sin_dev; g.pos = c->d_pos;
+    g.k_cache = c->k; g.v_cache = c->v; g.hq = h; g.hkv = c->h_kv; g.D = c->d; g.max_seq = c->max_seq;
+    return launch_gemv(ctx, g);
+}
+
+// Decode attention over the cache INCLUDING the row lumen_qkv_rope_append_f32 just wrote, q rotated already
+// (self_attention.rs:183-297); the cache length advances by one.
+extern "C" int lumen_attn_decode_prerotated_f32(lumen_kv_cache *c, const float *q_rot, float *out, int h, float scale) {
+    if (!c || !q_rot || !out) LUMEN_FAIL(LUMEN_ERR_INVALID, "attn_decode_prerotated: null argument");
+    if (h <= 0 || h % c->h_kv) LUMEN_FAIL(LUMEN_ERR_SHAPE, "attn_decode: %d heads over %d kv heads", h, c->h_kv);
+    if (c->len + 1 > c->max_seq)
+        LUMEN_FAIL(LUMEN_ERR_KV_OVERFLOW, "KV cache overflow: new_len=%d > max_seq=%d", c->len + 1, c->max_seq);
+    const int nsplit = attn_decode_nsplit(c->max_seq, c->d);
+    LUMEN_TRY(ensure_split_scratch(c, h, nsplit));
+    AttnDecodeArgs a = {};
+    a.q = q_rot; a.out = out; a.k_cache = c->k; a.v_cache = c->v;
+    a.pos_dev = nullptr; a.pos_host = c->len;
+    a.b = c->b; a.hq = h; a.hkv = c->h_kv; a.d = c->d; a.max_seq = c->max_seq; a.scale = scale;
+    a.part = c->part; a.counters = c->counters; a.nsplit = nsplit; a.pre_rotated = 1;
+    LUMEN_TRY(launch_attn_decode(c->ctx, a));
+    c->len += 1;
+    return LUMEN_OK;
 }
 
 // ------------------------------------------------ decode attention that allocates nothing

@@ -296,6 +296,7 @@ static int launch_ao(lumen_ctx *ctx, const AttnOprojArgs &a) {
     }
 #undef AO_LAUNCH
     LUMEN_CHECK_LAUNCH();
+    note_kernel(ctx, "attn_oproj_kernel<%d, %d, %s, %s>", D, nlo, BF16 ? "true" : "false", a.Wqkv ? "true" : "false");
     const int seg[3] = {nq, nq + a.attn.hq, n_wg};
     stage_times_report(ctx, "(q|k|v |) attention | o_proj chain", n_wg,
                        "start, then q|k|v: [1] requests out, [2] x staged, [3] acknowledged; attention: [1] rows done, "

@@ -1,5 +1,7 @@
 // Context, device memory, stopwatch and error reporting of liblumen_hip.so.
 #include "internal.h"
+#include <cstdarg>
+#include <cstdio>
 
 #include <cstring>
 
@@ -115,4 +117,25 @@ extern "C" int lumen_download(lumen_ctx *ctx, void *dst_host, const void *src_de
     HIP_TRY(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
     HIP_TRY(hipStreamSynchronize(ctx->stream));
     return LUMEN_OK;
+}
+
+extern "C" int lumen_ctx_num_cus(const lumen_ctx *ctx, int *num_cus_out) {
+    if (!ctx || !num_cus_out) LUMEN_FAIL(LUMEN_ERR_INVALID, "null argument");
+    *num_cus_out = ctx->num_cus;
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_copy_d2d(lumen_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes) {
+    if (!ctx || (bytes && (!dst_dev || !src_dev))) LUMEN_FAIL(LUMEN_ERR_INVALID, "null argument");
+    if (!bytes) return LUMEN_OK;
+    HIP_TRY(hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+    return LUMEN_OK;
+}
+
+void note_kernel(lumen_ctx *ctx, const char *fmt, ...) {
+    if (!ctx || !ctx->note_kernels) return;
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(ctx->last_kernel, sizeof ctx->last_kernel, fmt, ap);
+    va_end(ap);
 }

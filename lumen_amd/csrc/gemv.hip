@@ -565,7 +565,7 @@ static void launch_pro(const GemvArgs &a, dim3 grid, int threads, size_t lds, hi
 }
 
 // Grid of the fused kernel for an [N, K] product: workgroups and threads per workgroup.
-int gemv_grid(const lumen_ctx *ctx, int N, int K, int w_bf16, int epi, int *threads_out) {
+static int gemv_grid_cus(int num_cus, int N, int K, int w_bf16, int epi, int *threads_out) {
     const int vec = w_bf16 ? 8 : 4;
     const int R = (epi == EPI_SWIGLU || epi == EPI_ROPE_QKV || N >= 8192) ? 2 : 1;
     const int piece = 64 * vec * (8 / R);
@@ -576,8 +576,8 @@ int gemv_grid(const lumen_ctx *ctx, int N, int K, int w_bf16, int epi, int *thre
     // per compute unit, take that shape -- every compute unit gets the same share and stages x once
     // (q|k|v of a 2048-wide model: 1280 pairs = 256 x 5; its o_proj and down: 2048 rows = 256 x 8).
     int waves = GEMV_WAVES;
-    if (nunits % ctx->num_cus == 0) {
-        const int w = nunits / ctx->num_cus;
+    if (nunits % num_cus == 0) {
+        const int w = nunits / num_cus;
         if (w > GEMV_WAVES && w <= GEMV_MAX_WAVES) waves = w;
     }
     const int threads = waves * 64;
@@ -589,7 +589,7 @@ int gemv_grid(const lumen_ctx *ctx, int N, int K, int w_bf16, int epi, int *thre
     const int max_per_cu = 16 / waves > 1 ? 16 / waves : 1;  // 16 wavefronts per compute unit
     if (per_cu > max_per_cu) per_cu = max_per_cu;
     if (per_cu < 1) per_cu = 1;
-    const int cap = ctx->num_cus * per_cu;
+    const int cap = num_cus * per_cu;
     if (blocks > cap) {
         // every wavefront the same number of units: with the grid simply cut at the cap some wavefronts
         // would take one unit more than the others, and those late, dependent requests are the kernel's tail
@@ -600,68 +600,93 @@ int gemv_grid(const lumen_ctx *ctx, int N, int K, int w_bf16, int epi, int *thre
     return blocks;
 }
 
+int gemv_grid(const lumen_ctx *ctx, int N, int K, int w_bf16, int epi, int *threads_out) {
+    return gemv_grid_cus(ctx->num_cus, N, K, w_bf16, epi, threads_out);
+}
+
+GemvPick gemv_pick(int num_cus, int N, int K, int w_bf16, int pro, int epi, bool aligned) {
+    GemvPick p = {};
+    const int vec = w_bf16 ? 8 : 4;
+    p.R = (epi == EPI_SWIGLU || epi == EPI_ROPE_QKV || N >= 8192) ? 2 : 1;
+    const int piece = 64 * vec * (8 / p.R);  // x is staged zero-padded to whole pieces
+    const int kpad = (K + piece - 1) / piece * piece;
+    p.lds = (size_t)kpad * sizeof(float);
+    p.fast = (K % vec == 0) && aligned && p.lds <= 64 * 1024;
+    p.pro = pro;
+    p.epi = pro == PRO_ATTN_FOLD ? (int)EPI_RESIDUAL : epi;
+    if (!p.fast) {
+        p.threads = GEMV_THREADS;
+        p.blocks = (N + GEMV_WAVES - 1) / GEMV_WAVES;
+        if (p.blocks > num_cus * 8) p.blocks = num_cus * 8;
+        return p;
+    }
+    p.blocks = gemv_grid_cus(num_cus, N, K, w_bf16, epi, &p.threads);
+    // How x is staged (see stage_x, request_early): ahead of the weights where every wavefront has a
+    // single unit of at most two pieces -- all of its loads go out at once and the prologue is what the
+    // multiplies wait for -- and a thread stages at most GEMV_EARLY pieces; else in the loop, four pieces
+    // at a time from three pieces per thread on.
+    const int x_pieces = (kpad + p.threads * 4 - 1) / (p.threads * 4);
+    const int nunits = (N + p.R - 1) / p.R;
+    const bool early_x = pro != PRO_ATTN_FOLD && x_pieces <= GEMV_EARLY && kpad / piece <= 2 &&
+                         nunits <= p.blocks * (p.threads / 64);
+    p.xb = early_x ? 0 : x_pieces > 2 ? 4 : 1;
+    p.ka = K % piece == 0;  // whole pieces: no clamped load positions
+    return p;
+}
+
+int gemv_kernel_name(const GemvPick &p, int w_bf16, char *buf, int buf_len) {
+    if (!p.fast) return snprintf(buf, buf_len, "gemv_generic_kernel<%s>", w_bf16 ? "true" : "false");
+    return snprintf(buf, buf_len, "gemv_kernel<%s, %d, %d, %d, %d, %s>", w_bf16 ? "true" : "false", p.R, p.pro, p.epi, p.xb,
+                    p.ka ? "true" : "false");
+}
+
 int gemv_max_blocks(const lumen_ctx *ctx) { return ctx->num_cus * 4; }
 
 int launch_gemv(lumen_ctx *ctx, const GemvArgs &a) {
     if (a.N <= 0 || a.K <= 0) return LUMEN_OK;
     const int vec = a.w_bf16 ? 8 : 4;
-    const int R = (a.epi == EPI_SWIGLU || a.epi == EPI_ROPE_QKV || a.N >= 8192) ? 2 : 1;
-    const int piece = 64 * vec * (8 / R);  // x is staged zero-padded to whole pieces
-    const int kpad = (a.K + piece - 1) / piece * piece;
-    const size_t lds = (size_t)kpad * sizeof(float);
     const bool aligned = (((uintptr_t)a.W | (uintptr_t)a.x) & 15) == 0 && (((uintptr_t)a.attn_part) & 7) == 0 &&
                          (a.pro != PRO_RMSNORM || ((uintptr_t)a.norm_w & 15) == 0);
-    const bool fast = (a.K % vec == 0) && aligned && lds <= 64 * 1024;
-    if (!fast) {
+    const GemvPick p = gemv_pick(ctx->num_cus, a.N, a.K, a.w_bf16, a.pro, a.epi, aligned);
+    if (ctx->note_kernels) gemv_kernel_name(p, a.w_bf16, ctx->last_kernel, sizeof ctx->last_kernel);
+    if (!p.fast) {
         if (a.pro != PRO_NONE || a.epi != EPI_STORE || a.row_sel)
             LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "fused GEMV needs K %% %d == 0, 16-byte alignment and K <= %d (K=%d)", vec,
                        16384, a.K);
-        int blocks = (a.N + GEMV_WAVES - 1) / GEMV_WAVES;
-        if (blocks > ctx->num_cus * 8) blocks = ctx->num_cus * 8;
         if (a.w_bf16)
-            hipLaunchKernelGGL(gemv_generic_kernel<true>, dim3(blocks), dim3(GEMV_THREADS), 0, ctx->stream, a);
+            hipLaunchKernelGGL(gemv_generic_kernel<true>, dim3(p.blocks), dim3(p.threads), 0, ctx->stream, a);
         else
-            hipLaunchKernelGGL(gemv_generic_kernel<false>, dim3(blocks), dim3(GEMV_THREADS), 0, ctx->stream, a);
+            hipLaunchKernelGGL(gemv_generic_kernel<false>, dim3(p.blocks), dim3(p.threads), 0, ctx->stream, a);
         LUMEN_CHECK_LAUNCH();
         return LUMEN_OK;
     }
     if (a.pro == PRO_ATTN_FOLD) {
-        if (a.epi != EPI_RESIDUAL || R != 1 || !a.attn_part || !a.attn_pos || a.attn_d <= 0 || a.attn_d % 4 ||
+        if (a.epi != EPI_RESIDUAL || p.R != 1 || !a.attn_part || !a.attn_pos || a.attn_d <= 0 || a.attn_d % 4 ||
             a.K % a.attn_d || a.attn_nslices < 1 || a.attn_nslices > GEMV_FOLD_MAX_SLICES)
             LUMEN_FAIL(LUMEN_ERR_INVALID, "GEMV over attention partials: one row per unit, residual epilogue, at most %d slices (got %d)",
                        GEMV_FOLD_MAX_SLICES, a.attn_nslices);
     }
     if ((a.epi == EPI_SWIGLU || a.epi == EPI_ROPE_QKV) && (a.N & 1))
         LUMEN_FAIL(LUMEN_ERR_SHAPE, "paired-row epilogue needs an even row count, got %d", a.N);
-    int threads = 0;
-    const int blocks = gemv_grid(ctx, a.N, a.K, a.w_bf16, a.epi, &threads);
+    const int threads = p.threads, blocks = p.blocks;
+    const size_t lds = p.lds;
     dim3 grid(blocks);
-    // How x is staged (see stage_x, request_early): ahead of the weights where every wavefront has a
-    // single unit of at most two pieces -- all of its loads go out at once and the prologue is what the
-    // multiplies wait for -- and a thread stages at most GEMV_EARLY pieces; else in the loop, four pieces
-    // at a time from three pieces per thread on.
-    const int x_pieces = (kpad + threads * 4 - 1) / (threads * 4);
-    const int nunits = (a.N + R - 1) / R;
-    const bool early_x = a.pro != PRO_ATTN_FOLD && x_pieces <= GEMV_EARLY && kpad / piece <= 2 &&
-                         nunits <= blocks * (threads / 64);
-    const bool batch_x = x_pieces > 2;
-    const bool ka = a.K % piece == 0;  // whole pieces: no clamped load positions
 #define LAUNCH_GEMV_K(BF, RR, KAV)                                                       \
     do {                                                                                 \
-        if (early_x) launch_pro<BF, RR, 0, KAV>(a, grid, threads, lds, ctx->stream);      \
-        else if (batch_x) launch_pro<BF, RR, 4, KAV>(a, grid, threads, lds, ctx->stream); \
+        if (p.xb == 0) launch_pro<BF, RR, 0, KAV>(a, grid, threads, lds, ctx->stream);      \
+        else if (p.xb == 4) launch_pro<BF, RR, 4, KAV>(a, grid, threads, lds, ctx->stream); \
         else launch_pro<BF, RR, 1, KAV>(a, grid, threads, lds, ctx->stream);             \
     } while (0)
 #define LAUNCH_GEMV(BF, RR)                  \
     do {                                     \
-        if (ka) LAUNCH_GEMV_K(BF, RR, true); \
+        if (p.ka) LAUNCH_GEMV_K(BF, RR, true); \
         else LAUNCH_GEMV_K(BF, RR, false);   \
     } while (0)
     if (a.w_bf16) {
-        if (R == 2) LAUNCH_GEMV(true, 2);
+        if (p.R == 2) LAUNCH_GEMV(true, 2);
         else LAUNCH_GEMV(true, 1);
     } else {
-        if (R == 2) LAUNCH_GEMV(false, 2);
+        if (p.R == 2) LAUNCH_GEMV(false, 2);
         else LAUNCH_GEMV(false, 1);
     }
 #undef LAUNCH_GEMV
@@ -694,6 +719,42 @@ extern "C" int lumen_gemv_bf16w(lumen_ctx *ctx, const uint16_t *W, const float *
     GemvArgs a = {};
     a.W = W; a.x = x; a.y = y; a.N = N; a.K = K; a.w_bf16 = 1; a.pro = PRO_NONE; a.epi = EPI_STORE;
     return launch_gemv(ctx, a);
+}
+
+// The fused forms the decode step is made of, as an operator: optional RMSNorm on the way in (x is read from memory
+// once), the epilogue on the way out.
+extern "C" int lumen_gemv_fused_f32(lumen_ctx *ctx, const void *W, int w_bf16, const float *x, float *y, int N, int K,
+                                    const float *norm_w, float eps, int epilogue, const float *residual) {
+    LUMEN_TRY(check_gemv(ctx, W, x, y, N, K));
+    if (epilogue != LUMEN_GEMV_EPI_STORE && epilogue != LUMEN_GEMV_EPI_RESIDUAL && epilogue != LUMEN_GEMV_EPI_SWIGLU)
+        LUMEN_FAIL(LUMEN_ERR_INVALID, "gemv_fused: unknown epilogue %d", epilogue);
+    if (epilogue == LUMEN_GEMV_EPI_RESIDUAL && !residual) LUMEN_FAIL(LUMEN_ERR_INVALID, "gemv_fused: residual epilogue without a residual");
+    GemvArgs a = {};
+    a.W = W; a.x = x; a.y = y; a.N = N; a.K = K; a.w_bf16 = w_bf16 ? 1 : 0;
+    a.pro = norm_w ? PRO_RMSNORM : PRO_NONE; a.norm_w = norm_w; a.eps = eps;
+    a.epi = epilogue == LUMEN_GEMV_EPI_RESIDUAL ? EPI_RESIDUAL : epilogue == LUMEN_GEMV_EPI_SWIGLU ? EPI_SWIGLU : EPI_STORE;
+    a.residual = residual;
+    return launch_gemv(ctx, a);
+}
+
+// out row 2i = a row i, out row 2i + 1 = b row i: the layout the SwiGLU epilogue wants of gate_proj / up_proj
+extern "C" int lumen_interleave_rows(lumen_ctx *ctx, const void *a, const void *b, void *out, int rows, size_t row_bytes) {
+    if (!ctx || !a || !b || !out) LUMEN_FAIL(LUMEN_ERR_INVALID, "interleave_rows: null argument");
+    if (rows < 0) LUMEN_FAIL(LUMEN_ERR_SHAPE, "interleave_rows: negative row count");
+    if (rows == 0 || row_bytes == 0) return LUMEN_OK;
+    HIP_TRY(hipMemcpy2DAsync(out, 2 * row_bytes, a, row_bytes, row_bytes, (size_t)rows, hipMemcpyDeviceToDevice, ctx->stream));
+    HIP_TRY(hipMemcpy2DAsync((char *)out + row_bytes, 2 * row_bytes, b, row_bytes, row_bytes, (size_t)rows, hipMemcpyDeviceToDevice,
+                             ctx->stream));
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_gemv_kernel_name(int num_cus, int N, int K, int w_bf16, int rmsnorm, int epilogue, char *buf, int buf_len) {
+    if (!buf || buf_len <= 0 || num_cus <= 0 || N <= 0 || K <= 0) LUMEN_FAIL(LUMEN_ERR_INVALID, "gemv_kernel_name: bad argument");
+    if (epilogue < LUMEN_GEMV_EPI_STORE || epilogue > LUMEN_GEMV_EPI_ROPE_QKV)
+        LUMEN_FAIL(LUMEN_ERR_INVALID, "gemv_kernel_name: unknown epilogue %d", epilogue);
+    const GemvPick p = gemv_pick(num_cus, N, K, w_bf16, rmsnorm ? PRO_RMSNORM : PRO_NONE, epilogue, true);
+    gemv_kernel_name(p, w_bf16, buf, buf_len);
+    return LUMEN_OK;
 }
 
 extern "C" int lumen_matmul_f32(lumen_ctx *ctx, const float *A, const float *W, float *C, int M, int N, int K_a,

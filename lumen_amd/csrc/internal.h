@@ -49,7 +49,12 @@ struct lumen_ctx {
     // this device's address of the fixed scratch array behind lumen_attn_decode_static_f32
     unsigned char *attn_static = nullptr;
     size_t attn_static_bytes = 0;
+    // name of the kernel instance the decode-path launchers started last (template arguments as a profiler prints
+    // them), kept while note_kernels is set: the per-class profile hands these names out
+    bool note_kernels = false;
+    char last_kernel[160] = {0};
 };
+void note_kernel(lumen_ctx *ctx, const char *fmt, ...);
 int attn_static_scratch_init(lumen_ctx *ctx);
 
 struct lumen_rope {
@@ -70,6 +75,7 @@ struct lumen_kv_cache {
     float *part = nullptr;  // [b*h_q_max, nsplit, d + 2]
     int *counters = nullptr;
     int part_heads = 0;
+    int *d_pos = nullptr;    // device copy of len for lumen_qkv_rope_append_f32, allocated at its first call
     float *q_rot = nullptr;  // rotated queries of the prefill entry point, grown on demand
     size_t q_rot_floats = 0;
 };
@@ -121,6 +127,19 @@ int launch_gemv(lumen_ctx *ctx, const GemvArgs &a);
 int gemv_max_blocks(const lumen_ctx *ctx);
 // grid of the fused GEMV kernel for an [N, K] product (workgroups; threads per workgroup in *threads_out)
 int gemv_grid(const lumen_ctx *ctx, int N, int K, int w_bf16, int epi, int *threads_out);
+// The template instance and launch shape the fused GEMV takes for a product: ONE function decides, the launcher
+// and the name report (lumen_gemv_kernel_name) both read it.
+struct GemvPick {
+    bool fast;         // the fused kernel (else the generic one: K not a multiple of the load width, unaligned, K > 16384)
+    int R;             // rows per unit
+    int pro, epi;      // template prologue / epilogue
+    int xb;            // 0: x requested ahead of the weights, 1: staged piece by piece, 4: four pieces at a time
+    bool ka;           // K is a whole number of pieces
+    int threads, blocks;
+    size_t lds;
+};
+GemvPick gemv_pick(int num_cus, int N, int K, int w_bf16, int pro, int epi, bool aligned);
+int gemv_kernel_name(const GemvPick &p, int w_bf16, char *buf, int buf_len);
 
 struct GemmArgs {
     const float *A;   // [M, K]

@@ -54,6 +54,7 @@ struct lumen_llama {
     // timing of the chain's o_proj workgroups (units of 256 clocks), per form: pause before the weight requests,
     // before the first poll, between polls (measured optima on the 2048-wide model; see attn_oproj.hip)
     int chain_pre[3] = {0, 10, 47}, chain_delay[3] = {0, 16, 13}, chain_gap[3] = {0, 1, 1};
+    std::string prof_names[16];  // per kernel class: the instance the last lumen_llama_decode_profile launched
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
     int graph_expect_short = 0;            // the hint the captured attention launches carry
@@ -405,11 +406,13 @@ int lumen_llama_param_list(const lumen_llama *m, std::vector<std::string> &names
 // Kernel classes of a decode step, for per-kernel timing.
 enum { KC_EMBED = 0, KC_QKV, KC_ATTN, KC_OPROJ, KC_GATEUP, KC_DOWN, KC_LMHEAD, KC_ARGMAX, KC_ATTN_OPROJ, KC_COUNT };
 
-struct StepProbe {  // brackets every launch with a HIP event pair when profiling
+struct StepProbe {  // brackets every launch with a HIP event pair when profiling, and keeps the kernel's name
     std::vector<hipEvent_t> ev;
     std::vector<int> cls;
     hipStream_t s = nullptr;
     bool on = false;
+    lumen_ctx *ctx = nullptr;
+    std::string *names = nullptr;  // [KC_COUNT]
     void before(int c) {
         if (!on) return;
         hipEvent_t e0, e1;
@@ -421,7 +424,9 @@ struct StepProbe {  // brackets every launch with a HIP event pair when profilin
         hipEventRecord(e0, s);
     }
     void after() {
-        if (on) hipEventRecord(ev.back(), s);
+        if (!on) return;
+        hipEventRecord(ev.back(), s);
+        if (names && ctx) names[cls.back()] = ctx->last_kernel;
     }
 };
 
@@ -812,7 +817,11 @@ extern "C" int lumen_llama_decode_profile(lumen_llama *m, int first_id, int n, d
         StepProbe pr;
         pr.on = true;
         pr.s = st;
+        pr.ctx = m->ctx;
+        pr.names = m->prof_names;
+        m->ctx->note_kernels = true;
         rc = enqueue_decode_step(m, &pr);
+        m->ctx->note_kernels = false;
         const hipError_t e = hipStreamSynchronize(st);
         if (rc == LUMEN_OK && e == hipSuccess) {
             m->len += 1;
@@ -831,6 +840,14 @@ extern "C" int lumen_llama_decode_profile(lumen_llama *m, int first_id, int n, d
         }
     }
     return rc;
+}
+
+extern "C" int lumen_llama_profile_kernel_name(const lumen_llama *m, int kernel_class, char *buf, int buf_len) {
+    if (!m || !buf || buf_len <= 0) LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_profile_kernel_name: null argument");
+    if (kernel_class < 0 || kernel_class >= KC_COUNT)
+        LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_profile_kernel_name: class %d of %d", kernel_class, (int)KC_COUNT);
+    snprintf(buf, (size_t)buf_len, "%s", m->prof_names[kernel_class].c_str());
+    return LUMEN_OK;
 }
 
 extern "C" int lumen_llama_reset(lumen_llama *m) {

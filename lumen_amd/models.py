@@ -170,6 +170,12 @@ class LlamaModel:
     KERNEL_CLASSES = ("embedding", "norm_qkv_gemv", "attn_decode", "oproj_gemv", "norm_gateup_gemv", "down_gemv",
                       "norm_lmhead_gemv", "argmax", "attn_oproj_fused")
 
+    def profile_kernel_name(self, kernel_class):
+        """The kernel instance the last decode_profile launched for a class ('' if none)."""
+        buf = C.create_string_buffer(160)
+        check(lib.lumen_llama_profile_kernel_name(self.handle, self.KERNEL_CLASSES.index(kernel_class), buf, 160))
+        return buf.value.decode()
+
     def decode_profile(self, first_id, n):
         """n greedy steps with every launch bracketed by HIP events: {class: (ms_sum, launches)}."""
         k = len(self.KERNEL_CLASSES)
@@ -213,7 +219,49 @@ class LlamaDecoderLayer:
         self.post_attention_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps,
                                                 params[prefix + "post_attention_layernorm.weight"], ctx)
 
+    def fuse(self):
+        """Lays the weights out for the fused single-token operators: w_q | w_k | w_v rows one after the other,
+        gate_proj / up_proj rows interleaved (device-to-device copies, once)."""
+        a, ctx = self.self_attn, self.self_attn.ctx
+        wq, wk, wv = a.w_q.weight, a.w_k.weight, a.w_v.weight
+        k = wq.shape[1]
+        self.w_qkv = Tensor.empty((wq.shape[0] + wk.shape[0] + wv.shape[0], k), np.float32, ctx)
+        off = 0
+        for w in (wq, wk, wv):
+            check(lib.lumen_copy_d2d(ctx.handle, self.w_qkv.ptr + off, w.ptr, w.size * 4))
+            off += w.size * 4
+        g, u = self.mlp.gate_proj.weight, self.mlp.up_proj.weight
+        self.w_gate_up = Tensor.empty((2 * g.shape[0], g.shape[1]), np.float32, ctx)
+        check(lib.lumen_interleave_rows(ctx.handle, g.ptr, u.ptr, self.w_gate_up.ptr, g.shape[0], g.shape[1] * 4))
+        self.fused = True
+
+    def forward_token(self, x, cache):
+        """forward_infer for S == 1 through the fused operators: five launches (llama.rs:104-116 with the leaves
+        of :59-65 and self_attention.rs:106-108, :161-176, :183-303 folded as the decode step folds them)."""
+        a, ctx = self.self_attn, self.self_attn.ctx
+        h, d = a.n_head, a.head_dim
+        hidden = x.shape[-1]
+        q_rot = Tensor.empty((h * d,), np.float32, ctx)
+        check(lib.lumen_qkv_rope_append_f32(cache.handle, a.rope.handle, self.w_qkv.ptr, 0, x.ptr, hidden,
+                                            self.input_layernorm.weight.ptr, self.input_layernorm.eps, q_rot.ptr, h))
+        attn = Tensor.empty((h * d,), np.float32, ctx)
+        check(lib.lumen_attn_decode_prerotated_f32(cache.handle, q_rot.ptr, attn.ptr, h, a.scale))
+        hbuf = Tensor.empty(x.shape, np.float32, ctx)
+        check(lib.lumen_gemv_fused_f32(ctx.handle, a.w_o.weight.ptr, 0, attn.ptr, hbuf.ptr, hidden, h * d, None, 0.0,
+                                       _lib.GEMV_EPI_RESIDUAL, x.ptr))
+        inter = self.mlp.down_proj.weight.shape[1]
+        act = Tensor.empty((inter,), np.float32, ctx)
+        check(lib.lumen_gemv_fused_f32(ctx.handle, self.w_gate_up.ptr, 0, hbuf.ptr, act.ptr, 2 * inter, hidden,
+                                       self.post_attention_layernorm.weight.ptr, self.post_attention_layernorm.eps,
+                                       _lib.GEMV_EPI_SWIGLU, None))
+        out = Tensor.empty(x.shape, np.float32, ctx)
+        check(lib.lumen_gemv_fused_f32(ctx.handle, self.mlp.down_proj.weight.ptr, 0, act.ptr, out.ptr, hidden, inter,
+                                       None, 0.0, _lib.GEMV_EPI_RESIDUAL, hbuf.ptr))
+        return out, cache
+
     def forward_infer(self, x, cache):
+        if getattr(self, "fused", False) and x.shape[0] == 1 and x.shape[1] == 1:
+            return self.forward_token(x, cache)
         norm_x = self.input_layernorm.forward(x)
         attn_out, cache_out = self.self_attn.forward(norm_x, cache)
         h = x + attn_out
@@ -223,9 +271,11 @@ class LlamaDecoderLayer:
 
 
 class LayeredLlamaModel:
-    """LlamaModel::forward (llama.rs:181-206) composed operator by operator."""
+    """LlamaModel::forward (llama.rs:181-206) composed operator by operator.  fused=True (default): a single
+    token (S == 1) takes the fused operators -- five launches per layer, and the final norm rides on the lm_head
+    product -- as the model-level decode step does; fused=False: one call per reference leaf, every time."""
 
-    def __init__(self, config, params, ctx=None):
+    def __init__(self, config, params, ctx=None, fused=True):
         if isinstance(config, dict):
             config = LlamaConfig.from_dict(config)
         if config.head_dim or config.qk_norm or config.tie_embeddings or config.weight_dtype != "f32":
@@ -237,6 +287,10 @@ class LayeredLlamaModel:
                        for i in range(config.num_hidden_layers)]
         self.norm = RMSNorm(config.hidden_size, config.rms_norm_eps, params["model.norm.weight"], self.ctx)
         self.lm_head = Linear(Tensor.from_array_no_grad(params["lm_head.weight"], self.ctx))
+        self.fused = bool(fused)
+        if self.fused:
+            for layer in self.layers:
+                layer.fuse()
 
     def init_kv_caches(self, batch_size=1):
         c = self.config
@@ -256,5 +310,11 @@ class LayeredLlamaModel:
         x = self.embed_tokens.forward(ids)
         for i, layer in enumerate(self.layers):
             x, caches[i] = layer.forward_infer(x, caches[i])
+        if self.fused and ids.shape[1] == 1:  # final norm + lm_head in one launch (llama.rs:202-205)
+            w = self.lm_head.weight
+            logits = Tensor.empty((1, 1, w.shape[0]), np.float32, self.ctx)
+            check(lib.lumen_gemv_fused_f32(self.ctx.handle, w.ptr, 0, x.ptr, logits.ptr, w.shape[0], w.shape[1],
+                                           self.norm.weight.ptr, self.norm.eps, _lib.GEMV_EPI_STORE, None))
+            return logits
         x = self.norm.forward(x)
         return self.lm_head.forward(x)

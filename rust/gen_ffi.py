@@ -1,6 +1,6 @@
-"""Writes include/lumen_hip_ffi.rs, the Rust `extern "C"` block for every prototype of lumen_hip.h.
+"""Writes rust/src/ffi.rs, the Rust `extern "C"` block for every prototype of include/lumen_hip.h.
 
-Usage: python include/gen_rust_ffi.py [--check]    (--check: exit 1 when the committed file is out of date)
+Usage: python rust/gen_ffi.py [--check]    (--check: exit 1 when the committed file is out of date)
 
 The reference crate is Rust; this file is what a maintainer drops into it as src/ffi.rs (add `mod ffi;` and
 link liblumen_hip.so from build.rs).
@@ -10,8 +10,8 @@ import re
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-HEADER = os.path.join(HERE, "lumen_hip.h")
-OUT = os.path.join(HERE, "lumen_hip_ffi.rs")
+HEADER = os.path.join(os.path.dirname(HERE), "include", "lumen_hip.h")
+OUT = os.path.join(HERE, "src", "ffi.rs")
 
 SCALARS = {"int": "c_int", "float": "c_float", "double": "f64", "size_t": "usize", "int32_t": "i32", "uint16_t": "u16",
            "int64_t": "i64", "uint64_t": "u64", "char": "c_char", "void": "c_void"}
@@ -75,7 +75,7 @@ def struct_fields(text, name):
 
 def generate():
     text = open(HEADER).read()
-    out = ["// Generated from include/lumen_hip.h by include/gen_rust_ffi.py -- do not edit.",
+    out = ["// Generated from include/lumen_hip.h by rust/gen_ffi.py -- do not edit.",
            "// Rust binding of liblumen_hip.so: src/ffi.rs + `mod ffi;` in the reference crate; link the library from build.rs.",
            "#![allow(non_camel_case_types, dead_code)]",
            "use std::os::raw::{c_char, c_float, c_int, c_void};", ""]

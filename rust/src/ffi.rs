@@ -1,4 +1,4 @@
-// Generated from include/lumen_hip.h by include/gen_rust_ffi.py -- do not edit.
+// Generated from include/lumen_hip.h by rust/gen_ffi.py -- do not edit.
 // Rust binding of liblumen_hip.so: src/ffi.rs + `mod ffi;` in the reference crate; link the library from build.rs.
 #![allow(non_camel_case_types, dead_code)]
 use std::os::raw::{c_char, c_float, c_int, c_void};
@@ -49,6 +49,11 @@ pub const LUMEN_ERR_NO_DEVICE: c_int = 8;
 pub const LUMEN_ERR_UNSUPPORTED: c_int = 9;
 pub const LUMEN_DTYPE_F32: c_int = 0;
 pub const LUMEN_DTYPE_BF16: c_int = 1;
+pub const LUMEN_GEMV_EPI_STORE: c_int = 0;
+pub const LUMEN_GEMV_EPI_RESIDUAL: c_int = 1;
+pub const LUMEN_GEMV_EPI_SWIGLU: c_int = 2;
+pub const LUMEN_GEMV_EPI_ARGMAX: c_int = 3;
+pub const LUMEN_GEMV_EPI_ROPE_QKV: c_int = 4;
 pub const LUMEN_DECODE_EAGER: c_int = 0;
 pub const LUMEN_DECODE_GRAPH: c_int = 1;
 pub const LUMEN_DECODE_PERSISTENT: c_int = 2;
@@ -60,15 +65,20 @@ extern "C" {
     pub fn lumen_ctx_destroy(ctx: *mut lumen_ctx) -> c_int;
     pub fn lumen_ctx_set_stream(ctx: *mut lumen_ctx, hip_stream: *mut c_void) -> c_int;
     pub fn lumen_ctx_synchronize(ctx: *mut lumen_ctx) -> c_int;
+    pub fn lumen_ctx_num_cus(ctx: *const lumen_ctx, num_cus_out: *mut c_int) -> c_int;
     pub fn lumen_timer_start(ctx: *mut lumen_ctx) -> c_int;
     pub fn lumen_timer_stop(ctx: *mut lumen_ctx, ms_out: *mut c_float) -> c_int;
     pub fn lumen_malloc(ctx: *mut lumen_ctx, bytes: usize, dev_out: *mut *mut c_void) -> c_int;
     pub fn lumen_free(ctx: *mut lumen_ctx, dev: *mut c_void) -> c_int;
     pub fn lumen_upload(ctx: *mut lumen_ctx, dst_dev: *mut c_void, src_host: *const c_void, bytes: usize) -> c_int;
     pub fn lumen_download(ctx: *mut lumen_ctx, dst_host: *mut c_void, src_dev: *const c_void, bytes: usize) -> c_int;
+    pub fn lumen_copy_d2d(ctx: *mut lumen_ctx, dst_dev: *mut c_void, src_dev: *const c_void, bytes: usize) -> c_int;
     pub fn lumen_matmul_f32(ctx: *mut lumen_ctx, A_dev: *const c_float, W_dev: *const c_float, C_dev: *mut c_float, M: c_int, N: c_int, K_a: c_int, K_w: c_int) -> c_int;
     pub fn lumen_gemv_f32(ctx: *mut lumen_ctx, W_dev: *const c_float, x_dev: *const c_float, y_dev: *mut c_float, N: c_int, K: c_int) -> c_int;
     pub fn lumen_gemm_f32(ctx: *mut lumen_ctx, A_dev: *const c_float, W_dev: *const c_float, C_dev: *mut c_float, M: c_int, N: c_int, K: c_int) -> c_int;
+    pub fn lumen_gemv_fused_f32(ctx: *mut lumen_ctx, W_dev: *const c_void, w_bf16: c_int, x_dev: *const c_float, y_dev: *mut c_float, N: c_int, K: c_int, norm_w_dev: *const c_float, eps: c_float, epilogue: c_int, residual_dev: *const c_float) -> c_int;
+    pub fn lumen_interleave_rows(ctx: *mut lumen_ctx, a_dev: *const c_void, b_dev: *const c_void, out_dev: *mut c_void, rows: c_int, row_bytes: usize) -> c_int;
+    pub fn lumen_gemv_kernel_name(num_cus: c_int, N: c_int, K: c_int, w_bf16: c_int, rmsnorm: c_int, epilogue: c_int, buf: *mut c_char, buf_len: c_int) -> c_int;
     pub fn lumen_gemv_bf16w(ctx: *mut lumen_ctx, W_dev: *const u16, x_dev: *const c_float, y_dev: *mut c_float, N: c_int, K: c_int) -> c_int;
     pub fn lumen_gemm_bf16w(ctx: *mut lumen_ctx, A_dev: *const c_float, W_dev: *const u16, C_dev: *mut c_float, M: c_int, N: c_int, K: c_int) -> c_int;
     pub fn lumen_gemv_bench(ctx: *mut lumen_ctx, W_base_dev: *const c_void, stride_elems: usize, ncopies: c_int, w_bf16: c_int, x_dev: *const c_float, y_dev: *mut c_float, N: c_int, K: c_int, iters: c_int, ms_out: *mut c_float) -> c_int;
@@ -94,6 +104,8 @@ extern "C" {
     pub fn lumen_kv_cache_update(cache: *mut lumen_kv_cache, k_dev: *const c_float, v_dev: *const c_float, s: c_int, start_pos: c_int) -> c_int;
     pub fn lumen_kv_cache_get_view(cache: *const lumen_kv_cache, current_len: c_int, k_out_dev: *mut c_float, v_out_dev: *mut c_float) -> c_int;
     pub fn lumen_attn_decode_f32(cache: *mut lumen_kv_cache, rope: *mut lumen_rope, q3_dev: *const c_float, k3_dev: *const c_float, v3_dev: *const c_float, out_dev: *mut c_float, h: c_int, scale: c_float, causal: c_int) -> c_int;
+    pub fn lumen_qkv_rope_append_f32(cache: *mut lumen_kv_cache, rope: *mut lumen_rope, Wqkv_dev: *const c_void, w_bf16: c_int, x_dev: *const c_float, K: c_int, norm_w_dev: *const c_float, eps: c_float, q_rot_out_dev: *mut c_float, n_head: c_int) -> c_int;
+    pub fn lumen_attn_decode_prerotated_f32(cache: *mut lumen_kv_cache, q_rot_dev: *const c_float, out_dev: *mut c_float, n_head: c_int, scale: c_float) -> c_int;
     pub fn lumen_attn_decode_static_f32(cache: *mut lumen_kv_cache, rope: *mut lumen_rope, q3_dev: *const c_float, k3_dev: *const c_float, v3_dev: *const c_float, out_dev: *mut c_float, h: c_int, scale: c_float, causal: c_int) -> c_int;
     pub fn lumen_attn_prefill_f32(cache: *mut lumen_kv_cache, rope: *mut lumen_rope, q_dev: *const c_float, k_dev: *const c_float, v_dev: *const c_float, out_dev: *mut c_float, s: c_int, h: c_int, scale: c_float, causal: c_int) -> c_int;
     pub fn lumen_llama_create(ctx: *mut lumen_ctx, cfg: *const lumen_llama_config, out: *mut *mut lumen_llama) -> c_int;
@@ -109,6 +121,7 @@ extern "C" {
     pub fn lumen_llama_get_config(model: *const lumen_llama, cfg_out: *mut lumen_llama_config) -> c_int;
     pub fn lumen_llama_decode_profile(model: *mut lumen_llama, first_id: c_int, n: c_int, ms_sum_out: *mut f64, count_out: *mut c_int, n_classes: c_int) -> c_int;
     pub fn lumen_llama_set_decode_mode(model: *mut lumen_llama, mode: c_int) -> c_int;
+    pub fn lumen_llama_profile_kernel_name(model: *const lumen_llama, kernel_class: c_int, buf: *mut c_char, buf_len: c_int) -> c_int;
     pub fn lumen_llama_set_handover(model: *mut lumen_llama, enable: c_int, spin_limit: i64, pre_sleep: c_int, poll_delay: c_int, poll_gap: c_int) -> c_int;
     pub fn lumen_llama_get_decode_mode(model: *const lumen_llama, mode_out: *mut c_int) -> c_int;
     pub fn lumen_llama_reset(model: *mut lumen_llama) -> c_int;

@@ -225,3 +225,59 @@ def test_legacy_llama_kv_cache_update_and_view():
     with pytest.raises(_lib.LumenError) as e:
         c.update(dev(k), dev(v), 8)  # kv_cache.rs:33-36
     assert e.value.status == _lib.ERR_KV_OVERFLOW
+
+
+@pytest.mark.parametrize("h,h_kv,d,hidden,max_seq,prefill,steps,bf16", [
+    (32, 4, 64, 2048, 2048, 0, 6, False), (8, 2, 64, 512, 700, 509, 6, False), (16, 8, 128, 1024, 512, 100, 4, False),
+    (4, 4, 32, 128, 64, 3, 4, False), (16, 2, 64, 1024, 4096, 4000, 3, True)])
+def test_fused_qkv_rope_append_then_prerotated_attention_equals_the_unfused_step(h, h_kv, d, hidden, max_seq, prefill,
+                                                                                 steps, bf16):
+    """lumen_qkv_rope_append_f32 + lumen_attn_decode_prerotated_f32 against the checker's leaves: RMSNorm, the
+    three projections, then the decode attention core (which rotates, appends and attends).  The new cache row
+    and the output agree to the rounding of the projection sums; the length advances in the second call only;
+    overflow and RoPE range are refused before anything is written."""
+    rng = np.random.default_rng(h * 131 + d + prefill)
+    scale = 1.0 / math.sqrt(d)
+    rope = RotaryEmbedding(d, max_seq, 10000.0)
+    cos, sin = lo.rope_table(d, max_seq, 10000.0)
+    g, o = KVCacheInner(1, h_kv, max_seq, d), lo.KVCache(1, h_kv, max_seq, d)
+    if prefill:
+        q = f32(rng.normal(0, 1, (1, prefill, h, d)))
+        k = f32(rng.normal(0, 1, (1, prefill, h_kv, d)))
+        v = f32(rng.normal(0, 1, (1, prefill, h_kv, d)))
+        gpu_prefill(g, rope, q, k, v, scale)
+        lo.attn_prefill(o, q, k, v, cos, sin, scale)
+    W = f32(rng.normal(0, 0.05, ((h + 2 * h_kv) * d, hidden)))
+    Wh = lo.f32_to_bf16(W) if bf16 else W
+    Wref = lo.bf16_to_f32(Wh) if bf16 else W
+    gains = f32(rng.normal(1, 0.2, hidden))
+    Wd, gd = dev(Wh), dev(gains)
+    tol = 3e-5
+    for t in range(steps):
+        x = f32(rng.normal(0, 1, hidden))
+        xd = dev(x)
+        q_rot, out = Tensor.empty((h * d,)), Tensor.empty((h * d,))
+        check(lib.lumen_qkv_rope_append_f32(g.handle, rope.handle, Wd.ptr, int(bf16), xd.ptr, hidden, gd.ptr, 1e-5, q_rot.ptr, h))
+        assert g.len == prefill + t  # not advanced yet
+        check(lib.lumen_attn_decode_prerotated_f32(g.handle, q_rot.ptr, out.ptr, h, scale))
+        assert g.len == prefill + t + 1
+        xn = lo.rmsnorm(x[None], gains, 1e-5)[0]
+        qkv = lo.gemv(Wref, xn)
+        q3 = qkv[:h * d].reshape(1, h, d)
+        k3 = qkv[h * d:(h + h_kv) * d].reshape(1, h_kv, d)
+        v3 = qkv[(h + h_kv) * d:].reshape(1, h_kv, d)
+        rc, ref = lo.attn_decode(o, f32(q3), f32(k3), f32(v3), cos, sin, scale)
+        assert rc == lo.LO_OK
+        assert max_rel(out.data(), ref.reshape(-1)) <= tol, t
+        n = o.len
+        assert max_rel(g.k[:, :, n - 1], o.k[:, :, n - 1]) <= tol and max_rel(g.v[:, :, n - 1], o.v[:, :, n - 1]) <= tol
+        q_ref = np.stack([lo.rope_1token_copy(f32(q3[0, i]), cos, sin, n - 1)[1] for i in range(h)])
+        assert max_rel(q_rot.data().reshape(h, d), q_ref) <= tol
+    if prefill + steps < max_seq and max_seq <= 64:
+        g.len = max_seq  # full cache: self_attention.rs:144-149
+        with pytest.raises(_lib.LumenError) as e:
+            check(lib.lumen_qkv_rope_append_f32(g.handle, rope.handle, Wd.ptr, int(bf16), xd.ptr, hidden, gd.ptr, 1e-5, q_rot.ptr, h))
+        assert e.value.status == _lib.ERR_KV_OVERFLOW
+        with pytest.raises(_lib.LumenError) as e:
+            check(lib.lumen_attn_decode_prerotated_f32(g.handle, q_rot.ptr, out.ptr, h, scale))
+        assert e.value.status == _lib.ERR_KV_OVERFLOW

@@ -131,9 +131,12 @@ def test_greedy_generation_on_device_matches_oracle_loop():
     assert np.array_equal(gpu.decode_greedy(first, n), ids)
 
 
-def test_layered_operator_path_matches_fused_path_and_oracle():
+@pytest.mark.parametrize("fused_ops", [True, False], ids=["fused-operators", "leaf-operators"])
+def test_layered_operator_path_matches_fused_path_and_oracle(fused_ops):
+    """LlamaModel::forward composed operator by operator: one call per reference leaf, or -- single tokens -- the
+    fused operators (five launches per layer); both against the checker and the model-level path."""
     params = synth.make_params(TINY, seed=14, std=0.1, gains_one=False)
-    layered = LayeredLlamaModel(TINY, params)
+    layered = LayeredLlamaModel(TINY, params, fused=fused_ops)
     ora = lo.Llama(TINY, params)
     fused = LlamaModel(TINY)
     fused.load_params(params)

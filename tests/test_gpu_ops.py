@@ -7,6 +7,7 @@ import numpy as np
 import pytest
 
 from lumen_amd import _lib, ops
+from lumen_amd._lib import check, lib
 from lumen_amd.autograd import Tensor
 from lumen_amd.layers import Embedding, Linear, RMSNorm, RotaryEmbedding, SiLU
 from oracle import lumen_oracle as lo
@@ -202,3 +203,52 @@ def test_rope_tables_and_rotation_bit_exact(dim, max_seq, theta):
     with pytest.raises(_lib.LumenError) as e:
         rope.rope_1token_copy(dev(src), dst, max_seq)
     assert e.value.status == _lib.ERR_ROPE_RANGE
+
+
+@pytest.mark.parametrize("N,K,bf16", [(2048, 2048, False), (2048, 5632, False), (64, 512, False), (100, 264, False),
+                                      (512, 1024, True), (30, 4096, True)])
+def test_fused_product_equals_its_leaves(N, K, bf16):
+    """lumen_gemv_fused_f32: RMSNorm on the way in and the residual / SwiGLU epilogues against the leaf operators
+    of the checker (rms_norm.rs:45-58, matmul.rs:42-69, arithmetic.rs:48-51, llama.rs:59-65); gate/up rows are
+    interleaved on the device with lumen_interleave_rows."""
+    rng = np.random.default_rng(N * 7 + K)
+    ctx = dev(np.zeros(4, np.float32)).ctx
+    x = f32(rng.normal(0, 1, K))
+    g = f32(rng.normal(1, 0.2, K))
+    res = f32(rng.normal(0, 1, N))
+    W = f32(rng.normal(0, 0.05, (N, K)))
+    Wh = lo.f32_to_bf16(W) if bf16 else W
+    Wref = lo.bf16_to_f32(Wh) if bf16 else W
+    xd, gd, rd, Wd = dev(x), dev(g), dev(res), dev(Wh)
+    eps = 1e-5
+    xn = lo.rmsnorm(x[None], g, eps)[0]
+    y = Tensor.empty((N,))
+
+    def run(norm, epi, residual, out, w=Wd, n=N):
+        check(lib.lumen_gemv_fused_f32(ctx.handle, w.ptr, int(bf16), xd.ptr, out.ptr, n, K, gd.ptr if norm else None, eps,
+                                       epi, residual.ptr if residual is not None else None))
+        return out.data()
+
+    assert max_rel(run(False, _lib.GEMV_EPI_STORE, None, y), lo.gemv(Wref, x)) <= 1e-5
+    assert max_rel(run(True, _lib.GEMV_EPI_STORE, None, y), lo.gemv(Wref, xn)) <= 1e-5
+    assert max_rel(run(False, _lib.GEMV_EPI_RESIDUAL, rd, y), lo.add(res, lo.gemv(Wref, x))) <= 1e-5
+    assert max_rel(run(True, _lib.GEMV_EPI_RESIDUAL, rd, y), lo.add(res, lo.gemv(Wref, xn))) <= 1e-5
+    if N % 2 == 0:
+        # SwiGLU: gate = first N/2 rows, up = the rest, interleaved on the device
+        half = N // 2
+        gate, up = Wh[:half], Wh[half:]
+        gdv, udv = dev(gate), dev(up)
+        Wi = Tensor.empty((N, K), Wh.dtype)
+        check(lib.lumen_interleave_rows(ctx.handle, gdv.ptr, udv.ptr, Wi.ptr, half, K * Wh.itemsize))
+        inter = Wi.data()
+        assert np.array_equal(inter[0::2], gate) and np.array_equal(inter[1::2], up)
+        act = Tensor.empty((half,))
+        for norm, xin in ((False, x), (True, xn)):
+            ref = lo.mul(lo.silu(lo.gemv(Wref[:half], xin)), lo.gemv(Wref[half:], xin))
+            assert max_rel(run(norm, _lib.GEMV_EPI_SWIGLU, None, act, Wi, N), ref) <= 2e-5
+    with pytest.raises(_lib.LumenError) as e:
+        run(False, _lib.GEMV_EPI_RESIDUAL, None, y)
+    assert e.value.status == _lib.ERR_INVALID
+    with pytest.raises(_lib.LumenError) as e:
+        run(False, 7, None, y)
+    assert e.value.status == _lib.ERR_INVALID
