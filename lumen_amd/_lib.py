@@ -7,7 +7,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "liblumen_hip.so")
+# LUMEN_HIP_LIB: another build of the same library (e.g. the stage-time build of the Makefile)
+LIB_PATH = os.environ.get("LUMEN_HIP_LIB") or os.path.join(_HERE, "lib", "liblumen_hip.so")
 
 OK, ERR_SHAPE, ERR_KV_OVERFLOW, ERR_ROPE_RANGE, ERR_EMBED_OOB, ERR_CACHE_COUNT, ERR_INVALID, ERR_HIP, \
     ERR_NO_DEVICE, ERR_UNSUPPORTED = range(10)
