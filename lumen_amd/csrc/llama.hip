@@ -76,6 +76,13 @@ static int dmalloc(lumen_llama *m, void **p, size_t bytes) {
     return LUMEN_OK;
 }
 
+// a weight matrix: zero until a parameter is set, so that a file that lacks a tensor gives defined results
+static int dmalloc_weight(lumen_llama *m, void **p, size_t bytes) {
+    LUMEN_TRY(dmalloc(m, p, bytes));
+    HIP_TRY(hipMemsetAsync(*p, 0, bytes ? bytes : 16, m->ctx->stream));
+    return LUMEN_OK;
+}
+
 template <typename T>
 static int dmalloc_t(lumen_llama *m, T **p, size_t count) { return dmalloc(m, (void **)p, count * sizeof(T)); }
 
@@ -127,21 +134,21 @@ extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg,
     m->layers.resize(L);
     int rc = LUMEN_OK;
 #define M_TRY(e) do { rc = (e); if (rc != LUMEN_OK) { lumen_llama_destroy(m); return rc; } } while (0)
-    M_TRY(dmalloc_t(m, &m->embed, (size_t)V * H));
+    M_TRY(dmalloc_weight(m, (void **)&m->embed, (size_t)V * H * sizeof(float)));
     if (cfg->tie_embeddings && !m->bf16) {
         m->lm_head = m->embed;
     } else {
-        M_TRY(dmalloc(m, &m->lm_head, (size_t)V * H * m->esz));
+        M_TRY(dmalloc_weight(m, &m->lm_head, (size_t)V * H * m->esz));
         m->lm_head_owned = true;
     }
     M_TRY(dmalloc_t(m, &m->final_norm, (size_t)H));
     M_TRY(fill_ones(m, m->final_norm, H));  // RMSNorm::new, rms_norm.rs:14-20
     for (int l = 0; l < L; ++l) {
         LayerW &w = m->layers[l];
-        M_TRY(dmalloc(m, &w.wqkv, (size_t)m->qkvd * H * m->esz));
-        M_TRY(dmalloc(m, &w.wo, (size_t)H * m->qd * m->esz));
-        M_TRY(dmalloc(m, &w.wgu, (size_t)2 * I * H * m->esz));
-        M_TRY(dmalloc(m, &w.wdown, (size_t)H * I * m->esz));
+        M_TRY(dmalloc_weight(m, &w.wqkv, (size_t)m->qkvd * H * m->esz));
+        M_TRY(dmalloc_weight(m, &w.wo, (size_t)H * m->qd * m->esz));
+        M_TRY(dmalloc_weight(m, &w.wgu, (size_t)2 * I * H * m->esz));
+        M_TRY(dmalloc_weight(m, &w.wdown, (size_t)H * I * m->esz));
         M_TRY(dmalloc_t(m, &w.in_norm, (size_t)H));
         M_TRY(dmalloc_t(m, &w.post_norm, (size_t)H));
         M_TRY(fill_ones(m, w.in_norm, H));
@@ -560,8 +567,13 @@ static int ensure_decode_graph(lumen_llama *m) {
         return rc;
     }
     if (e != hipSuccess) LUMEN_FAIL(LUMEN_ERR_HIP, "hipStreamEndCapture failed: %s", hipGetErrorString(e));
+    const hipError_t ei = hipGraphInstantiate(&m->graph_exec, g, nullptr, nullptr, 0);
+    if (ei != hipSuccess) {
+        hipGraphDestroy(g);
+        m->graph_exec = nullptr;
+        LUMEN_FAIL(LUMEN_ERR_HIP, "hipGraphInstantiate failed: %s", hipGetErrorString(ei));
+    }
     m->graph = g;
-    HIP_TRY(hipGraphInstantiate(&m->graph_exec, m->graph, nullptr, nullptr, 0));
     return LUMEN_OK;
 }
 

@@ -91,9 +91,9 @@ struct Json {
         while (p < e && *p >= '0' && *p <= '9') v = v * 10 + (uint64_t)(*p++ - '0');
         return p > s;
     }
-    void skip() {  // any value
+    void skip(int depth = 0) {  // any value; nesting beyond 64 levels is refused (no file of this format has it)
         ws();
-        if (p >= e) {
+        if (p >= e || depth > 64) {
             fail = true;
             return;
         }
@@ -108,13 +108,13 @@ struct Json {
                     fail = true;
                     return;
                 }
-                skip();
+                skip(depth + 1);
             } while (!fail && eat(','));
             if (!eat('}')) fail = true;
         } else if (*p == '[') {
             ++p;
             if (eat(']')) return;
-            do skip();
+            do skip(depth + 1);
             while (!fail && eat(','));
             if (!eat(']')) fail = true;
         } else {

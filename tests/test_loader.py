@@ -63,6 +63,16 @@ def test_other_dtypes_and_damaged_files(tmp_path):
     bad.write_bytes(raw[:8] + b"[" + raw[9:])
     with pytest.raises(_lib.LumenError):
         find(bad, "a")
+    # a header whose unknown value nests deeper than any real file: refused, not recursed into without bound;
+    # 40 levels are still read
+    def with_metadata(depth):
+        hdr = ('{"__metadata__":' + "[" * depth + "]" * depth + ',"a":{"dtype":"F32","shape":[1],"data_offsets":[0,4]}}').encode()
+        return struct.pack("<Q", len(hdr)) + hdr + b"\0\0\0\0"
+    bad.write_bytes(with_metadata(40))
+    assert find(bad, "a")[1] == (1,)
+    bad.write_bytes(with_metadata(200000))
+    with pytest.raises(_lib.LumenError):
+        find(bad, "a")
 
 
 @pytest.mark.gpu
@@ -101,6 +111,10 @@ def test_model_loaded_from_a_file_equals_the_model_loaded_tensor_by_tensor(tmp_p
     m3.set_param("lm_head.weight", params["lm_head.weight"])
     assert m3.load_safetensors(pp) == (len(params) - 1, 1)
     assert np.array_equal(m3.forward(ids, all_rows=True), want)
+    # ... and a weight nobody ever set is zero, not whatever the allocation held: all-zero logits here
+    m4 = LlamaModel(CFG)
+    assert m4.load_safetensors(pp) == (len(params) - 1, 1)
+    assert not m4.forward(ids, all_rows=True).any()
 
     # unsupported dtype (loader.rs:67) and element-count mismatch (:44-46)
     ph = tmp_path / "f16.safetensors"
