@@ -315,14 +315,20 @@ int lumen_llama_decode_profile(lumen_llama *model, int first_id, int n, double *
 int lumen_llama_set_decode_mode(lumen_llama *model, int mode);
 /* name of the kernel instance the last lumen_llama_decode_profile launched for a class ("" if none) */
 int lumen_llama_profile_kernel_name(const lumen_llama *model, int kernel_class, char *buf, int buf_len);
-/* While the cache is short (up to 512 rows, 256 for head_dim 128) and the shape allows (no q/k norm, head_dim 64 or
- * 128, n_head * head_dim a multiple of 512), decode attention and the o_proj product of a layer are ONE launch:
- * attention workgroups hand their output to resident o_proj workgroups, whose weights are already in registers,
- * through tagged 8-byte words (no reference counterpart; same results as the two launches it replaces).  Where
- * n_head * head_dim == hidden_size and two weight rows fit a wavefront's registers (hidden 512, 1024 or 2048 in f32, twice
- * that in bf16) the RMSNorm + q|k|v + RoPE product joins the same launch in front, handing q and the new key /
- * value to the attention workgroups the same way.  This call picks the form (enable 0: separate launches,
- * 1: attention + o_proj, 2: q|k|v + attention + o_proj, the default where covered) and sets its waits: spin_limit = polls after which a waiting
+/* Where the shape allows (head_dim 64 or 128, n_head * head_dim a multiple of 512 and at most 4096 values of f32 /
+ * 8192 of bf16 weights per row) and the cache is not too long (up to 16 trips of rows: 4096 rows for head_dim 64, 2048
+ * for 128), decode attention and the o_proj product of a layer are ONE launch: attention workgroups hand their
+ * output to resident o_proj workgroups, whose weights are already in registers, through tagged 8-byte words (no
+ * reference counterpart; same results as the launches it replaces).  Form 2 puts the RMSNorm + q|k|v + RoPE product
+ * in front in the same launch, handing q and the new key / value to the attention workgroups the same way: it needs
+ * two q|k|v weight rows to fit a wavefront's registers (hidden 512, 1024 or 2048 in f32, twice that in bf16) and
+ * n_head * head_dim == hidden (head_dim 128: also 2 * hidden); q/k-norm models (head_dim 128) are served by form 2
+ * only (norm and rotation then happen in the attention workgroups).  Caches of more than two trips of rows are cut
+ * into slices taken by several attention workgroups per head in parallel and folded by a further set of workgroups.
+ * lumen_llama_create switches the chain on where every role is at most one workgroup per compute unit (models up to
+ * ~2048 wide; wider products stream better as launches of their own).  This call picks the form (enable 0: separate
+ * launches, 1: attention + o_proj, 2: q|k|v + attention + o_proj) and sets its waits:
+ * spin_limit = polls after which a waiting
  * workgroup gives up -- the call that finds a wait given up returns LUMEN_ERR_HIP, its results are invalid, every
  * wavefront still exits -- and the pauses, in units of 256 clocks, of the o_proj workgroups before their weight
  * requests, before their first poll and between polls (kept per form; the call sets those of the form in use

@@ -81,7 +81,9 @@ __device__ __forceinline__ unsigned rows_mask(int first, int stride, int end) {
 //   ATTN_SRC_CACHE   q is rotated and cache row pos_new written already (an earlier launch did both);
 //   ATTN_SRC_TAGGED  rotated q, new key and new value arrive as tagged words from other workgroups of THIS launch
 //                    (which also store the row): they are polled for after the first trip of rows is requested, go to
-//                    LDS, and the new row is taken from there.
+//                    LDS, and the new row is taken from there;
+//   ATTN_SRC_TAGGED_RAW  the same words hold the UN-rotated projections (q/k-norm models): ATTN_SRC_RAW with the
+//                    tagged words in the place of the projections in memory.
 //
 // pos_new < 0: the position is not known yet.  The first trip of rows and the query are requested
 // before it is read -- they do not depend on it: a row past the cached ones is only masked later --
@@ -90,12 +92,21 @@ __device__ __forceinline__ unsigned rows_mask(int first, int stride, int end) {
 #define ATTN_SRC_RAW 0
 #define ATTN_SRC_CACHE 1
 #define ATTN_SRC_TAGGED 2
-template <int D, int WAVES, int SRC>
+#define ATTN_SRC_TAGGED_RAW 3
+//
+// SLICED (the chained launch, which may run several workgroups per query head): this workgroup takes the rows
+// [slice * R, (slice + 1) * R), R = 1 << a.slice_shift, a whole number of trips, walked trip by trip.  With `n` =
+// position / R + 1 slices in use, a workgroup of a later slice returns at once; the slice the new token falls
+// into adds the new row; with n == 1 the output is final as in the plain form, else the workgroup leaves its state
+// (ctx[D], m, l) as tagged words in a.part_tagged [head][a.tslices][D + 2] for the workgroup that folds the slices
+// of the head.
+template <int D, int WAVES, int SRC, bool SLICED = false>
 __device__ __forceinline__ bool attn_decode_short(const AttnDecodeArgs &a, int r, int nrep, int hk, int bb, int pos_new,
                                                   int short_rows, float *q_rot, float *k_new,
-                                                  float *v_new, float *sm, float *sl, float *sacc) {
+                                                  float *v_new, float *sm, float *sl, float *sacc, int slice = 0) {
     constexpr int LPR = D / 4, RPW = 64 / LPR, RPI = WAVES * RPW, UB = ShortTrip<D>::loads, THREADS = WAVES * 64;
     constexpr bool PRE = SRC == ATTN_SRC_CACHE;
+    const int row0 = SLICED ? slice << a.slice_shift : 0;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int off = wave * RPW + lane / LPR, c = lane % LPR;
     const int hq = hk * nrep + r;
@@ -111,7 +122,7 @@ __device__ __forceinline__ bool attn_decode_short(const AttnDecodeArgs &a, int r
     v4f kv0[UB], vv0[UB];
 #pragma unroll
     for (int u = 0; u < UB; ++u) {
-        const int j = min(u * RPI + off, a.max_seq - 1);
+        const int j = min(row0 + u * RPI + off, a.max_seq - 1);
         kv0[u] = ld_row<D>(Kb, j, c4);
         vv0[u] = ld_row<D>(Vb, j, c4);
     }
@@ -121,7 +132,10 @@ __device__ __forceinline__ bool attn_decode_short(const AttnDecodeArgs &a, int r
     }
     if (pos_new < 0) pos_new = a.pos_dev ? *a.pos_dev : a.pos_host;
     if (pos_new + 1 > short_rows) return false;
-    const int pos = PRE ? pos_new + 1 : pos_new;  // rows read from the cache
+    const int nact = SLICED ? (pos_new >> a.slice_shift) + 1 : 1;  // slices in use
+    if (SLICED && slice >= nact) return true;
+    const bool owner = !SLICED || slice == nact - 1;  // the new token falls into this slice
+    const int pos = SLICED ? min(PRE ? pos_new + 1 : pos_new, row0 + (1 << a.slice_shift)) : (PRE ? pos_new + 1 : pos_new);  // end of the cached rows read here
     auto get_q = [&]() __attribute__((always_inline)) {
         if (PRE) {
             load_q_scaled<D, 1>(q, a.q + ((size_t)bb * a.hq + hq) * D, c, a.scale);
@@ -136,27 +150,40 @@ __device__ __forceinline__ bool attn_decode_short(const AttnDecodeArgs &a, int r
                 for (int e = 0; e < EPL; ++e) dst[lane * EPL + e] = v[e];
             };
             if (wave == 0) take(q_rot, hq);
-            else if (wave == 1) take(k_new, a.hq + hk);
-            else if (wave == 2) take(v_new, a.hq + a.hkv + hk);
+            else if (wave == 1 && owner) take(k_new, a.hq + hk);
+            else if (wave == 2 && owner) take(v_new, a.hq + a.hkv + hk);
             __syncthreads();
             load_q_scaled<D, 1>(q, q_rot, c, a.scale);
         } else {
             // wavefront 0 takes the query head, wavefront 1 the new key, wavefront 2 copies the new value:
             // lane j holds the pair (j, j + D/2); everything they need from memory is requested at once
             constexpr int HALF = D / 2;
+            constexpr bool WORDS = SRC == ATTN_SRC_TAGGED_RAW;
             const float *cs = a.cos_t + (size_t)pos_new * D, *sn = a.sin_t + (size_t)pos_new * D;
-            if (wave < 2) {
+            auto word = [&](size_t i) __attribute__((always_inline)) {  // one tagged word of q | k | v (batch 1)
+                float v[1];
+                if (!take_tagged<1>(a.qkv_tagged + i, a.tag, a.spin_limit, a.poll_gap, v))
+                    __hip_atomic_store(a.err_dev, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                return v[0];
+            };
+            if (wave == 0 || (wave == 1 && owner)) {
                 const float *src = wave == 0 ? a.q + ((size_t)bb * a.hq + hq) * D : a.k_new + ((size_t)bb * a.hkv + hk) * D;
+                const size_t wbase = (size_t)(wave == 0 ? hq : a.hq + hk) * D;
                 const float *g = wave == 0 ? a.q_norm_w : a.k_norm_w;
                 float x1 = 0.f, x2 = 0.f, cc = 0.f, ss_ = 0.f, g1 = 1.f, g2 = 1.f;
                 if (lane < HALF) {
-                    x1 = src[lane];
-                    x2 = src[lane + HALF];
                     cc = cs[lane];
                     ss_ = sn[lane];
                     if (g) {
                         g1 = g[lane];
                         g2 = g[lane + HALF];
+                    }
+                    if (WORDS) {
+                        x1 = word(wbase + lane);
+                        x2 = word(wbase + lane + HALF);
+                    } else {
+                        x1 = src[lane];
+                        x2 = src[lane + HALF];
                     }
                 }
                 if (g) {  // per-head RMSNorm before the rotation
@@ -177,12 +204,12 @@ __device__ __forceinline__ bool attn_decode_short(const AttnDecodeArgs &a, int r
                     dst[lane] = o1;
                     dst[lane + HALF] = o2;
                 }
-            } else if (wave == 2) {
+            } else if (wave == 2 && owner) {
                 const float *v_src = a.v_new + ((size_t)bb * a.hkv + hk) * D;
-                for (int i = lane; i < D; i += 64) v_new[i] = v_src[i];
+                for (int i = lane; i < D; i += 64) v_new[i] = WORDS ? word((size_t)(a.hq + a.hkv + hk) * D + i) : v_src[i];
             }
             __syncthreads();
-            if (r == 0) {  // self_attention.rs:161-176: rotated k and raw v go to cache row pos_new
+            if (r == 0 && owner) {  // self_attention.rs:161-176: rotated k and raw v go to cache row pos_new
                 for (int i = threadIdx.x; i < D; i += THREADS) {
                     a.k_cache[head_base + (size_t)pos_new * D + i] = k_new[i];
                     a.v_cache[head_base + (size_t)pos_new * D + i] = v_new[i];
@@ -192,9 +219,9 @@ __device__ __forceinline__ bool attn_decode_short(const AttnDecodeArgs &a, int r
         }
         have_q = true;
     };
-    if (!have_q && pos > 0) get_q();
-    attn_batch<D, UB>(st, q[0], kv0, vv0, rows_mask<UB>(off, RPI, pos));
-    for (int base = RPI * UB; base < pos; base += RPI * UB) {
+    if (!have_q && (SLICED || pos > 0)) get_q();
+    attn_batch<D, UB>(st, q[0], kv0, vv0, rows_mask<UB>(row0 + off, RPI, pos));
+    for (int base = row0 + RPI * UB; base < pos; base += RPI * UB) {
         v4f kv[UB], vv[UB];
 #pragma unroll
         for (int u = 0; u < UB; ++u) {  // rows past the end are clamped here and masked in attn_batch
@@ -206,7 +233,7 @@ __device__ __forceinline__ bool attn_decode_short(const AttnDecodeArgs &a, int r
     }
     if (!PRE) {
         if (!have_q) get_q();  // empty cache: the new token attends to itself only
-        if (wave == 0) {       // the new row, from LDS (lane group 0 of wavefront 0)
+        if (wave == 0 && owner) {  // the new row, from LDS (lane group 0 of wavefront 0)
             const v4f kn = *(const v4f *)(k_new + c * 4), vn = *(const v4f *)(v_new + c * 4);
             attn_step<D, 1>(st, q, kn, vn, lane / LPR == 0);
         }
@@ -219,7 +246,14 @@ __device__ __forceinline__ bool attn_decode_short(const AttnDecodeArgs &a, int r
     for (int dd = threadIdx.x; dd < D; dd += THREADS) {
         float mm, ls, cx;
         wave_fold<D, 1, WAVES>(sm, sl, sacc, 0, dd, mm, ls, cx);
-        if (a.defer_merge) {  // the consumer divides
+        if (SLICED && nact > 1) {  // one of several slices: the state travels on
+            unsigned long long *pt = a.part_tagged + (((size_t)bb * a.hq + hq) * a.tslices + slice) * (D + 2);
+            tagged_store(pt + dd, cx, a.tag);
+            if (dd == 0) {
+                tagged_store(pt + D, mm, a.tag);
+                tagged_store(pt + D + 1, ls, a.tag);
+            }
+        } else if (a.defer_merge) {  // the consumer divides
             part0[dd] = cx;
             if (dd == 0) {
                 part0[D] = mm;

@@ -196,6 +196,10 @@ struct AttnDecodeArgs {
     // q, the new key and the new value ARRIVE as tagged words, [hq + 2 hkv, D] rotated (the q|k|v -> attention ->
     // o_proj chain): the cache row of the new token is not read, nothing is rotated or stored here; null everywhere else
     const unsigned long long *qkv_tagged;
+    // the chained launch with several workgroups per query head: slices launched, and where a slice leaves its
+    // state for the workgroup that folds them, [hq][tslices][d + 2] tagged words
+    int tslices, slice_shift;  // (a slice covers 1 << slice_shift rows)
+    unsigned long long *part_tagged;
     unsigned spin_limit;  // polls before a wait for tagged words gives up (then *err_dev = 1)
     int poll_gap;         // pause between polls, units of 256 clocks
     int *err_dev;
@@ -221,14 +225,22 @@ struct AttnOprojArgs {
     int pre_sleep, poll_delay, poll_gap;  // timing of the o_proj workgroups (units of 256 clocks), see attn_oproj.hip
     // With Wqkv set the launch starts one step earlier: its first workgroups are RMSNorm + the q|k|v product + RoPE
     // + KV append (src/models/llama.rs:107, self_attention.rs:106-108, :161-176, :220-227) on `residual` (the layer
-    // input), and q / new key / new value travel to the attention workgroups as tagged words.  Needs N == K.
+    // input), and q / new key / new value travel to the attention workgroups as tagged words -- un-rotated when
+    // attn.q_norm_w / attn.k_norm_w are set (per-head norm, rotation and cache write then happen in the attention role).
     const void *Wqkv;             // [(hq + 2 hkv) * d, N] f32 or bf16 bits, or null
     const float *in_norm_w;       // [N] gains of the input RMSNorm
     float norm_eps;
     unsigned long long *qkv_tagged;  // [(hq + 2 hkv) * d]
+    // Attention workgroups per query head (1 to ATTN_CHAIN_MAX_SLICES): slice s takes the cached rows
+    // [s R, (s + 1) R), R = slice_rows (a power of two, a multiple of attn_decode_trip_rows(d)); with more
+    // than one, hq further workgroups fold the slices of a head (part_tagged [hq][nslices][d + 2]) and hand the
+    // result to the o_proj workgroups.  The position must lie below nslices * slice_rows.
+    int nslices, slice_rows;
+    unsigned long long *part_tagged;
 };
+#define ATTN_CHAIN_MAX_SLICES 16
 bool attn_oproj_supported(int hq, int hkv, int d, int N, int K, int w_bf16);
-bool qkv_attn_oproj_supported(int hq, int hkv, int d, int N, int K, int w_bf16);
+bool qkv_attn_oproj_supported(int hq, int hkv, int d, int N, int K, int w_bf16, int qk_norm);
 int launch_attn_oproj(lumen_ctx *ctx, const AttnOprojArgs &a);
 
 struct AttnPrefillArgs {

@@ -58,6 +58,10 @@ struct lumen_llama {
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
     int graph_expect_short = 0;            // the hint the captured attention launches carry
+    int graph_slices = 0;                  // ... and the slices of their chained launch
+    int chain_max_slices = 8;                      // caches beyond that many slices take separate launches
+    int chain_slice_trips = 0;                     // > 0: trips per slice fixed (measurements), else chosen by length
+    unsigned long long *part_tagged = nullptr;     // [Hq][ATTN_CHAIN_MAX_SLICES][D + 2]
     int decode_mode = LUMEN_DECODE_GRAPH;
     float *amax_val = nullptr;
     int *amax_idx = nullptr;
@@ -202,16 +206,26 @@ extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg,
                      cfg->max_seq_len <= m->nsplit * attn_decode_trip_rows(D) && fold_bytes <= ((size_t)64 << 20);
     M_TRY(dmalloc_t(m, &m->part, attn_decode_part_floats(1, Hq, D, m->nsplit)));
     M_TRY(dmalloc_t(m, &m->counters, (size_t)Hq));
-    // (q/k-norm models rotate inside the attention kernel: the chain wants a rotated q and a written cache row)
-    m->chain_ao = (cfg->qk_norm || !attn_oproj_supported(Hq, Hkv, D, H, m->qd, m->bf16)) ? 0
-                  : qkv_attn_oproj_supported(Hq, Hkv, D, H, m->qd, m->bf16)              ? 2
-                                                                                         : 1;
+    // (q/k-norm models rotate inside the attention role: only the three-role form serves them)
+    m->chain_ao = qkv_attn_oproj_supported(Hq, Hkv, D, H, m->qd, m->bf16, cfg->qk_norm)                 ? 2
+                  : (!cfg->qk_norm && attn_oproj_supported(Hq, Hkv, D, H, m->qd, m->bf16)) ? 1
+                                                                                           : 0;
+    // The chain pays where its products are latency: every role at most one workgroup per compute unit (hidden and
+    // q|k|v rows up to ~2048-4096).  Larger products stream better as launches of their own (Llama-2-7B shape: 2.73
+    // against 2.95 ms per token); lumen_llama_set_handover can still switch the chain on.
+    if (m->chain_ao == 2 && m->qkvd / 16 > ctx->num_cus) m->chain_ao = cfg->qk_norm ? 0 : 1;
+    if (m->chain_ao && (H + 7) / 8 > ctx->num_cus) m->chain_ao = 0;
+    // the o_proj workgroups hold their weight requests back until q has changed hands, which takes longer the more
+    // q|k|v weights stream in front (measured optima: 47 at 21 MB, 40-43 at 17 MB)
+    m->chain_pre[2] = 26 + (int)((size_t)m->qkvd * H * m->esz / 1000000);
     M_TRY(dmalloc_t(m, &m->x_tagged, (size_t)m->qd));
     M_TRY(dmalloc_t(m, &m->qkv_tagged, (size_t)m->qkvd));
+    M_TRY(dmalloc_t(m, &m->part_tagged, (size_t)Hq * ATTN_CHAIN_MAX_SLICES * (D + 2)));
     M_TRY(dmalloc_t(m, &m->d_step, 4));
     M_TRY(dmalloc_t(m, &m->d_err, 4));
     if (hipMemsetAsync(m->x_tagged, 0, sizeof(unsigned long long) * m->qd, ctx->stream) != hipSuccess ||
         hipMemsetAsync(m->qkv_tagged, 0, sizeof(unsigned long long) * m->qkvd, ctx->stream) != hipSuccess ||
+        hipMemsetAsync(m->part_tagged, 0, sizeof(unsigned long long) * Hq * ATTN_CHAIN_MAX_SLICES * (D + 2), ctx->stream) != hipSuccess ||
         hipMemsetAsync(m->d_step, 0, 4 * sizeof(unsigned), ctx->stream) != hipSuccess ||
         hipMemsetAsync(m->d_err, 0, 4 * sizeof(int), ctx->stream) != hipSuccess) {
         lumen_llama_destroy(m);
@@ -439,7 +453,32 @@ struct StepProbe {  // brackets every launch with a HIP event pair when profilin
 
 // Is the cache short enough for the one-workgroup-per-head form of decode attention?  A hint for the
 // kernel (it starts that form before it has read the position); a wrong one only costs time.
-static int expect_short_cache(const lumen_llama *m) { return m->len + 1 <= (m->D >= 128 ? 256 : 512); }
+static int expect_short_cache(const lumen_llama *m) { return m->len + 1 <= attn_decode_short_rows(m->D); }
+
+// Attention workgroups per query head of the chained launch for the step at the current length, and the rows each
+// takes.  Up to two trips of rows one workgroup walks them in turn (a second trip costs what handing a slice's
+// state on would); up to four trips the slices are one trip each, beyond that two -- more, shorter slices mean more
+// workgroups than the chip holds at once.  The count is rounded up to a power of two so that a captured step
+// serves a range of lengths.  0: the cache is too long for the chain (or the model has none): separate launches.
+static int chain_slices(const lumen_llama *m, int *slice_rows_out = nullptr) {
+    if (!m->chain_ao) return 0;
+    const int T = attn_decode_trip_rows(m->D);
+    const int trips = m->len / T + 1;
+    int per = trips <= 2 ? 2 : trips <= 4 ? 1 : 2;
+    if (m->chain_slice_trips > 0) per = m->chain_slice_trips;
+    const int need = trips <= 2 && m->chain_slice_trips <= 0 ? 1 : (trips + per - 1) / per;
+    int s = 1;
+    while (s < need) s *= 2;
+    if (slice_rows_out) *slice_rows_out = per * T;
+    return s <= m->chain_max_slices ? s : 0;
+}
+
+// what a captured step depends on: slices and rows per slice
+static int chain_plan_key(const lumen_llama *m) {
+    int rows = 0;
+    const int s = chain_slices(m, &rows);
+    return s ? s * 65536 + rows : 0;
+}
 
 static int enqueue_decode_step(lumen_llama *m, StepProbe *pr = nullptr) {
     StepProbe none;
@@ -462,7 +501,9 @@ static int enqueue_decode_step(lumen_llama *m, StepProbe *pr = nullptr) {
             g.k_cache = m->k_slab + m->cache_stride * l; g.v_cache = m->v_slab + m->cache_stride * l;
             g.hq = c.num_attention_heads; g.hkv = c.num_key_value_heads; g.D = m->D; g.max_seq = c.max_seq_len;
         }
-        const bool chain_short = m->chain_ao && expect_short_cache(m);
+        int slice_rows = 0;
+        const int slices = chain_slices(m, &slice_rows);
+        const bool chain_short = slices > 0;
         const bool chain_qkv = chain_short && m->chain_ao > 1;
         if (!chain_qkv) {
             pr->before(KC_QKV);
@@ -490,6 +531,8 @@ static int enqueue_decode_step(lumen_llama *m, StepProbe *pr = nullptr) {
             f.tag_mul = (unsigned)c.num_hidden_layers; f.tag_add = (unsigned)l + 1u;
             f.err_dev = m->d_err; f.spin_limit = m->spin_limit;
             f.pre_sleep = m->chain_pre[m->chain_ao]; f.poll_delay = m->chain_delay[m->chain_ao]; f.poll_gap = m->chain_gap[m->chain_ao];
+            if (slices > 1) f.poll_delay += 12;  // (the fold of the slices is one more hand-over in front of o_proj)
+            f.nslices = slices; f.slice_rows = slice_rows; f.part_tagged = m->part_tagged;
             if (chain_qkv) {
                 f.Wqkv = w.wqkv; f.in_norm_w = w.in_norm; f.norm_eps = c.rms_norm_eps; f.qkv_tagged = m->qkv_tagged;
             }
@@ -546,7 +589,7 @@ static int enqueue_decode_step(lumen_llama *m, StepProbe *pr = nullptr) {
 
 static int ensure_decode_graph(lumen_llama *m) {
     if (m->decode_mode != LUMEN_DECODE_GRAPH) return LUMEN_OK;
-    if (m->graph_exec && m->graph_expect_short != expect_short_cache(m)) {
+    if (m->graph_exec && (m->graph_expect_short != expect_short_cache(m) || m->graph_slices != chain_plan_key(m))) {
         // the captured attention launches carry the hint for the other side of the boundary
         HIP_TRY(hipStreamSynchronize(m->ctx->stream));
         hipGraphExecDestroy(m->graph_exec);
@@ -556,6 +599,7 @@ static int ensure_decode_graph(lumen_llama *m) {
     }
     if (m->graph_exec) return LUMEN_OK;
     m->graph_expect_short = expect_short_cache(m);
+    m->graph_slices = chain_plan_key(m);
     hipStream_t s = m->ctx->stream;
     HIP_TRY(hipStreamSynchronize(s));
     HIP_TRY(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
@@ -597,11 +641,11 @@ extern "C" int lumen_llama_set_decode_mode(lumen_llama *m, int mode) {
 
 extern "C" int lumen_llama_set_handover(lumen_llama *m, int enable, int64_t spin_limit, int pre_sleep, int poll_delay, int poll_gap) {
     if (!m) LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_set_handover: null model");
-    if (enable > 0 && (m->cfg.qk_norm || !attn_oproj_supported(m->cfg.num_attention_heads, m->cfg.num_key_value_heads, m->D,
-                                                               m->cfg.hidden_size, m->qd, m->bf16)))
+    if (enable == 1 && (m->cfg.qk_norm || !attn_oproj_supported(m->cfg.num_attention_heads, m->cfg.num_key_value_heads, m->D,
+                                                                m->cfg.hidden_size, m->qd, m->bf16)))
         LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "the attention -> o_proj launch does not cover this model shape");
     if (enable > 1 && !qkv_attn_oproj_supported(m->cfg.num_attention_heads, m->cfg.num_key_value_heads, m->D, m->cfg.hidden_size,
-                                                m->qd, m->bf16))
+                                                m->qd, m->bf16, m->cfg.qk_norm))
         LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "the q|k|v -> attention -> o_proj launch does not cover this model shape");
     if (enable >= 0) m->chain_ao = enable > 2 ? 2 : enable;
     if (spin_limit >= 0) m->spin_limit = spin_limit > 0xffffffffLL ? 0xffffffffu : (unsigned)spin_limit;

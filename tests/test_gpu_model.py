@@ -329,15 +329,23 @@ CHAIN = dict(vocab_size=1200, hidden_size=512, intermediate_size=1408, num_hidde
                                             (dict(hidden_size=2048, num_attention_heads=16, num_key_value_heads=4,
                                                   intermediate_size=512, num_hidden_layers=2), False),
                                             (dict(hidden_size=2048, num_attention_heads=32, num_key_value_heads=4,
-                                                  intermediate_size=512, num_hidden_layers=2), True)],
+                                                  intermediate_size=512, num_hidden_layers=2), True),
+                                            (dict(hidden_size=512, num_attention_heads=8, num_key_value_heads=4, head_dim=128,
+                                                  qk_norm=True, tie_embeddings=True, rope_theta=1.0e6, rms_norm_eps=1e-6), False),
+                                            (dict(hidden_size=1024, num_attention_heads=8, num_key_value_heads=2, head_dim=128,
+                                                  qk_norm=True, intermediate_size=1024, num_hidden_layers=2), True),
+                                            (dict(hidden_size=512, num_attention_heads=8, num_key_value_heads=8, head_dim=128,
+                                                  intermediate_size=1024, num_hidden_layers=2), False)],
                          ids=["d64-nrep4", "d64-mha", "d128-nrep2", "d64-nrep8-bf16", "d128-nrep4-h2048",
-                              "d64-nrep8-h2048-bf16"])
+                              "d64-nrep8-h2048-bf16", "qwen-d128-nrep2-wide", "qwen-d128-nrep4-bf16", "d128-mha-wide"])
 def test_chained_launches_equal_the_separate_launches_they_replace(cfg_extra, bf16):
     """Short caches: decode attention and o_proj run as one launch whose attention workgroups hand their output to
     the o_proj workgroups through tagged words (form 1), with the RMSNorm + q|k|v + RoPE product in front handing q
     and the new row to the attention workgroups the same way (form 2).  Same steps with separate launches (form 0): the attention arithmetic is the same code, so
     logits agree to rounding of the sums; every form is held to the checker; the cache crosses a trip boundary
-    (256 rows, 128 for head_dim 128) on the way."""
+    (256 rows, 128 for head_dim 128) on the way.  q/k-norm models (head_dim 128) take form 2 with un-rotated
+    projections handed over -- norm, rotation and cache write happen in the attention workgroups; o_proj rows may be
+    twice as long as the q|k|v rows (n_head * head_dim = 2 * hidden)."""
     cfg = dict(CHAIN)
     cfg.update(cfg_extra)
     tol = 2e-2 if bf16 else 1e-4
@@ -346,6 +354,11 @@ def test_chained_launches_equal_the_separate_launches_they_replace(cfg_extra, bf
     ids = synth.make_tokens(n_prompt, cfg["vocab_size"], seed=51)
     out = {}
     for enable in (2, 1, 0):
+        if enable == 1 and cfg.get("qk_norm"):  # form 1 wants a rotated q from an earlier launch: not with q/k norm
+            with pytest.raises(_lib.LumenError) as e:
+                gpu.set_handover(enable=1)
+            assert e.value.status == _lib.ERR_UNSUPPORTED
+            continue
         gpu.set_handover(enable=enable)
         gpu.reset_kv_caches()
         ora.reset()
@@ -380,12 +393,14 @@ def test_attention_oproj_launch_gives_up_a_wait_that_cannot_end_in_time_and_says
     _, ref = ora.forward(ids)
     assert max_rel(last, ref[-1]) <= 1e-4
     _greedy_call_checked(gpu, ora, lo.argmax(ref[-1]), 12, 1e-4)
-    with pytest.raises(_lib.LumenError) as e:  # a q/k-norm model rotates inside the attention kernel: not covered
-        build(TINY_QWEN, seed=1)[0].set_handover(enable=1)
-    assert e.value.status == _lib.ERR_UNSUPPORTED
-    wide = build(dict(CHAIN, head_dim=128, num_hidden_layers=1), seed=2)[0]  # n_head * head_dim = 2 * hidden
+    for enable in (1, 2):  # a q/k-norm model with head_dim 64: no form covers it
+        with pytest.raises(_lib.LumenError) as e:
+            build(TINY_QWEN, seed=1)[0].set_handover(enable=enable)
+        assert e.value.status == _lib.ERR_UNSUPPORTED
+    # n_head * head_dim = 2 * hidden with head_dim 64
+    wide = build(dict(CHAIN, num_attention_heads=16, num_key_value_heads=4, head_dim=64, num_hidden_layers=1), seed=2)[0]
     wide.set_handover(enable=1)
-    with pytest.raises(_lib.LumenError) as e:  # the q|k|v role shares the row length of o_proj
+    with pytest.raises(_lib.LumenError) as e:  # o_proj rows twice as long as the q|k|v rows: head_dim 128 only
         wide.set_handover(enable=2)
     assert e.value.status == _lib.ERR_UNSUPPORTED
 
