@@ -301,7 +301,7 @@ int lumen_llama_get_config(const lumen_llama *model, lumen_llama_config *cfg_out
  * kernel, every launch bracketed by HIP events on the ctx stream.  Classes:
  * 0 embedding, 1 norm+q|k|v GEMV, 2 decode attention, 3 o_proj GEMV, 4 norm+gate|up
  * GEMV, 5 down GEMV, 6 norm+lm_head GEMV, 7 argmax, 8 decode attention + o_proj in one launch
- * (short caches).  ms_sum_out / count_out [n_classes >= 9]. */
+ * (short caches), 9 gate|up + down in one launch (narrow models).  ms_sum_out / count_out [n_classes >= 10]. */
 int lumen_llama_decode_profile(lumen_llama *model, int first_id, int n, double *ms_sum_out,
                                int *count_out, int n_classes);
 /* how S == 1 steps are issued (no reference counterpart; the results are the same):

@@ -243,6 +243,27 @@ bool attn_oproj_supported(int hq, int hkv, int d, int N, int K, int w_bf16);
 bool qkv_attn_oproj_supported(int hq, int hkv, int d, int N, int K, int w_bf16, int qk_norm);
 int launch_attn_oproj(lumen_ctx *ctx, const AttnOprojArgs &a);
 
+// RMSNorm + gate|up + SwiGLU and down + residual chained inside ONE launch (mlp_chain.hip); act travels between the
+// roles as tagged words.
+struct MlpChainArgs {
+    const void *Wgu;     // [2 I, N] gate / up rows interleaved, f32 or bf16 bits
+    const float *h;      // [N] layer-internal input: normalised for gate|up, added to the down product
+    const float *norm_w; // [N] gains of the post-attention RMSNorm
+    float eps;
+    const void *Wdown;   // [N, I]
+    float *y;            // [N]
+    int N, I, w_bf16;    // hidden, intermediate
+    unsigned long long *act_tagged;  // [I]
+    const unsigned *step_dev;        // the tag is *step_dev * tag_mul + tag_add
+    unsigned tag_mul, tag_add;
+    int *err_dev;
+    unsigned spin_limit;
+    int pre_sleep, poll_delay, poll_gap;  // timing of the down workgroups (units of 256 clocks)
+};
+bool mlp_chain_supported(int hidden, int inter, int w_bf16);
+int mlp_chain_workgroups(int hidden, int inter);
+int launch_mlp_chain(lumen_ctx *ctx, const MlpChainArgs &a);
+
 struct AttnPrefillArgs {
     const float *q;  // [B, S, Hq, D] un-rotated
     const float *k;  // [B, S, Hkv, D] un-rotated

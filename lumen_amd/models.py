@@ -168,7 +168,7 @@ class LlamaModel:
         return {n: k for k, n in self.DECODE_MODES.items()}[v.value]
 
     KERNEL_CLASSES = ("embedding", "norm_qkv_gemv", "attn_decode", "oproj_gemv", "norm_gateup_gemv", "down_gemv",
-                      "norm_lmhead_gemv", "argmax", "attn_oproj_fused")
+                      "norm_lmhead_gemv", "argmax", "attn_oproj_fused", "mlp_fused")
 
     def profile_kernel_name(self, kernel_class):
         """The kernel instance the last decode_profile launched for a class ('' if none)."""

@@ -335,9 +335,13 @@ CHAIN = dict(vocab_size=1200, hidden_size=512, intermediate_size=1408, num_hidde
                                             (dict(hidden_size=1024, num_attention_heads=8, num_key_value_heads=2, head_dim=128,
                                                   qk_norm=True, intermediate_size=1024, num_hidden_layers=2), True),
                                             (dict(hidden_size=512, num_attention_heads=8, num_key_value_heads=8, head_dim=128,
-                                                  intermediate_size=1024, num_hidden_layers=2), False)],
+                                                  intermediate_size=1024, num_hidden_layers=2), False),
+                                            (dict(intermediate_size=3072), False),
+                                            (dict(hidden_size=1024, num_attention_heads=16, num_key_value_heads=4,
+                                                  intermediate_size=2048, num_hidden_layers=2), True)],
                          ids=["d64-nrep4", "d64-mha", "d128-nrep2", "d64-nrep8-bf16", "d128-nrep4-h2048",
-                              "d64-nrep8-h2048-bf16", "qwen-d128-nrep2-wide", "qwen-d128-nrep4-bf16", "d128-mha-wide"])
+                              "d64-nrep8-h2048-bf16", "qwen-d128-nrep2-wide", "qwen-d128-nrep4-bf16", "d128-mha-wide", "mlp-chain-3072",
+                              "mlp-chain-2048-bf16"])
 def test_chained_launches_equal_the_separate_launches_they_replace(cfg_extra, bf16):
     """Short caches: decode attention and o_proj run as one launch whose attention workgroups hand their output to
     the o_proj workgroups through tagged words (form 1), with the RMSNorm + q|k|v + RoPE product in front handing q
@@ -345,7 +349,9 @@ def test_chained_launches_equal_the_separate_launches_they_replace(cfg_extra, bf
     logits agree to rounding of the sums; every form is held to the checker; the cache crosses a trip boundary
     (256 rows, 128 for head_dim 128) on the way.  q/k-norm models (head_dim 128) take form 2 with un-rotated
     projections handed over -- norm, rotation and cache write happen in the attention workgroups; o_proj rows may be
-    twice as long as the q|k|v rows (n_head * head_dim = 2 * hidden)."""
+    twice as long as the q|k|v rows (n_head * head_dim = 2 * hidden).  Where the intermediate size allows (a
+    multiple of 1024 values of f32 / 2048 of bf16 weights up to 16 loads per lane) forms 1 and 2 also run gate|up and
+    down as one launch (act handed over as tagged words); form 0 takes that apart as well."""
     cfg = dict(CHAIN)
     cfg.update(cfg_extra)
     tol = 2e-2 if bf16 else 1e-4
