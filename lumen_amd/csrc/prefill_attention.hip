@@ -288,7 +288,7 @@ static int launch_fa_d(lumen_ctx *ctx, const AttnPrefillArgs &a) {
 
 // Worth it from a few hundred positions on: below that the tile loop of the few workgroups is
 // longer than the row loop of one workgroup per position.
-bool attn_prefill_mfma_supported(const AttnPrefillArgs &a) { return (a.d == 64 || a.d == 128) && a.s >= 192; }
+bool attn_prefill_mfma_supported(const AttnPrefillArgs &a) { return (a.d == 64 || a.d == 128) && a.s >= 96; }
 
 int launch_attn_prefill_mfma(lumen_ctx *ctx, const AttnPrefillArgs &a) {
     if (a.d == 64) return launch_fa_d<64>(ctx, a);
