@@ -38,6 +38,11 @@ def main():
     ap.add_argument("--max-seq", type=int, default=2048,
                     help="rows of the static KV cache (2048: the headline configuration; 4096 with --prompt 3968 "
                          "--steps 32 is the long-context configuration)")
+    ap.add_argument("--model", choices=["tinyllama-1.1b", "qwen3-0.6b", "llama2-7b-bf16"], default="tinyllama-1.1b",
+                    help="shape of the random-init model: the headline configuration (default); the Qwen3-0.6B shape "
+                         "(q/k norm, head_dim 128, tied embeddings: use --prompt 256 --steps 80 --max-seq 1024); the "
+                         "Llama-2-7B shape with bf16 weights (--prompt 512 --steps 40 --max-seq 1024).  The bench line "
+                         "the driver reads is the default one; the others carry no cpu_baseline")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--mode", choices=["graph", "eager"], default="graph",
                     help="how decode steps are issued: a HIP graph replay per token (default) or kernel by kernel "
@@ -67,7 +72,12 @@ def main():
     from lumen_amd import _lib, synth
     from lumen_amd.models import LlamaModel
 
-    cfg = dict(synth.TINYLLAMA_1B, max_seq_len=args.max_seq)
+    base = {"tinyllama-1.1b": synth.TINYLLAMA_1B, "qwen3-0.6b": synth.QWEN3_0P6B, "llama2-7b-bf16": synth.LLAMA2_7B}[args.model]
+    cfg = dict(base, max_seq_len=args.max_seq)
+    headline = args.model == "tinyllama-1.1b"
+    if not headline:
+        args.no_cpu_baseline = True
+    w_bf16 = cfg.get("weight_dtype") == "bf16"
     need = args.prompt + args.warmup + 3 * args.steps + 8
     if need > cfg["max_seq_len"]:
         sys.exit("bench.py: prompt + warmup + 3*steps = %d exceeds max_seq_len %d" % (need, cfg["max_seq_len"]))
@@ -78,6 +88,8 @@ def main():
     keep_host = not args.no_cpu_baseline
     params = {}
     for name, a in synth.iter_params(cfg, seed=0):
+        if w_bf16 and a.ndim == 2 and "embed" not in name:
+            a = synth.bf16_round(a)  # bf16-stored weights: the values the reference would widen at load time
         model.set_param(name, a)
         if keep_host:
             params[name] = a
@@ -128,8 +140,10 @@ def main():
     event_overhead_ms = max(0.0, (bracketed_ms - eager_ms) / max(n_launches, 1))
     H, I = cfg["hidden_size"], cfg["intermediate_size"]
     # dominant kernel: RMSNorm + gate|up GEMV + SwiGLU, W [2I, H] f32 read once per launch
-    gu_ms, gu_n = prof["norm_gateup_gemv"]
-    gu_bytes = 4.0 * (2.0 * I * H + H + I)
+    esz = 2.0 if w_bf16 else 4.0
+    mlp_fused = prof["mlp_fused"][1] > 0  # narrow models: gate|up and down are one launch
+    gu_ms, gu_n = prof["mlp_fused"] if mlp_fused else prof["norm_gateup_gemv"]
+    gu_bytes = esz * 2.0 * I * H + 4.0 * (H + I) + (esz * H * I + 4.0 * 2 * H if mlp_fused else 0.0)
     gu_raw_ms = gu_ms / max(gu_n, 1)
     gu_avg_ms = gu_raw_ms - event_overhead_ms
     achieved = gu_bytes / (gu_avg_ms * 1e-3) / 1e9
@@ -145,9 +159,9 @@ def main():
     # library's own dispatch reports for [2I, H] (lumen_gemv_kernel_name reads the decision launch_gemv takes), and
     # the committed counter figures are only quoted when they were taken on that same instance.
     names = {k: model.profile_kernel_name(k) for k in prof if prof[k][1]}
-    gu_kernel = names["norm_gateup_gemv"]
-    picked = _lib.gemv_kernel_name(ctx.num_cus, 2 * I, H, cfg.get("weight_dtype", "f32") == "bf16", True, _lib.GEMV_EPI_SWIGLU)
-    if gu_kernel != picked:
+    gu_kernel = names["mlp_fused" if mlp_fused else "norm_gateup_gemv"]
+    picked = _lib.gemv_kernel_name(ctx.num_cus, 2 * I, H, w_bf16, True, _lib.GEMV_EPI_SWIGLU)
+    if not mlp_fused and gu_kernel != picked:
         raise SystemExit("bench: gate|up launched %r but the dispatch reports %r" % (gu_kernel, picked))
     hq, hkv = cfg["num_attention_heads"], cfg["num_key_value_heads"]
     D = cfg.get("head_dim") or H // hq
@@ -158,22 +172,25 @@ def main():
     at_bytes = 2.0 * hkv * mean_len * D * 4  # K and V rows
     at_what = "decode attention"
     if fused_attn:
-        at_bytes += 4.0 * H * hq * D  # + W_o
+        at_bytes += esz * H * hq * D  # + W_o
         at_what = "decode attention + o_proj"
         if prof["norm_qkv_gemv"][1] == 0:  # + W_qkv: the q|k|v product is part of the same launch
-            at_bytes += 4.0 * (hq + 2 * hkv) * D * H
+            at_bytes += esz * (hq + 2 * hkv) * D * H
             at_what = "RMSNorm + q|k|v + RoPE, decode attention, o_proj + residual"
     out = {
         "metric": "batch-1 decode tokens/s", "value": round(tok_s, 2), "unit": "tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "TinyLlama-1.1B-shaped Llama fp32 random-init seed 0, batch 1, prompt %d random ids, "
-                               "greedy decode, static KV cache max_seq_len %d" % (args.prompt, cfg["max_seq_len"]),
+        "config": {"workload": "%s-shaped model %s random-init seed 0, batch 1, prompt %d random ids, "
+                               "greedy decode, static KV cache max_seq_len %d"
+                               % ({"tinyllama-1.1b": "TinyLlama-1.1B", "qwen3-0.6b": "Qwen3-0.6B", "llama2-7b-bf16": "Llama-2-7B"}[args.model],
+                                  "bf16 weights" if w_bf16 else "fp32", args.prompt, cfg["max_seq_len"]),
                    "layers": cfg["num_hidden_layers"], "hidden": H, "heads": "%dq/%dkv" % (hq, hkv), "head_dim": D,
                    "intermediate": I, "vocab": cfg["vocab_size"], "kv_len_during_timing": [len0, len0 + args.steps]},
-        "roofline": {"bound": "hbm", "kernel": "%s (RMSNorm + gate|up GEMV [%d,%d] + SwiGLU)" % (gu_kernel, 2 * I, H),
+        "roofline": {"bound": "hbm", "kernel": "%s (RMSNorm + gate|up GEMV [%d,%d] + SwiGLU%s)"
+                               % (gu_kernel, 2 * I, H, ", down [%d,%d] + residual" % (H, I) if mlp_fused else ""),
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic(gu_kernel),
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic(gu_kernel) if headline else None,
                      "bytes_per_launch": gu_bytes, "avg_launch_us": round(gu_avg_ms * 1e3, 3),
                      "avg_event_bracketed_us": round(gu_raw_ms * 1e3, 3),
                      "event_pair_overhead_us": round(event_overhead_ms * 1e3, 3)},

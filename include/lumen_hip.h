@@ -330,9 +330,10 @@ int lumen_llama_profile_kernel_name(const lumen_llama *model, int kernel_class, 
  * launches, 1: attention + o_proj, 2: q|k|v + attention + o_proj) and sets its waits:
  * spin_limit = polls after which a waiting
  * workgroup gives up -- the call that finds a wait given up returns LUMEN_ERR_HIP, its results are invalid, every
- * wavefront still exits -- and the pauses, in units of 256 clocks, of the o_proj workgroups before their weight
- * requests, before their first poll and between polls (kept per form; the call sets those of the form in use
- * after it).  A negative argument leaves that setting as it is.
+ * wavefront still exits -- and the timing of the o_proj workgroups: pre_sleep, their weight requests go out that
+ * many tenths of a microsecond after the workgroup's start; poll_delay, their first poll follows that many tenths
+ * later; poll_gap, pause between polls in units of 256 clocks (kept per form; the call sets those of the form in
+ * use after it).  A negative argument leaves that setting as it is.
  * enable = 1 or 2 on a shape that form does not cover -> LUMEN_ERR_UNSUPPORTED. */
 int lumen_llama_set_handover(lumen_llama *model, int enable, int64_t spin_limit, int pre_sleep, int poll_delay, int poll_gap);
 int lumen_llama_get_decode_mode(const lumen_llama *model, int *mode_out);

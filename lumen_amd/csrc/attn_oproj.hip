@@ -22,9 +22,12 @@
 // finished) before an o_proj workgroup starts to wait, and every wait ends.  Waits are bounded all the same
 // (spin_limit polls, then *err_dev = 1 and the workgroup goes on with whatever it has), so that every wavefront exits.
 //
-// Timing of the o_proj workgroups (units of 256 clocks, set by the caller): pre_sleep before the weight requests, so
-// that the attention's own few requests enter the memory system first; poll_delay before the first poll and poll_gap
-// between polls, because every poll of the 131072 threads is a trip to memory that the weights compete with.
+// Timing of the o_proj workgroups (set by the caller): the weight requests go out pre_sleep x 0.1 us after the
+// workgroup's start, so that what the roles before ask for enters the memory system first; the first poll follows
+// poll_delay x 0.1 us later, and poll_gap x 256 clocks lie between polls, because every poll of the 131072 threads is a
+// trip to memory that the weights compete with.  The two delays are taken from the 100 MHz wall clock, not from the
+// shader clock: what they are timed against -- the memory system -- does not follow the shader clock either, and
+// with cycle-counted pauses the optimum moved from box to box.
 //
 // q arrives rotated and cache row `pos` is already written (both by the q|k|v product's epilogue) -- or, QKV form,
 // that product is a third role in FRONT of the two:
@@ -103,6 +106,7 @@ __global__ __launch_bounds__(AO_THREADS) void attn_oproj_kernel(const void *Wo_h
     __shared__ float sm[AO_WAVES], sl[AO_WAVES];
     __shared__ __align__(16) float xs[K > KQ ? K : KQ];
     STAGE_T(0);
+    const unsigned long long t_start = wall_clock64();
     const int hq = hq_hot, hkv = hkv_slices_hot & 0xffff, S = hkv_slices_hot >> 16, N = N_hot;  // S: attention slices
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n_o = (N + AO_WAVES - 1) / AO_WAVES;  // o_proj workgroups
@@ -294,7 +298,7 @@ __global__ __launch_bounds__(AO_THREADS) void attn_oproj_kernel(const void *Wo_h
     if (blk < n_o) {
         // ---- o_proj: one row per wavefront, all of its weights requested at once (rows past N: clamped, not stored)
         const int row = blk * AO_WAVES + wave;
-        handover_pause(a_mem.pre_sleep);  // (see the head of the file)
+        handover_pause_until(t_start, a_mem.pre_sleep);  // (see the head of the file)
         v4u raw[NLO];
         {
             const char *rp = (const char *)Wo_hot + ((size_t)min(row, N - 1) * K + (size_t)lane * VEC) * ESZ;
@@ -307,7 +311,7 @@ __global__ __launch_bounds__(AO_THREADS) void attn_oproj_kernel(const void *Wo_h
         const float res = residual[min(row, N - 1)];
         STAGE_T(5);
         // the attention output: this thread's EPT words, polled until every one carries this launch's tag
-        handover_pause(a_mem.poll_delay);
+        handover_pause_until(wall_clock64(), a_mem.poll_delay);
         {
             float v[EPT];
             if (!take_tagged<EPT>(a_mem.x_tagged + (size_t)tid * EPT, tag, a_mem.spin_limit, a_mem.poll_gap, v))

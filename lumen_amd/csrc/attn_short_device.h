@@ -21,6 +21,12 @@ __device__ __forceinline__ unsigned long long tagged_load(const unsigned long lo
 __device__ __forceinline__ void handover_pause(int n) {
     for (int i = 0; i < n; ++i) __builtin_amdgcn_s_sleep(4);  // 256 clocks each
 }
+// Pause until `tenths` x 0.1 us after `t0` (a wall_clock64() reading: 100 MHz, whatever the shader clock does --
+// what the pauses are timed against is the memory system, which does not follow the shader clock either).
+__device__ __forceinline__ void handover_pause_until(unsigned long long t0, int tenths) {
+    const unsigned long long ticks = (unsigned long long)(tenths > 0 ? tenths : 0) * 10u;
+    while (wall_clock64() - t0 < ticks) __builtin_amdgcn_s_sleep(1);
+}
 
 // This thread's EPT words of a tagged vector, polled until every one carries `tag`; false after `limit` polls.
 template <int EPT>

@@ -51,9 +51,10 @@ struct lumen_llama {
     unsigned *d_step = nullptr;
     int *d_err = nullptr;
     unsigned spin_limit = 1u << 22;
-    // timing of the chain's o_proj workgroups (units of 256 clocks), per form: pause before the weight requests,
-    // before the first poll, between polls (measured optima on the 2048-wide model; see attn_oproj.hip)
-    int chain_pre[3] = {0, 10, 47}, chain_delay[3] = {0, 16, 13}, chain_gap[3] = {0, 1, 1};
+    // timing of the chain's o_proj workgroups, per form: weight requests this long after the workgroup's start and
+    // first poll this long after them (units of 0.1 us), pause between polls (units of 256 clocks); measured optima
+    // on the 2048-wide model, see attn_oproj.hip
+    int chain_pre[3] = {0, 11, 55}, chain_delay[3] = {0, 17, 15}, chain_gap[3] = {0, 1, 1};
     std::string prof_names[16];  // per kernel class: the instance the last lumen_llama_decode_profile launched
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
@@ -222,8 +223,8 @@ extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg,
     if (m->chain_ao == 2 && m->qkvd / 16 > ctx->num_cus) m->chain_ao = cfg->qk_norm ? 0 : 1;
     if (m->chain_ao && (H + 7) / 8 > ctx->num_cus) m->chain_ao = 0;
     // the o_proj workgroups hold their weight requests back until q has changed hands, which takes longer the more
-    // q|k|v weights stream in front (measured optima: 47 at 21 MB, 40-43 at 17 MB)
-    m->chain_pre[2] = 26 + (int)((size_t)m->qkvd * H * m->esz / 1000000);
+    // q|k|v weights stream in front (measured optima: 5.4-5.7 us at 21 MB, 4.5-4.7 us at 17 MB)
+    m->chain_pre[2] = 25 + (int)(1.45 * (double)((size_t)m->qkvd * H * m->esz) / 1e6);
     // (every role of the MLP chain at most ... two rounds of workgroups: the products of a narrow model)
     m->chain_mlp = mlp_chain_supported(H, I, m->bf16) && mlp_chain_workgroups(H, I) <= 2 * ctx->num_cus;
     M_TRY(dmalloc_t(m, &m->act_tagged, (size_t)I));

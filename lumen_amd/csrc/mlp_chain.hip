@@ -63,6 +63,7 @@ __global__ __launch_bounds__(MC_THREADS) void mlp_chain_kernel(const void *Wgu_h
     __shared__ __align__(16) float xs[KD > KH ? KD : KH];
     __shared__ float sm[MC_WAVES];
     STAGE_T(0);
+    const unsigned long long t_start = wall_clock64();
     const int N = N_hot;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int ngu = KD / MC_WAVES;
@@ -137,7 +138,7 @@ __global__ __launch_bounds__(MC_THREADS) void mlp_chain_kernel(const void *Wgu_h
     {
         // ---- down + residual: one row per wavefront (rows past N: clamped, not stored)
         const int row = blk * MC_WAVES + wave;
-        handover_pause(a_mem.pre_sleep);  // (the requests of the role before go first)
+        handover_pause_until(t_start, a_mem.pre_sleep);  // (the requests of the role before go first)
         v4u raw[NLD];
         {
             const char *rp = (const char *)Wdown_hot + ((size_t)min(row, N - 1) * KD + (size_t)lane * VEC) * ESZ;
@@ -147,7 +148,7 @@ __global__ __launch_bounds__(MC_THREADS) void mlp_chain_kernel(const void *Wgu_h
         const unsigned tag = *step_dev_hot * a_mem.tag_mul + a_mem.tag_add;
         const float res = h_hot[min(row, N - 1)];
         STAGE_T(5);
-        handover_pause(a_mem.poll_delay);
+        handover_pause_until(wall_clock64(), a_mem.poll_delay);
         {
             float v[EPT];
             if (!take_tagged<EPT>(a_mem.act_tagged + (size_t)tid * EPT, tag, a_mem.spin_limit, a_mem.poll_gap, v))

@@ -392,8 +392,8 @@ def test_attention_oproj_launch_gives_up_a_wait_that_cannot_end_in_time_and_says
         with pytest.raises(_lib.LumenError) as e:
             gpu.decode_greedy(int(np.argmax(last)), 3)
         assert e.value.status == _lib.ERR_HIP and "gave up waiting" in str(e.value)
-    gpu.set_handover(enable=1, spin_limit=1 << 22, pre_sleep=10, poll_delay=16, poll_gap=1)
-    gpu.set_handover(enable=2, pre_sleep=47, poll_delay=13, poll_gap=1)
+    gpu.set_handover(enable=1, spin_limit=1 << 22, pre_sleep=11, poll_delay=17, poll_gap=1)
+    gpu.set_handover(enable=2, pre_sleep=55, poll_delay=15, poll_gap=1)
     gpu.reset_kv_caches()
     last = gpu.forward(ids, all_rows=False)
     _, ref = ora.forward(ids)
