@@ -106,7 +106,11 @@ __global__ __launch_bounds__(AO_THREADS) void attn_oproj_kernel(const void *Wo_h
     __shared__ float sm[AO_WAVES], sl[AO_WAVES];
     __shared__ __align__(16) float xs[K > KQ ? K : KQ];
     STAGE_T(0);
-    const unsigned long long t_start = wall_clock64();
+    const unsigned t_start = (unsigned)wall_clock64();
+    // the launch's own start, for workgroups that start late (a grid larger than the chip holds at once): the first
+    // workgroup leaves its clock reading as a tagged word
+    if (blockIdx.x == 0 && threadIdx.x == 0)
+        tagged_store(a_mem.t0_tagged, __uint_as_float(t_start), *step_dev_hot * a_mem.tag_mul + a_mem.tag_add);
     const int hq = hq_hot, hkv = hkv_slices_hot & 0xffff, S = hkv_slices_hot >> 16, N = N_hot;  // S: attention slices
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n_o = (N + AO_WAVES - 1) / AO_WAVES;  // o_proj workgroups
@@ -298,7 +302,14 @@ __global__ __launch_bounds__(AO_THREADS) void attn_oproj_kernel(const void *Wo_h
     if (blk < n_o) {
         // ---- o_proj: one row per wavefront, all of its weights requested at once (rows past N: clamped, not stored)
         const int row = blk * AO_WAVES + wave;
-        handover_pause_until(t_start, a_mem.pre_sleep);  // (see the head of the file)
+        // (see the head of the file; counted from the launch's start where that is known: with long caches these
+        // workgroups wait for a free slot first, and a pause counted from their own start would begin too late)
+        unsigned t_ref = t_start;
+        {
+            const unsigned long long w0 = tagged_load(a_mem.t0_tagged);
+            if ((unsigned)(w0 >> 32) == *step_dev_hot * a_mem.tag_mul + a_mem.tag_add) t_ref = (unsigned)w0;
+        }
+        handover_pause_until32(t_ref, a_mem.pre_sleep);
         v4u raw[NLO];
         {
             const char *rp = (const char *)Wo_hot + ((size_t)min(row, N - 1) * K + (size_t)lane * VEC) * ESZ;
@@ -414,7 +425,7 @@ int launch_attn_oproj(lumen_ctx *ctx, const AttnOprojArgs &a) {
     if (!attn_oproj_supported(a.attn.hq, a.attn.hkv, a.attn.d, a.N, a.K, a.w_bf16))
         LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "attention -> o_proj chain: %d/%d heads of %d, W_o [%d, %d] not covered", a.attn.hq,
                    a.attn.hkv, a.attn.d, a.N, a.K);
-    if (!a.attn.pos_dev || a.attn.b != 1 || !a.x_tagged || !a.step_dev || !a.err_dev || !a.attn.out_tagged)
+    if (!a.attn.pos_dev || a.attn.b != 1 || !a.x_tagged || !a.step_dev || !a.err_dev || !a.attn.out_tagged || !a.t0_tagged)
         LUMEN_FAIL(LUMEN_ERR_INVALID, "attention -> o_proj chain: needs a device position, batch 1 and a hand-over buffer");
     if (a.Wqkv) {
         if (!qkv_attn_oproj_supported(a.attn.hq, a.attn.hkv, a.attn.d, a.N, a.K, a.w_bf16, a.attn.q_norm_w != nullptr))

@@ -27,6 +27,11 @@ __device__ __forceinline__ void handover_pause_until(unsigned long long t0, int 
     const unsigned long long ticks = (unsigned long long)(tenths > 0 ? tenths : 0) * 10u;
     while (wall_clock64() - t0 < ticks) __builtin_amdgcn_s_sleep(1);
 }
+// the same against a 32-bit reading of the clock (differences survive the wrap)
+__device__ __forceinline__ void handover_pause_until32(unsigned t0, int tenths) {
+    const unsigned ticks = (unsigned)(tenths > 0 ? tenths : 0) * 10u;
+    while ((unsigned)wall_clock64() - t0 < ticks) __builtin_amdgcn_s_sleep(1);
+}
 
 // This thread's EPT words of a tagged vector, polled until every one carries `tag`; false after `limit` polls.
 template <int EPT>

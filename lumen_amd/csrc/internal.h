@@ -237,6 +237,7 @@ struct AttnOprojArgs {
     // result to the o_proj workgroups.  The position must lie below nslices * slice_rows.
     int nslices, slice_rows;
     unsigned long long *part_tagged;
+    unsigned long long *t0_tagged;  // one word: the first workgroup's clock reading at its start
 };
 #define ATTN_CHAIN_MAX_SLICES 16
 bool attn_oproj_supported(int hq, int hkv, int d, int N, int K, int w_bf16);

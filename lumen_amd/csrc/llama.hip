@@ -230,13 +230,13 @@ extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg,
     M_TRY(dmalloc_t(m, &m->act_tagged, (size_t)I));
     M_TRY(dmalloc_t(m, &m->x_tagged, (size_t)m->qd));
     M_TRY(dmalloc_t(m, &m->qkv_tagged, (size_t)m->qkvd));
-    M_TRY(dmalloc_t(m, &m->part_tagged, (size_t)Hq * ATTN_CHAIN_MAX_SLICES * (D + 2)));
+    M_TRY(dmalloc_t(m, &m->part_tagged, (size_t)Hq * ATTN_CHAIN_MAX_SLICES * (D + 2) + 2));
     M_TRY(dmalloc_t(m, &m->d_step, 4));
     M_TRY(dmalloc_t(m, &m->d_err, 4));
     if (hipMemsetAsync(m->x_tagged, 0, sizeof(unsigned long long) * m->qd, ctx->stream) != hipSuccess ||
         hipMemsetAsync(m->qkv_tagged, 0, sizeof(unsigned long long) * m->qkvd, ctx->stream) != hipSuccess ||
         hipMemsetAsync(m->act_tagged, 0, sizeof(unsigned long long) * I, ctx->stream) != hipSuccess ||
-        hipMemsetAsync(m->part_tagged, 0, sizeof(unsigned long long) * Hq * ATTN_CHAIN_MAX_SLICES * (D + 2), ctx->stream) != hipSuccess ||
+        hipMemsetAsync(m->part_tagged, 0, sizeof(unsigned long long) * ((size_t)Hq * ATTN_CHAIN_MAX_SLICES * (D + 2) + 2), ctx->stream) != hipSuccess ||
         hipMemsetAsync(m->d_step, 0, 4 * sizeof(unsigned), ctx->stream) != hipSuccess ||
         hipMemsetAsync(m->d_err, 0, 4 * sizeof(int), ctx->stream) != hipSuccess) {
         lumen_llama_destroy(m);
@@ -542,8 +542,11 @@ static int enqueue_decode_step(lumen_llama *m, StepProbe *pr = nullptr) {
             f.tag_mul = (unsigned)c.num_hidden_layers; f.tag_add = (unsigned)l + 1u;
             f.err_dev = m->d_err; f.spin_limit = m->spin_limit;
             f.pre_sleep = m->chain_pre[m->chain_ao]; f.poll_delay = m->chain_delay[m->chain_ao]; f.poll_gap = m->chain_gap[m->chain_ao];
-            if (slices > 1) f.poll_delay += 12;  // (the fold of the slices is one more hand-over in front of o_proj)
+            // (the fold of the slices is one more hand-over in front of o_proj, and two-trip slices take a trip longer:
+            // polling earlier only puts polls in the way of those hand-overs; measured optima, 1.7 / 3.7 us)
+            if (slices > 1) f.poll_delay += slice_rows > attn_decode_trip_rows(m->D) ? 37 : 17;
             f.nslices = slices; f.slice_rows = slice_rows; f.part_tagged = m->part_tagged;
+            f.t0_tagged = m->part_tagged + (size_t)c.num_attention_heads * ATTN_CHAIN_MAX_SLICES * (m->D + 2);  // (one word behind the states)
             if (chain_qkv) {
                 f.Wqkv = w.wqkv; f.in_norm_w = w.in_norm; f.norm_eps = c.rms_norm_eps; f.qkv_tagged = m->qkv_tagged;
             }
