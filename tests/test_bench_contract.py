@@ -21,7 +21,8 @@ def test_more_than_one_gpu_is_refused_with_a_message():
 def test_help_names_the_workloads():
     r = run("--help")
     assert r.returncode == 0
-    for word in ("--steps", "--warmup", "--gpus", "decode", "gemv", "prefill", "--max-seq"):
+    for word in ("--steps", "--warmup", "--gpus", "decode", "gemv", "prefill", "--max-seq", "--model", "qwen3-0.6b",
+                 "llama2-7b-bf16"):
         assert word in r.stdout
 
 
