@@ -579,6 +579,7 @@ static int gemv_grid_cus(int num_cus, int N, int K, int w_bf16, int epi, int *th
     if (nunits % num_cus == 0) {
         const int w = nunits / num_cus;
         if (w > GEMV_WAVES && w <= GEMV_MAX_WAVES) waves = w;
+        else if (w > GEMV_MAX_WAVES && w % GEMV_MAX_WAVES == 0) waves = GEMV_MAX_WAVES;  // several units per wavefront, x staged once per compute unit
     }
     const int threads = waves * 64;
     int blocks = (nunits + waves - 1) / waves;
