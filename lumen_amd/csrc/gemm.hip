@@ -20,6 +20,7 @@
 // a workspace and a second kernel adds the splits in index order and applies the epilogue, so the
 // result does not depend on scheduling.
 #include "internal.h"
+#include "wave_reduce.h"
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
@@ -438,6 +439,64 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(GemmArgs a, int splits
     }
 }
 
+// The same for whole rows, with the RMSNorm of the finished row on top: one workgroup per row of C (N <= 4096, a
+// multiple of 4); a thread keeps its pieces of the row in registers between the sum of squares and the scaling.
+// Splits are added in index order, the sum of squares in the order of rmsnorm_vec_kernel: same bits as the two
+// launches it replaces.
+#define GEMM_ROW_VPT 4
+__global__ __launch_bounds__(256) void gemm_reduce_norm_kernel(GemmArgs a, int splits) {
+    typedef float v4 __attribute__((ext_vector_type(4)));
+    __shared__ float red[4];
+    const int row = blockIdx.x, tid = threadIdx.x, N = a.N;
+    const size_t MN = (size_t)a.M * N, base = (size_t)row * N;
+    v4 v[GEMM_ROW_VPT], g[GEMM_ROW_VPT];
+#pragma unroll
+    for (int i = 0; i < GEMM_ROW_VPT; ++i) {
+        const int k = (tid + i * 256) * 4;
+        v[i] = v4{0.f, 0.f, 0.f, 0.f};
+        g[i] = v[i];
+        if (k < N) {
+            v4 pv[GEMM_MAX_SPLITS];
+#pragma unroll
+            for (int s = 0; s < GEMM_MAX_SPLITS; ++s)
+                if (s < splits) pv[s] = *(const v4 *)(a.part + (size_t)s * MN + base + k);
+            const v4 r4 = *(const v4 *)(a.residual + base + k);
+            g[i] = *(const v4 *)(a.norm_w + k);
+            v4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < GEMM_MAX_SPLITS; ++s)
+                if (s < splits) acc += pv[s];
+            v[i] = r4 + acc;
+            *(v4 *)(a.C + base + k) = v[i];
+        }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < GEMM_ROW_VPT; ++i) {
+        ss = fmaf(v[i].x, v[i].x, ss);
+        ss = fmaf(v[i].y, v[i].y, ss);
+        ss = fmaf(v[i].z, v[i].z, ss);
+        ss = fmaf(v[i].w, v[i].w, ss);
+    }
+    ss = wave_sum(ss);
+    if ((tid & 63) == 0) red[tid >> 6] = ss;
+    __syncthreads();
+    const float tot = (red[0] + red[1]) + (red[2] + red[3]);
+    const float inv = 1.0f / sqrtf(tot / (float)N + a.norm_eps);
+#pragma unroll
+    for (int i = 0; i < GEMM_ROW_VPT; ++i) {
+        const int k = (tid + i * 256) * 4;
+        if (k < N) {
+            v4 r;
+            r.x = v[i].x * inv * g[i].x;
+            r.y = v[i].y * inv * g[i].y;
+            r.z = v[i].z * inv * g[i].z;
+            r.w = v[i].w * inv * g[i].w;
+            *(v4 *)(a.norm_out + base + k) = r;
+        }
+    }
+}
+
 // Any K / alignment: one thread per output element.
 template <bool BF16>
 __global__ __launch_bounds__(256) void gemm_generic_kernel(GemmArgs a) {
@@ -592,12 +651,21 @@ int launch_gemm(lumen_ctx *ctx, const GemmArgs &a) {
         launch_gemm_epi<false>(g, grid, ctx->stream);
     }
     LUMEN_CHECK_LAUNCH();
+    const bool want_norm = a.norm_w && a.norm_out && a.epi == EPI_RESIDUAL;
+    bool norm_done = false;
     if (splits > 1) {
-        size_t blocks = ((size_t)a.M * a.N + 255) / 256;
-        if (blocks > (size_t)ctx->num_cus * 8) blocks = (size_t)ctx->num_cus * 8;
-        launch_gemm_reduce(g, splits, (int)blocks, ctx->stream);
+        if (want_norm && splits <= GEMM_MAX_SPLITS && a.N % 4 == 0 && a.N <= 256 * 4 * GEMM_ROW_VPT &&
+            ((((uintptr_t)a.C | (uintptr_t)a.residual | (uintptr_t)g.part | (uintptr_t)a.norm_w | (uintptr_t)a.norm_out) & 15) == 0)) {
+            hipLaunchKernelGGL(gemm_reduce_norm_kernel, dim3(a.M), dim3(256), 0, ctx->stream, g, splits);
+            norm_done = true;
+        } else {
+            size_t blocks = ((size_t)a.M * a.N + 255) / 256;
+            if (blocks > (size_t)ctx->num_cus * 8) blocks = (size_t)ctx->num_cus * 8;
+            launch_gemm_reduce(g, splits, (int)blocks, ctx->stream);
+        }
         LUMEN_CHECK_LAUNCH();
     }
+    if (want_norm && !norm_done) LUMEN_TRY(launch_rmsnorm(ctx, a.C, a.norm_w, a.norm_out, a.M, a.N, a.norm_eps));
     return LUMEN_OK;
 }
 

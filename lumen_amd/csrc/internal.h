@@ -150,6 +150,12 @@ struct GemmArgs {
     int epi;
     const float *residual;  // [M, N]
     float *part;            // split-K partial tiles [splits, M, N] (set by the launcher)
+    // optional, with EPI_RESIDUAL: the RMSNorm of the finished rows as well, norm_out [M, N] = (C * inv_rms) * norm_w
+    // (src/layers/norm/rms_norm.rs:45-58): where K is split the pass that adds the splits takes it along (one
+    // launch instead of two), else a launch of its own follows
+    const float *norm_w;    // [N] or null
+    float *norm_out;
+    float norm_eps;
 };
 int launch_gemm(lumen_ctx *ctx, const GemmArgs &a);
 

@@ -776,7 +776,8 @@ static int run_prefill(lumen_llama *m, const std::vector<int> &ids, float *logit
     LUMEN_TRY(launch_embedding(ctx, m->embed, m->p_ids, s, H, V, m->p_x));
     for (int l = 0; l < c.num_hidden_layers; ++l) {
         const LayerW &w = m->layers[l];
-        LUMEN_TRY(launch_rmsnorm(ctx, m->p_x, w.in_norm, m->p_n, s, H, c.rms_norm_eps));
+        // (from the second layer on the down product of the layer before has left the normalised rows in p_n)
+        if (l == 0) LUMEN_TRY(launch_rmsnorm(ctx, m->p_x, w.in_norm, m->p_n, s, H, c.rms_norm_eps));
         GemmArgs g = {};
         g.A = m->p_n; g.W = w.wqkv; g.C = m->p_qkv; g.M = s; g.N = m->qkvd; g.K = H; g.w_bf16 = m->bf16; g.epi = EPI_STORE;
         LUMEN_TRY(launch_gemm(ctx, g));
@@ -793,19 +794,22 @@ static int run_prefill(lumen_llama *m, const std::vector<int> &ids, float *logit
         g = {};
         g.A = m->p_attn; g.W = w.wo; g.C = m->p_h; g.M = s; g.N = H; g.K = m->qd; g.w_bf16 = m->bf16;
         g.epi = EPI_RESIDUAL; g.residual = m->p_x;
+        g.norm_w = w.post_norm; g.norm_out = m->p_n; g.norm_eps = c.rms_norm_eps;  // post_attention_layernorm rides along
         LUMEN_TRY(launch_gemm(ctx, g));
-        LUMEN_TRY(launch_rmsnorm(ctx, m->p_h, w.post_norm, m->p_n, s, H, c.rms_norm_eps));
         g = {};
         g.A = m->p_n; g.W = w.wgu; g.C = m->p_act; g.M = s; g.N = 2 * I; g.K = H; g.w_bf16 = m->bf16; g.epi = EPI_SWIGLU;
         LUMEN_TRY(launch_gemm(ctx, g));
         g = {};
         g.A = m->p_act; g.W = w.wdown; g.C = m->p_x; g.M = s; g.N = H; g.K = I; g.w_bf16 = m->bf16;
         g.epi = EPI_RESIDUAL; g.residual = m->p_h;
+        // the next layer's input_layernorm -- or, where every row's logits are wanted, the final norm -- rides along
+        if (l + 1 < c.num_hidden_layers) { g.norm_w = m->layers[l + 1].in_norm; g.norm_out = m->p_n; g.norm_eps = c.rms_norm_eps; }
+        else if (all_rows) { g.norm_w = m->final_norm; g.norm_out = m->p_n; g.norm_eps = c.rms_norm_eps; }
         LUMEN_TRY(launch_gemm(ctx, g));
     }
     const int head_bf16 = (m->lm_head == (void *)m->embed) ? 0 : (int)m->bf16;
-    if (all_rows) {  // what the reference computes, llama.rs:202-205
-        LUMEN_TRY(launch_rmsnorm(ctx, m->p_x, m->final_norm, m->p_n, s, H, c.rms_norm_eps));
+    if (all_rows) {  // what the reference computes, llama.rs:202-205 (the final norm came with the last down product)
+        if (c.num_hidden_layers == 0) LUMEN_TRY(launch_rmsnorm(ctx, m->p_x, m->final_norm, m->p_n, s, H, c.rms_norm_eps));
         GemmArgs g = {};
         g.A = m->p_n; g.W = m->lm_head; g.C = m->p_logits; g.M = s; g.N = V; g.K = H; g.w_bf16 = head_bf16; g.epi = EPI_STORE;
         LUMEN_TRY(launch_gemm(ctx, g));
