@@ -421,6 +421,67 @@ __global__ __launch_bounds__(ATT_THREADS) void prefill_rope_kernel(AttnPrefillAr
     }
 }
 
+// The same without q/k norm, where a rotation needs nothing but its own pair: no LDS, no barriers, all heads of a
+// position at once, four pairs (or four values of v) per thread and trip.  The inputs may be the K splits of the
+// q|k|v product, added here in split order (one launch and one pass over q|k|v less than a separate sum).
+#define ROPE_MAX_SPLITS 16
+template <int D>
+__global__ __launch_bounds__(ATT_THREADS) void prefill_rope_sum_kernel(AttnPrefillArgs a) {
+    constexpr int HALF = D / 2, UPH = HALF / 4, VPH = D / 4;  // units of four per head
+    const int ss = blockIdx.x, bb = blockIdx.y;
+    const int pos = a.past_len + ss;
+    const float *cs = a.cos_t + (size_t)pos * D, *sn = a.sin_t + (size_t)pos * D;
+    const size_t row = (size_t)bb * a.s + ss;
+    const float *qrow = a.q + row * a.q_stride, *krow = a.k + row * a.k_stride, *vrow = a.v + row * a.v_stride;
+    float *qo = a.q_rot + row * (size_t)a.hq * D;
+    const int nq = a.hq * UPH, nk = a.hkv * UPH, nv = a.hkv * VPH;
+    const int splits = a.in_splits > 1 ? a.in_splits : 1;
+    const size_t sst = a.in_split_stride;
+    // all splits are requested before the first is added: one trip to memory, not one per split
+    auto sum4 = [&](const float *src) {
+        v4f pv[ROPE_MAX_SPLITS];
+#pragma unroll
+        for (int i = 0; i < ROPE_MAX_SPLITS; ++i)
+            if (i < splits) pv[i] = *(const v4f *)(src + (size_t)i * sst);
+        v4f v = pv[0];
+#pragma unroll
+        for (int i = 1; i < ROPE_MAX_SPLITS; ++i)
+            if (i < splits) v += pv[i];
+        return v;
+    };
+    {
+        const int u = blockIdx.z * ATT_THREADS + threadIdx.x;
+        if (u >= nq + nk + nv) return;
+        if (u < nq + nk) {
+            const bool isq = u < nq;
+            const int uu = isq ? u : u - nq, h = uu / UPH, j = (uu % UPH) * 4;
+            const float *src = (isq ? qrow : krow) + (size_t)h * D + j;
+            const v4f x1 = sum4(src), x2 = sum4(src + HALF);
+            const v4f c = *(const v4f *)(cs + j), s = *(const v4f *)(sn + j);
+            v4f r1, r2;
+            {
+#pragma clang fp contract(off)  // separate multiplies and add, like the reference's compiled code
+                r1 = x1 * c - x2 * s;
+                r2 = x1 * s + x2 * c;
+            }
+            float *dst = isq ? qo + (size_t)h * D + j : a.k_cache + (((size_t)bb * a.hkv + h) * a.max_seq + pos) * D + j;
+            *(v4f *)dst = r1;
+            *(v4f *)(dst + HALF) = r2;
+        } else {
+            const int uu = u - nq - nk, h = uu / VPH, j = (uu % VPH) * 4;
+            *(v4f *)(a.v_cache + (((size_t)bb * a.hkv + h) * a.max_seq + pos) * D + j) = sum4(vrow + (size_t)h * D + j);
+        }
+    }
+}
+
+static bool prefill_rope_sum_ok(const AttnPrefillArgs &a) {
+    if (a.q_norm_w || a.k_norm_w || a.d < 8) return false;
+    const uintptr_t ptrs = (uintptr_t)a.q | (uintptr_t)a.k | (uintptr_t)a.v | (uintptr_t)a.q_rot | (uintptr_t)a.k_cache |
+                           (uintptr_t)a.v_cache | (uintptr_t)a.cos_t | (uintptr_t)a.sin_t;
+    return (ptrs & 15) == 0 && ((a.q_stride | a.k_stride | a.v_stride) & 3) == 0 && (a.in_split_stride & 3) == 0 &&
+           a.in_splits <= ROPE_MAX_SPLITS;
+}
+
 // One workgroup per (query position, KV group): scores over the causal prefix
 // j <= past_len + i (softmax_inplace_view, self_attention.rs:643-678), ctx = P V,
 // out [B,S,Hq,D] (BSHD, :534).
@@ -454,7 +515,14 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_prefill_kernel(AttnPrefillAr
 
 template <int D>
 static int launch_prefill_d(lumen_ctx *ctx, const AttnPrefillArgs &a) {
-    hipLaunchKernelGGL(prefill_rope_kernel<D>, dim3(a.s, a.b), dim3(ATT_THREADS), 0, ctx->stream, a);
+    if (prefill_rope_sum_ok(a)) {
+        const int units = (a.hq + a.hkv) * (D / 8) + a.hkv * (D / 4);  // of four pairs / four values of v
+        hipLaunchKernelGGL(prefill_rope_sum_kernel<D>, dim3(a.s, a.b, (units + ATT_THREADS - 1) / ATT_THREADS), dim3(ATT_THREADS), 0,
+                           ctx->stream, a);
+    } else {
+        if (a.in_splits > 1) LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "prefill attention: split q|k|v inputs need 16-byte alignment and no q/k norm");
+        hipLaunchKernelGGL(prefill_rope_kernel<D>, dim3(a.s, a.b), dim3(ATT_THREADS), 0, ctx->stream, a);
+    }
     LUMEN_CHECK_LAUNCH();
     if (attn_prefill_mfma_supported(a)) return launch_attn_prefill_mfma(ctx, a);  // head_dim 64 / 128: matrix cores
     dim3 grid(a.s, a.hkv, a.b), block(ATT_THREADS);

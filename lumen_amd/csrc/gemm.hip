@@ -651,6 +651,11 @@ int launch_gemm(lumen_ctx *ctx, const GemmArgs &a) {
         launch_gemm_epi<false>(g, grid, ctx->stream);
     }
     LUMEN_CHECK_LAUNCH();
+    if (a.splits_used) *a.splits_used = 1;
+    if (a.keep_splits && a.splits_used && a.epi == EPI_STORE && splits > 1) {
+        *a.splits_used = splits;  // the consumer adds the partial products
+        return LUMEN_OK;
+    }
     const bool want_norm = a.norm_w && a.norm_out && a.epi == EPI_RESIDUAL;
     bool norm_done = false;
     if (splits > 1) {

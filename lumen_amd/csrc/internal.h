@@ -156,6 +156,10 @@ struct GemmArgs {
     const float *norm_w;    // [N] or null
     float *norm_out;
     float norm_eps;
+    // optional, with EPI_STORE: where K is split, leave the partial products [splits, M, N] in the workspace for a
+    // consumer that adds them itself (in split order) and report how many there are; 1 = C holds the product
+    int keep_splits;
+    int *splits_used;
 };
 int launch_gemm(lumen_ctx *ctx, const GemmArgs &a);
 
@@ -286,6 +290,10 @@ struct AttnPrefillArgs {
     const float *q_norm_w, *k_norm_w;
     float norm_eps;
     float *q_rot;    // scratch [B, S, Hq, D]
+    // q, k and v may arrive as in_splits partial sums (a GEMM's K splits), copy i at pointer + i * in_split_stride
+    // floats, to be added in index order; 0 or 1 = plain values.  Not with q/k norm.
+    int in_splits;
+    size_t in_split_stride;
 };
 int launch_attn_prefill(lumen_ctx *ctx, const AttnPrefillArgs &a);
 // the scores / softmax / context part on the matrix cores (q_rot and the cache rows already written)

@@ -780,9 +780,15 @@ static int run_prefill(lumen_llama *m, const std::vector<int> &ids, float *logit
         if (l == 0) LUMEN_TRY(launch_rmsnorm(ctx, m->p_x, w.in_norm, m->p_n, s, H, c.rms_norm_eps));
         GemmArgs g = {};
         g.A = m->p_n; g.W = w.wqkv; g.C = m->p_qkv; g.M = s; g.N = m->qkvd; g.K = H; g.w_bf16 = m->bf16; g.epi = EPI_STORE;
+        // without q/k norm the RoPE pass adds the K splits of this product itself (one launch and one pass less)
+        int qkv_splits = 1;
+        g.keep_splits = !w.q_norm && !w.k_norm && m->qkvd % 4 == 0;
+        g.splits_used = &qkv_splits;
         LUMEN_TRY(launch_gemm(ctx, g));
+        const float *qkv = qkv_splits > 1 ? ctx->gemm_ws : m->p_qkv;
         AttnPrefillArgs a = {};
-        a.q = m->p_qkv; a.k = m->p_qkv + m->qd; a.v = m->p_qkv + m->qd + m->kvd; a.out = m->p_attn;
+        a.in_splits = qkv_splits; a.in_split_stride = (size_t)s * m->qkvd;
+        a.q = qkv; a.k = qkv + m->qd; a.v = qkv + m->qd + m->kvd; a.out = m->p_attn;
         a.k_cache = m->k_slab + m->cache_stride * l; a.v_cache = m->v_slab + m->cache_stride * l;
         a.cos_t = m->cos_dev; a.sin_t = m->sin_dev;
         a.b = 1; a.s = s; a.hq = c.num_attention_heads; a.hkv = c.num_key_value_heads; a.d = m->D;
