@@ -858,3 +858,5 @@ extern "C" int lumen_attn_prefill_f32(lumen_kv_cache *c, lumen_rope *rope, const
     if (rc == LUMEN_OK) c->len = new_len;
     return rc;
 }
+
+LUMEN_DEFINE_WARM(attention)

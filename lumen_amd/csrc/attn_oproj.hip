@@ -451,3 +451,5 @@ int launch_attn_oproj(lumen_ctx *ctx, const AttnOprojArgs &a) {
     if (a.attn.d == 64) return a.w_bf16 ? launch_ao<64, true>(ctx, a) : launch_ao<64, false>(ctx, a);
     return a.w_bf16 ? launch_ao<128, true>(ctx, a) : launch_ao<128, false>(ctx, a);
 }
+
+LUMEN_DEFINE_WARM(attn_oproj)

@@ -40,6 +40,25 @@ extern "C" int lumen_ctx_create(int device, lumen_ctx **out) {
     HIP_TRY(hipEventCreate(&c->ev0));
     HIP_TRY(hipEventCreate(&c->ev1));
     HIP_TRY(hipMalloc((void **)&c->d_scratch_int, 64 * sizeof(int)));
+    HIP_TRY(hipHostMalloc(&c->bounce, LUMEN_BOUNCE_BYTES, hipHostMallocDefault));
+    // load the device code of every translation unit now rather than under the first prompt
+    lumen_warm_attention(c->stream);
+    lumen_warm_attn_oproj(c->stream);
+    lumen_warm_elementwise(c->stream);
+    lumen_warm_gemm(c->stream);
+    lumen_warm_gemv(c->stream);
+    lumen_warm_mlp_chain(c->stream);
+    lumen_warm_prefill_attention(c->stream);
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    {   // the runtime sets up its device-to-host copy path over the first few copies of a process: have them here
+        void *tmp = nullptr;
+        HIP_TRY(hipMalloc(&tmp, (size_t)256 << 10));
+        for (int i = 0; i < 3; ++i) {
+            HIP_TRY(hipMemcpyAsync(c->bounce, tmp, (size_t)256 << 10, hipMemcpyDeviceToHost, c->stream));
+            HIP_TRY(hipStreamSynchronize(c->stream));
+        }
+        HIP_TRY(hipFree(tmp));
+    }
     const int src = attn_static_scratch_init(c);
     if (src != LUMEN_OK) {
         lumen_ctx_destroy(c);
@@ -54,6 +73,7 @@ extern "C" int lumen_ctx_destroy(lumen_ctx *ctx) {
     hipSetDevice(ctx->device);
     hipStreamSynchronize(ctx->stream);
     hipFree(ctx->d_scratch_int);
+    if (ctx->bounce) hipHostFree(ctx->bounce);
     if (ctx->gemm_ws) hipFree(ctx->gemm_ws);
     hipEventDestroy(ctx->ev0);
     hipEventDestroy(ctx->ev1);
@@ -114,6 +134,14 @@ extern "C" int lumen_upload(lumen_ctx *ctx, void *dst_dev, const void *src_host,
 extern "C" int lumen_download(lumen_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes) {
     if (!ctx || (bytes && (!dst_host || !src_dev))) LUMEN_FAIL(LUMEN_ERR_INVALID, "null argument");
     if (!bytes) return LUMEN_OK;
+    // A row of logits goes through the context's pinned buffer: a copy into pageable memory leaves it to the runtime
+    // whether to stage or to pin the caller's pages, and the second such copy of a process took 5 ms for 128 KB.
+    if (bytes <= LUMEN_BOUNCE_BYTES && ctx->bounce) {
+        HIP_TRY(hipMemcpyAsync(ctx->bounce, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
+        HIP_TRY(hipStreamSynchronize(ctx->stream));
+        memcpy(dst_host, ctx->bounce, bytes);
+        return LUMEN_OK;
+    }
     HIP_TRY(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
     HIP_TRY(hipStreamSynchronize(ctx->stream));
     return LUMEN_OK;

@@ -371,3 +371,5 @@ extern "C" int lumen_rope_1token_copy_f32(lumen_rope *r, const float *src, float
         LUMEN_FAIL(LUMEN_ERR_ROPE_RANGE, "RoPE index out of range: pos %d >= max %d", pos, r->max_seq);
     return launch_rope_bhsd(r->ctx, src, dst, r->cos_dev, r->sin_dev, 1, 1, 1, d, pos);
 }
+
+LUMEN_DEFINE_WARM(elementwise)

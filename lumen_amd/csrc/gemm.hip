@@ -604,6 +604,27 @@ static int gemm_big_splits(const lumen_ctx *ctx, const GemmArgs &a) {
     return best;
 }
 
+int gemm_reserve_workspace(lumen_ctx *ctx, size_t need) {
+    if (ctx->gemm_ws_bytes >= need) return LUMEN_OK;
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    if (ctx->gemm_ws) hipFree(ctx->gemm_ws);
+    ctx->gemm_ws = nullptr;
+    ctx->gemm_ws_bytes = 0;
+    HIP_TRY(hipMalloc((void **)&ctx->gemm_ws, need));
+    ctx->gemm_ws_bytes = need;
+    return LUMEN_OK;
+}
+
+// bytes of partial tiles launch_gemm would want for this product (0: no K split)
+size_t gemm_workspace_bytes(const lumen_ctx *ctx, int M, int N, int K, int w_bf16) {
+    GemmArgs a = {};
+    a.M = M; a.N = N; a.K = K; a.w_bf16 = w_bf16;
+    if (M <= 0 || N <= 0 || K <= 0 || K % (w_bf16 ? 8 : 4)) return 0;
+    int splits = gemm_big_splits(ctx, a);
+    if (splits <= 0) splits = gemm_splits(ctx, a);
+    return splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
+}
+
 int launch_gemm(lumen_ctx *ctx, const GemmArgs &a) {
     if (a.M <= 0 || a.N <= 0) return LUMEN_OK;
     const bool aligned = (((uintptr_t)a.A | (uintptr_t)a.W) & 15) == 0;
@@ -625,15 +646,7 @@ int launch_gemm(lumen_ctx *ctx, const GemmArgs &a) {
     const bool big = splits > 0;
     if (!big) splits = gemm_splits(ctx, a);
     if (splits > 1) {
-        const size_t need = (size_t)splits * a.M * a.N * sizeof(float);
-        if (ctx->gemm_ws_bytes < need) {
-            HIP_TRY(hipStreamSynchronize(ctx->stream));
-            if (ctx->gemm_ws) hipFree(ctx->gemm_ws);
-            ctx->gemm_ws = nullptr;
-            ctx->gemm_ws_bytes = 0;
-            HIP_TRY(hipMalloc((void **)&ctx->gemm_ws, need));
-            ctx->gemm_ws_bytes = need;
-        }
+        LUMEN_TRY(gemm_reserve_workspace(ctx, (size_t)splits * a.M * a.N * sizeof(float)));
         g.part = ctx->gemm_ws;
     }
     dim3 grid((a.N + BN - 1) / BN, (a.M + BM - 1) / BM, splits);
@@ -693,3 +706,5 @@ extern "C" int lumen_gemm_bf16w(lumen_ctx *ctx, const float *A, const uint16_t *
     a.A = A; a.W = W; a.C = C; a.M = M; a.N = N; a.K = K; a.w_bf16 = 1; a.epi = EPI_STORE;
     return launch_gemm(ctx, a);
 }
+
+LUMEN_DEFINE_WARM(gemm)

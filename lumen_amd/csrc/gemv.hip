@@ -785,3 +785,5 @@ extern "C" int lumen_gemv_bench(lumen_ctx *ctx, const void *W_base, size_t strid
     }
     return lumen_timer_stop(ctx, ms_out);
 }
+
+LUMEN_DEFINE_WARM(gemv)

@@ -37,6 +37,7 @@ void lumen_set_error(const char *fmt, ...);
 #define LUMEN_CHECK_LAUNCH() HIP_TRY(hipGetLastError())
 
 // ---------------------------------------------------------------- objects
+#define LUMEN_BOUNCE_BYTES ((size_t)1 << 20)
 struct lumen_ctx {
     int device = 0;
     int num_cus = 0;
@@ -44,6 +45,7 @@ struct lumen_ctx {
     hipStream_t stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     int *d_scratch_int = nullptr;  // small device scratch (argmax result etc.)
+    void *bounce = nullptr;        // pinned host memory that small downloads travel through (LUMEN_BOUNCE_BYTES)
     float *gemm_ws = nullptr;      // split-K workspace of the prefill GEMM, grown on demand
     size_t gemm_ws_bytes = 0;
     // this device's address of the fixed scratch array behind lumen_attn_decode_static_f32
@@ -162,6 +164,23 @@ struct GemmArgs {
     int *splits_used;
 };
 int launch_gemm(lumen_ctx *ctx, const GemmArgs &a);
+int gemm_reserve_workspace(lumen_ctx *ctx, size_t bytes);  // grows the split-K workspace (synchronises the stream when it does)
+size_t gemm_workspace_bytes(const lumen_ctx *ctx, int M, int N, int K, int w_bf16);
+
+// One empty kernel per translation unit with kernels.  The runtime loads a translation unit's device code at the first
+// launch of one of its kernels (milliseconds for the larger ones); lumen_ctx_create launches these so that the first
+// prompt does not pay for it.
+#define LUMEN_DEFINE_WARM(name)                                                                  \
+    __global__ void warm_##name##_kernel() {}                                                    \
+    void lumen_warm_##name(hipStream_t s) { hipLaunchKernelGGL(warm_##name##_kernel, dim3(1), dim3(1), 0, s); }
+void lumen_warm_attention(hipStream_t s);
+void lumen_warm_attn_oproj(hipStream_t s);
+void lumen_warm_elementwise(hipStream_t s);
+void lumen_warm_gemm(hipStream_t s);
+void lumen_warm_gemv(hipStream_t s);
+void lumen_warm_mlp_chain(hipStream_t s);
+void lumen_warm_prefill_attention(hipStream_t s);
+
 
 int launch_rmsnorm(lumen_ctx *ctx, const float *x, const float *w, float *out, int rows, int dim, float eps);
 int launch_silu(lumen_ctx *ctx, const float *x, float *out, size_t n);

@@ -114,6 +114,9 @@ extern "C" int lumen_llama_destroy(lumen_llama *m) {
     return LUMEN_OK;
 }
 
+static int ensure_prefill_buffers(lumen_llama *m, int s, bool all_rows);
+static int ensure_decode_graph(lumen_llama *m);
+
 extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg, lumen_llama **out) {
     if (!ctx || !cfg || !out) LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_create: null argument");
     *out = nullptr;
@@ -261,6 +264,15 @@ extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg,
         }
     }
     m->decode_mode = LUMEN_DECODE_GRAPH;
+    // buffers of a prompt pass of up to 512 rows now, not under the first prompt (longer prompts grow them)
+    M_TRY(ensure_prefill_buffers(m, std::min(cfg->max_seq_len, 512), false));
+    // ... and the decode step recorded and instantiated for a short cache (recorded again when the cache outgrows it)
+    M_TRY(ensure_decode_graph(m));
+    if (m->graph_exec) hipGraphUpload(m->graph_exec, ctx->stream);
+    if (hipStreamSynchronize(ctx->stream) != hipSuccess) {
+        lumen_llama_destroy(m);
+        LUMEN_FAIL(LUMEN_ERR_HIP, "llama_create: preparing the decode graph failed");
+    }
 #undef M_TRY
     *out = m;
     return LUMEN_OK;
@@ -754,6 +766,13 @@ static int ensure_prefill_buffers(lumen_llama *m, int s, bool all_rows) {
         HIP_TRY(hipMalloc((void **)&m->p_act, S * c.intermediate_size * 4));
         HIP_TRY(hipMalloc((void **)&m->p_ids, S * sizeof(int)));
         m->pf_cap = s;
+        // the split-K workspace of the four products at this many rows, so that no launch has to grow it
+        const int H = c.hidden_size, I = c.intermediate_size;
+        size_t ws = gemm_workspace_bytes(m->ctx, s, m->qkvd, H, m->bf16);
+        ws = std::max(ws, gemm_workspace_bytes(m->ctx, s, H, m->qd, m->bf16));
+        ws = std::max(ws, gemm_workspace_bytes(m->ctx, s, 2 * I, H, m->bf16));
+        ws = std::max(ws, gemm_workspace_bytes(m->ctx, s, H, I, m->bf16));
+        if (ws) LUMEN_TRY(gemm_reserve_workspace(m->ctx, ws));
     }
     if (all_rows && s > m->pf_logit_cap) {
         HIP_TRY(hipStreamSynchronize(m->ctx->stream));

@@ -228,3 +228,5 @@ int launch_mlp_chain(lumen_ctx *ctx, const MlpChainArgs &a) {
         LUMEN_FAIL(LUMEN_ERR_INVALID, "MLP chain: operands must be 16-byte aligned");
     return a.w_bf16 ? launch_mc<true>(ctx, a) : launch_mc<false>(ctx, a);
 }
+
+LUMEN_DEFINE_WARM(mlp_chain)

@@ -295,3 +295,5 @@ int launch_attn_prefill_mfma(lumen_ctx *ctx, const AttnPrefillArgs &a) {
     if (a.d == 128) return launch_fa_d<128>(ctx, a);
     LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "matrix-core prefill attention: head_dim=%d (supported 64, 128)", a.d);
 }
+
+LUMEN_DEFINE_WARM(prefill_attention)
