@@ -425,7 +425,7 @@ __global__ __launch_bounds__(ATT_THREADS) void prefill_rope_kernel(AttnPrefillAr
 // position at once, four pairs (or four values of v) per thread and trip.  The inputs may be the K splits of the
 // q|k|v product, added here in split order (one launch and one pass over q|k|v less than a separate sum).
 #define ROPE_MAX_SPLITS 16
-template <int D>
+template <int D, bool SPLIT>
 __global__ __launch_bounds__(ATT_THREADS) void prefill_rope_sum_kernel(AttnPrefillArgs a) {
     constexpr int HALF = D / 2, UPH = HALF / 4, VPH = D / 4;  // units of four per head
     const int ss = blockIdx.x, bb = blockIdx.y;
@@ -439,6 +439,7 @@ __global__ __launch_bounds__(ATT_THREADS) void prefill_rope_sum_kernel(AttnPrefi
     const size_t sst = a.in_split_stride;
     // all splits are requested before the first is added: one trip to memory, not one per split
     auto sum4 = [&](const float *src) {
+        if (!SPLIT) return *(const v4f *)src;
         v4f pv[ROPE_MAX_SPLITS];
 #pragma unroll
         for (int i = 0; i < ROPE_MAX_SPLITS; ++i)
@@ -517,8 +518,9 @@ template <int D>
 static int launch_prefill_d(lumen_ctx *ctx, const AttnPrefillArgs &a) {
     if (prefill_rope_sum_ok(a)) {
         const int units = (a.hq + a.hkv) * (D / 8) + a.hkv * (D / 4);  // of four pairs / four values of v
-        hipLaunchKernelGGL(prefill_rope_sum_kernel<D>, dim3(a.s, a.b, (units + ATT_THREADS - 1) / ATT_THREADS), dim3(ATT_THREADS), 0,
-                           ctx->stream, a);
+        const dim3 rgrid(a.s, a.b, (units + ATT_THREADS - 1) / ATT_THREADS);
+        if (a.in_splits > 1) hipLaunchKernelGGL((prefill_rope_sum_kernel<D, true>), rgrid, dim3(ATT_THREADS), 0, ctx->stream, a);
+        else hipLaunchKernelGGL((prefill_rope_sum_kernel<D, false>), rgrid, dim3(ATT_THREADS), 0, ctx->stream, a);
     } else {
         if (a.in_splits > 1) LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "prefill attention: split q|k|v inputs need 16-byte alignment and no q/k norm");
         hipLaunchKernelGGL(prefill_rope_kernel<D>, dim3(a.s, a.b), dim3(ATT_THREADS), 0, ctx->stream, a);
