@@ -207,9 +207,10 @@ __global__ __launch_bounds__(256) void gemm_bf16x3_kernel(GemmArgs a) {
 // The pipelined kernel: F x F tiles of 32x32 per wavefront, 2 x 2 wavefronts, 16-deep slices, LDS
 // double-buffered.  The split of slice s+1 into the other LDS half stands in the same block as the matrix
 // instructions of slice s, one bf16 plane of one 16-byte piece ("plane step") after every F of them, and
-// runs in their shadow; slice s+2 travels from memory meanwhile; one barrier per slice.  LDS rows are the
-// 16 bf16 of a slice (32 bytes): operand reads and staging writes of a wavefront are contiguous, so no
-// swizzle is needed.
+// runs in their shadow; slice s+2 travels from memory meanwhile; one barrier per slice.  In LDS the two k halves
+// of a slice lie in planes of their own, [k half][row][8 bf16]: 8 neighbouring lanes of an operand read (8 rows, one
+// half) take 128 contiguous bytes (with the halves side by side in 32-byte rows a third of the LDS cycles of this
+// kernel were bank conflicts).
 //   F = 4: 256x256 output tile, all 256 accumulator registers of a wavefront, one workgroup per compute
 //          unit.  A 4x4 register tile reads half the LDS bytes per matrix instruction of a 2x2 one, which
 //          is what bounds gemm_bf16x3_kernel.  For thousands of prompt rows.
@@ -251,8 +252,13 @@ __global__ __launch_bounds__(256, (F == 4 ? 1 : 2)) void gemm_bf16x3_tile_kernel
     constexpr int TM = 64 * F, TN = 64 * F;
     constexpr int AST = F;                    // 16-byte pieces of A per thread per slice: TM rows x 16 k / 256 threads
     constexpr int WST = WBF16 ? F / 2 : F;
-    __shared__ __align__(16) uint16_t As[2][3][TM][GB_K];
-    __shared__ __align__(16) uint16_t Ws[2][PW][TN][GB_K];
+    // [half][part][k half g][row][8 bf16]: the 8 k of an operand lane are one 16-byte unit, units of neighbouring rows
+    // are neighbours, so the 8 lanes of an LDS pass (8 rows, one g) read 128 contiguous bytes; the two k halves are
+    // 64 bytes further apart than a power of two (LPAD rows), so that a staging write of 4 rows x 2 halves x 2 pieces
+    // covers all banks once.
+    constexpr int LPAD = 4;
+    __shared__ __align__(16) uint16_t As[2][3][2][TM + LPAD][8];
+    __shared__ __align__(16) uint16_t Ws[2][PW][2][TN + LPAD][8];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int bm = blockIdx.y * TM, bn = blockIdx.x * TN;
@@ -311,15 +317,15 @@ __global__ __launch_bounds__(256, (F == 4 ? 1 : 2)) void gemm_bf16x3_tile_kernel
                 ra[0] = va[pc].x; ra[1] = va[pc].y; ra[2] = va[pc].z; ra[3] = va[pc].w;
             }
         }
-        if (WBF16 && u < WST) *(v4u *)&Ws[b][0][(tid + u * 256) >> 1][(tid & 1) * 8] = vw[u < WST ? u : 0];
-        uint16_t *dst = isw ? &Ws[b][p][idx >> 2][(idx & 3) * 4] : &As[b][p][idx >> 2][(idx & 3) * 4];
+        if (WBF16 && u < WST) *(v4u *)&Ws[b][0][tid & 1][(tid + u * 256) >> 1][0] = vw[u < WST ? u : 0];
+        uint16_t *dst = isw ? &Ws[b][p][(idx & 3) >> 1][idx >> 2][(idx & 1) * 4] : &As[b][p][(idx & 3) >> 1][idx >> 2][(idx & 1) * 4];
         *(v2u *)dst = (v2u){pack_hi(ra[1], ra[0]), pack_hi(ra[3], ra[2])};
         if (p < 2) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) ra[e] -= __uint_as_float(__float_as_uint(ra[e]) & 0xffff0000u);
         }
     };
-    const int c = lane & 31, g8 = (lane >> 5) * 8;
+    const int c = lane & 31, gk = lane >> 5;
     // The matrix instructions of the slice in LDS half b.  With with_stage the next slice is split into the
     // other half between them, a plane step after every F matrix instructions, so that the vector ALU works
     // in their shadow.
@@ -330,13 +336,13 @@ __global__ __launch_bounds__(256, (F == 4 ? 1 : 2)) void gemm_bf16x3_tile_kernel
         for (int i = 0; i < F; ++i)
 #pragma unroll
             for (int p = 0; p < 3; ++p)
-                af[i][p] = __builtin_bit_cast(bf16x8, *(const v4u *)&As[b][p][wm * (F * 32) + i * 32 + c][g8]);
+                af[i][p] = __builtin_bit_cast(bf16x8, *(const v4u *)&As[b][p][gk][wm * (F * 32) + i * 32 + c][0]);
 #pragma unroll
         for (int j = 0; j < F; ++j) {
             bf16x8 wf[PW];
 #pragma unroll
             for (int p = 0; p < PW; ++p)
-                wf[p] = __builtin_bit_cast(bf16x8, *(const v4u *)&Ws[b][p][wn * (F * 32) + j * 32 + c][g8]);
+                wf[p] = __builtin_bit_cast(bf16x8, *(const v4u *)&Ws[b][p][gk][wn * (F * 32) + j * 32 + c][0]);
 #pragma unroll
             for (int q = 0; q < NPROD; ++q) {
                 const int xa = WBF16 ? 2 - q : PA_[q], xw = WBF16 ? 0 : PW_[q];
