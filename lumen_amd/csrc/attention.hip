@@ -421,11 +421,11 @@ __global__ __launch_bounds__(ATT_THREADS) void prefill_rope_kernel(AttnPrefillAr
     }
 }
 
-// The same without q/k norm, where a rotation needs nothing but its own pair: no LDS, no barriers, all heads of a
-// position at once, four pairs (or four values of v) per thread and trip.  The inputs may be the K splits of the
+// The same with 16-byte accesses: no LDS, no barriers, all heads of a position at once, four pairs (or four values of
+// v) per thread; the sum of squares of a q/k norm is taken over the head's D / 8 neighbouring lanes.  The inputs may be the K splits of the
 // q|k|v product, added here in split order (one launch and one pass over q|k|v less than a separate sum).
 #define ROPE_MAX_SPLITS 16
-template <int D, bool SPLIT>
+template <int D, bool SPLIT, bool NORM>
 __global__ __launch_bounds__(ATT_THREADS) void prefill_rope_sum_kernel(AttnPrefillArgs a) {
     constexpr int HALF = D / 2, UPH = HALF / 4, VPH = D / 4;  // units of four per head
     const int ss = blockIdx.x, bb = blockIdx.y;
@@ -457,7 +457,21 @@ __global__ __launch_bounds__(ATT_THREADS) void prefill_rope_sum_kernel(AttnPrefi
             const bool isq = u < nq;
             const int uu = isq ? u : u - nq, h = uu / UPH, j = (uu % UPH) * 4;
             const float *src = (isq ? qrow : krow) + (size_t)h * D + j;
-            const v4f x1 = sum4(src), x2 = sum4(src + HALF);
+            v4f x1 = sum4(src), x2 = sum4(src + HALF);
+            if (NORM) {
+                // q/k norm over the head (rms_norm.rs:45-58 on [.., D]): the head's D / 8 units are neighbouring lanes
+                const float *g = isq ? a.q_norm_w : a.k_norm_w;
+                if (g) {
+                    float sq = x1.x * x1.x + x1.y * x1.y + x1.z * x1.z + x1.w * x1.w + x2.x * x2.x + x2.y * x2.y + x2.z * x2.z +
+                               x2.w * x2.w;
+#pragma unroll
+                    for (int o = 1; o < UPH; o <<= 1) sq += __shfl_xor(sq, o, 64);
+                    const float inv = 1.0f / sqrtf(sq / (float)D + a.norm_eps);
+                    const v4f g1 = *(const v4f *)(g + j), g2 = *(const v4f *)(g + j + HALF);
+                    x1 = x1 * inv * g1;
+                    x2 = x2 * inv * g2;
+                }
+            }
             const v4f c = *(const v4f *)(cs + j), s = *(const v4f *)(sn + j);
             v4f r1, r2;
             {
@@ -476,9 +490,10 @@ __global__ __launch_bounds__(ATT_THREADS) void prefill_rope_sum_kernel(AttnPrefi
 }
 
 static bool prefill_rope_sum_ok(const AttnPrefillArgs &a) {
-    if (a.q_norm_w || a.k_norm_w || a.d < 8) return false;
+    if (a.d < 8) return false;
     const uintptr_t ptrs = (uintptr_t)a.q | (uintptr_t)a.k | (uintptr_t)a.v | (uintptr_t)a.q_rot | (uintptr_t)a.k_cache |
-                           (uintptr_t)a.v_cache | (uintptr_t)a.cos_t | (uintptr_t)a.sin_t;
+                           (uintptr_t)a.v_cache | (uintptr_t)a.cos_t | (uintptr_t)a.sin_t | (uintptr_t)a.q_norm_w |
+                           (uintptr_t)a.k_norm_w;
     return (ptrs & 15) == 0 && ((a.q_stride | a.k_stride | a.v_stride) & 3) == 0 && (a.in_split_stride & 3) == 0 &&
            a.in_splits <= ROPE_MAX_SPLITS;
 }
@@ -519,10 +534,16 @@ static int launch_prefill_d(lumen_ctx *ctx, const AttnPrefillArgs &a) {
     if (prefill_rope_sum_ok(a)) {
         const int units = (a.hq + a.hkv) * (D / 8) + a.hkv * (D / 4);  // of four pairs / four values of v
         const dim3 rgrid(a.s, a.b, (units + ATT_THREADS - 1) / ATT_THREADS);
-        if (a.in_splits > 1) hipLaunchKernelGGL((prefill_rope_sum_kernel<D, true>), rgrid, dim3(ATT_THREADS), 0, ctx->stream, a);
-        else hipLaunchKernelGGL((prefill_rope_sum_kernel<D, false>), rgrid, dim3(ATT_THREADS), 0, ctx->stream, a);
+        const bool norm = a.q_norm_w || a.k_norm_w;
+        if (a.in_splits > 1) {
+            if (norm) hipLaunchKernelGGL((prefill_rope_sum_kernel<D, true, true>), rgrid, dim3(ATT_THREADS), 0, ctx->stream, a);
+            else hipLaunchKernelGGL((prefill_rope_sum_kernel<D, true, false>), rgrid, dim3(ATT_THREADS), 0, ctx->stream, a);
+        } else {
+            if (norm) hipLaunchKernelGGL((prefill_rope_sum_kernel<D, false, true>), rgrid, dim3(ATT_THREADS), 0, ctx->stream, a);
+            else hipLaunchKernelGGL((prefill_rope_sum_kernel<D, false, false>), rgrid, dim3(ATT_THREADS), 0, ctx->stream, a);
+        }
     } else {
-        if (a.in_splits > 1) LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "prefill attention: split q|k|v inputs need 16-byte alignment and no q/k norm");
+        if (a.in_splits > 1) LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "prefill attention: split q|k|v inputs need 16-byte alignment");
         hipLaunchKernelGGL(prefill_rope_kernel<D>, dim3(a.s, a.b), dim3(ATT_THREADS), 0, ctx->stream, a);
     }
     LUMEN_CHECK_LAUNCH();

@@ -310,7 +310,7 @@ struct AttnPrefillArgs {
     float norm_eps;
     float *q_rot;    // scratch [B, S, Hq, D]
     // q, k and v may arrive as in_splits partial sums (a GEMM's K splits), copy i at pointer + i * in_split_stride
-    // floats, to be added in index order; 0 or 1 = plain values.  Not with q/k norm.
+    // floats, to be added in index order; 0 or 1 = plain values.
     int in_splits;
     size_t in_split_stride;
 };

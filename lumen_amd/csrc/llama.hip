@@ -799,9 +799,9 @@ static int run_prefill(lumen_llama *m, const std::vector<int> &ids, float *logit
         if (l == 0) LUMEN_TRY(launch_rmsnorm(ctx, m->p_x, w.in_norm, m->p_n, s, H, c.rms_norm_eps));
         GemmArgs g = {};
         g.A = m->p_n; g.W = w.wqkv; g.C = m->p_qkv; g.M = s; g.N = m->qkvd; g.K = H; g.w_bf16 = m->bf16; g.epi = EPI_STORE;
-        // without q/k norm the RoPE pass adds the K splits of this product itself (one launch and one pass less)
+        // the RoPE pass adds the K splits of this product itself (one launch and one pass less)
         int qkv_splits = 1;
-        g.keep_splits = !w.q_norm && !w.k_norm && m->qkvd % 4 == 0;
+        g.keep_splits = m->qkvd % 4 == 0;
         g.splits_used = &qkv_splits;
         LUMEN_TRY(launch_gemm(ctx, g));
         const float *qkv = qkv_splits > 1 ? ctx->gemm_ws : m->p_qkv;
