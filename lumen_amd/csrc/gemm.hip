@@ -394,6 +394,160 @@ __global__ __launch_bounds__(256, (F == 4 ? 1 : 2)) void gemm_bf16x3_tile_kernel
     store_wave_tiles<EPI, PARTIAL, F>(a, acc, bm, bn, wm, wn, lane);
 }
 
+// Prompts of two to four rows (a batch of drafted tokens, the tail of a chunked prompt): the product is bound by the weights,
+// which the tile kernels above cannot stream at anything like the memory's rate (they take 100 us per layer whatever M
+// is).  This kernel walks W the way the single-row product does: a wavefront takes units of two whole rows, lanes across
+// K with 16-byte loads, in pieces of 4 sweeps x 2 rows = 8 loads per lane, two pieces in flight and the next one
+// requested as soon as a register set is free, unit after unit.  Every piece is multiplied with MS rows of A at once:
+// plain f32 multiply-adds in the lanes, a wavefront reduction per (row of A, row of W) when a unit is complete -- the
+// accumulation order of the single-row product (src/ops/matmul.rs:42-69 applied to each row of A).  The MS rows of A
+// lie in LDS for the whole launch, staged once per workgroup (K padded with zeros to whole pieces); more rows of A than
+// MS: tiles of MS over gridDim.y (W is then streamed once per tile).
+#define SK_WAVES 8
+#define SK_THREADS (SK_WAVES * 64)
+template <int MS, bool BF16, int EPI>
+__global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(GemmArgs a, int kpad) {
+    constexpr int VEC = BF16 ? 8 : 4;          // elements per 16-byte load
+    constexpr int SWEEP = 64 * VEC;            // elements of a row one wavefront covers per load
+    constexpr int R = 2, U = 4;
+    constexpr int PIECE = SWEEP * U;
+    constexpr int ESZ = BF16 ? 2 : 4;
+    extern __shared__ __align__(16) float As[];  // [MS][kpad]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int M = a.M, N = a.N, K = a.K;
+    const int m0 = blockIdx.y * MS;
+    const int nunits = (N + R - 1) / R;
+    const int gw = blockIdx.x * SK_WAVES + wave, nw = gridDim.x * SK_WAVES;
+    const char *Wb = (const char *)a.W;
+    const size_t row_bytes = (size_t)K * ESZ;
+
+    // every load is issued unconditionally: positions past the end of a row are clamped to its last 16 bytes (they meet
+    // the zero padding of A), a row past N to row N-1 (not stored)
+    auto load_piece = [&](int u, int k0, v4u (&raw)[R][U]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const char *rp = Wb + (size_t)min(u * R + r, N - 1) * row_bytes;
+#pragma unroll
+            for (int uu = 0; uu < U; ++uu) {
+                const int kk = min(k0 + uu * SWEEP + lane * VEC, K - VEC);
+                raw[r][uu] = __builtin_nontemporal_load((const v4u *)(rp + (size_t)kk * ESZ));
+            }
+        }
+    };
+    const int np = kpad / PIECE;
+    int lu = gw, lk = 0;  // unit / element offset of the next piece to load
+    auto advance_load = [&]() __attribute__((always_inline)) {
+        lk += PIECE;
+        if (lk >= kpad) {
+            lk = 0;
+            lu += nw;
+        }
+    };
+    const int my_units = (nunits > gw) ? (nunits - gw + nw - 1) / nw : 0;
+    const int T = my_units * np;
+    // the first weights are on their way before A is staged: they do not depend on it
+    v4u rawA[R][U], rawB[R][U];
+    load_piece(min(lu, nunits - 1), lk, rawA);
+    advance_load();
+    if (T > 1) {
+        load_piece(lu, lk, rawB);
+        advance_load();
+    }
+    for (int i = tid * 4; i < MS * kpad; i += SK_THREADS * 4) {
+        const int m = i / kpad, k = i - m * kpad;
+        v4f v = {0.f, 0.f, 0.f, 0.f};
+        if (m0 + m < M && k < K) v = *(const v4f *)(a.A + (size_t)(m0 + m) * K + k);  // K % 4 == 0
+        *(v4f *)&As[i] = v;
+    }
+    __syncthreads();
+
+    float acc[R][MS];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int m = 0; m < MS; ++m) acc[r][m] = 0.f;
+    int u = gw, k0 = 0;  // unit / element offset of the piece being multiplied
+    auto consume = [&](const v4u (&raw)[R][U]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int uu = 0; uu < U; ++uu) {
+            const int kl = k0 + uu * SWEEP + lane * VEC;
+#pragma unroll
+            for (int m = 0; m < MS; ++m) {
+                const v4f x0 = *(const v4f *)&As[m * kpad + kl];
+                v4f x1 = x0;
+                if (BF16) x1 = *(const v4f *)&As[m * kpad + kl + 4];
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const v4u w = raw[r][uu];
+                    float s = acc[r][m];
+                    if (BF16) {  // eight bf16 values, widened by a shift (src/loader.rs:58)
+                        s = fmaf(__uint_as_float(w.x << 16), x0.x, s);
+                        s = fmaf(__uint_as_float(w.x & 0xffff0000u), x0.y, s);
+                        s = fmaf(__uint_as_float(w.y << 16), x0.z, s);
+                        s = fmaf(__uint_as_float(w.y & 0xffff0000u), x0.w, s);
+                        s = fmaf(__uint_as_float(w.z << 16), x1.x, s);
+                        s = fmaf(__uint_as_float(w.z & 0xffff0000u), x1.y, s);
+                        s = fmaf(__uint_as_float(w.w << 16), x1.z, s);
+                        s = fmaf(__uint_as_float(w.w & 0xffff0000u), x1.w, s);
+                    } else {
+                        s = fmaf(__uint_as_float(w.x), x0.x, s);
+                        s = fmaf(__uint_as_float(w.y), x0.y, s);
+                        s = fmaf(__uint_as_float(w.z), x0.z, s);
+                        s = fmaf(__uint_as_float(w.w), x0.w, s);
+                    }
+                    acc[r][m] = s;
+                }
+            }
+        }
+        k0 += PIECE;
+        if (k0 >= kpad) {  // unit complete
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int m = 0; m < MS; ++m) acc[r][m] = wave_sum(acc[r][m]);
+            if (lane == 0) {
+                const int row = u * R;
+#pragma unroll
+                for (int m = 0; m < MS; ++m) {
+                    if (m0 + m >= M) continue;
+                    const size_t mrow = (size_t)(m0 + m);
+                    if (EPI == EPI_SWIGLU) {
+                        // rows (2u, 2u + 1) hold (gate_u, up_u): silu(gate) * up, src/models/llama.rs:60-63
+                        if (row + 1 < N) a.C[mrow * (N >> 1) + u] = silu_g(acc[0][m]) * acc[1][m];
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < R; ++r)
+                            if (row + r < N) {
+                                const size_t o = mrow * N + row + r;
+                                a.C[o] = (EPI == EPI_RESIDUAL) ? a.residual[o] + acc[r][m] : acc[r][m];
+                            }
+                    }
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int m = 0; m < MS; ++m) acc[r][m] = 0.f;
+            k0 = 0;
+            u += nw;
+        }
+    };
+    for (int t = 0; t < T; t += 2) {
+        consume(rawA);
+        if (t + 2 < T) {
+            load_piece(lu, lk, rawA);
+            advance_load();
+        }
+        if (t + 1 < T) {
+            consume(rawB);
+            if (t + 3 < T) {
+                load_piece(lu, lk, rawB);
+                advance_load();
+            }
+        }
+    }
+}
+
 #define GEMM_MAX_SPLITS 16
 // Adds the K splits of every output element in split order and applies the epilogue.
 template <int EPI>
@@ -631,10 +785,65 @@ size_t gemm_workspace_bytes(const lumen_ctx *ctx, int M, int N, int K, int w_bf1
     return splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
 }
 
+// up to 4 rows of A the weight-streaming kernel wins (TinyLlama shape: prompt pass of 2 tokens 2.45 -> 1.48 ms, of 4
+// tokens 2.46 -> 1.89 ms); at 8 rows the two are level, beyond that the multiply-adds and LDS reads per piece cost more
+// than the tile kernels' fixed 100 us per layer
+#ifndef GEMM_SKINNY_MAX_M
+#define GEMM_SKINNY_MAX_M 4
+#endif
+template <int MS, bool BF16>
+static int launch_gemm_skinny(lumen_ctx *ctx, const GemmArgs &a, int kpad) {
+    const size_t lds = (size_t)MS * kpad * sizeof(float);
+    // one round of workgroups: as many as fit the compute units' LDS side by side, two at most (16 wavefronts)
+    int per_cu = (int)((size_t)(160 * 1024) / (lds + 512));
+    if (per_cu > 2) per_cu = 2;
+    if (per_cu < 1) per_cu = 1;
+    const int nunits = (a.N + 1) / 2;
+    int blocks = (nunits + SK_WAVES - 1) / SK_WAVES;
+    const int cap = ctx->num_cus * per_cu;
+    if (blocks > cap) {  // every wavefront the same number of units
+        const int per_wave = (nunits + cap * SK_WAVES - 1) / (cap * SK_WAVES);
+        blocks = (nunits + SK_WAVES * per_wave - 1) / (SK_WAVES * per_wave);
+    }
+    dim3 grid(blocks, (a.M + MS - 1) / MS);
+#define SK_LAUNCH(E)                                                                                                  \
+    do {                                                                                                              \
+        if (lds > 64 * 1024)                                                                                          \
+            HIP_TRY(hipFuncSetAttribute((const void *)gemm_skinny_kernel<MS, BF16, E>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
+        hipLaunchKernelGGL((gemm_skinny_kernel<MS, BF16, E>), grid, dim3(SK_THREADS), lds, ctx->stream, a, kpad);      \
+    } while (0)
+    switch (a.epi) {
+        case EPI_STORE: SK_LAUNCH(EPI_STORE); break;
+        case EPI_RESIDUAL: SK_LAUNCH(EPI_RESIDUAL); break;
+        default: SK_LAUNCH(EPI_SWIGLU); break;
+    }
+#undef SK_LAUNCH
+    LUMEN_CHECK_LAUNCH();
+    return LUMEN_OK;
+}
+
 int launch_gemm(lumen_ctx *ctx, const GemmArgs &a) {
     if (a.M <= 0 || a.N <= 0) return LUMEN_OK;
     const bool aligned = (((uintptr_t)a.A | (uintptr_t)a.W) & 15) == 0;
     const bool fast = (a.K % (a.w_bf16 ? 8 : 4) == 0) && aligned && a.K > 0;  // rows of 16-byte pieces
+    if (fast && a.M <= GEMM_SKINNY_MAX_M && (a.epi != EPI_SWIGLU || !(a.N & 1))) {
+        // two to four rows of A: the weights are streamed the way the single-row product streams them, once per MS rows
+        // of A (4, or 2 where 4 rows of K padded to whole pieces do not fit LDS)
+        const int piece = 64 * (a.w_bf16 ? 8 : 4) * 4;
+        const int kpad = (a.K + piece - 1) / piece * piece;
+        int ms = a.M <= 2 ? 2 : 4;
+        if ((size_t)ms * kpad * sizeof(float) > 150 * 1024) ms = 2;
+        if ((size_t)ms * kpad * sizeof(float) <= 150 * 1024) {
+            if (a.splits_used) *a.splits_used = 1;
+            int rc;
+            if (a.w_bf16) rc = ms == 4 ? launch_gemm_skinny<4, true>(ctx, a, kpad) : launch_gemm_skinny<2, true>(ctx, a, kpad);
+            else rc = ms == 4 ? launch_gemm_skinny<4, false>(ctx, a, kpad) : launch_gemm_skinny<2, false>(ctx, a, kpad);
+            LUMEN_TRY(rc);
+            if (a.norm_w && a.norm_out && a.epi == EPI_RESIDUAL)
+                LUMEN_TRY(launch_rmsnorm(ctx, a.C, a.norm_w, a.norm_out, a.M, a.N, a.norm_eps));
+            return LUMEN_OK;
+        }
+    }
     if (!fast) {
         if (a.epi != EPI_STORE) LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "fused GEMM needs rows of whole 16-byte pieces and 16-byte alignment (K=%d)", a.K);
         size_t blocks = ((size_t)a.M * a.N + 255) / 256;

@@ -106,6 +106,29 @@ def test_last_row_only_prefill_equals_all_rows_and_incremental_prefill():
     assert max_rel(full, ref) <= 1e-4
 
 
+@pytest.mark.parametrize("cfg,tol,bf16", [(TINY, 1e-4, False), (TINY_QWEN, 1e-4, False), (SMALL, 1e-4, False),
+                                          (TINY, 2e-2, True)], ids=["gqa", "qwen3", "small", "gqa-bf16"])
+@pytest.mark.parametrize("n", [2, 3, 4])
+def test_prompts_of_two_to_four_tokens(cfg, tol, bf16, n):
+    """Prompt passes of up to four rows take the weight-streaming product (whole weight rows per wavefront, the rows of
+    the prompt multiplied side by side, store / residual / SwiGLU epilogues) instead of the matrix-core tiles: same
+    branch of the reference (S > 1, matmul.rs:70-92), checked into an empty and into a live cache."""
+    gpu, ora, _ = build(cfg, seed=30 + n, bf16=bf16)
+    ids = synth.make_tokens(3 * n + 1, cfg["vocab_size"], seed=30 + n)
+    got = gpu.forward(ids[:n], all_rows=True)
+    rc, ref = ora.forward(ids[:n])
+    assert rc == lo.LO_OK and max_rel(got, ref) <= tol
+    got = gpu.forward(ids[n:2 * n], all_rows=True)          # into a live cache (main.rs:333-335)
+    rc, ref = ora.forward(ids[n:2 * n])
+    assert max_rel(got, ref) <= tol
+    last = gpu.forward(ids[2 * n:3 * n], all_rows=False)    # what a chat turn keeps: the last row
+    rc, ref = ora.forward(ids[2 * n:3 * n])
+    assert max_rel(last, ref[-1]) <= tol
+    one = gpu.forward(ids[3 * n:], all_rows=False)           # and a decode step on top of it
+    rc, ref = ora.forward(ids[3 * n:])
+    assert max_rel(one, ref[-1]) <= tol and gpu.kv_len == 3 * n + 1
+
+
 def test_greedy_generation_on_device_matches_oracle_loop():
     gpu, ora, _ = build(SMALL, seed=13)
     prompt = synth.make_tokens(12, SMALL["vocab_size"], seed=13)

@@ -72,7 +72,11 @@ def test_matmul_shape_errors_and_empty():
 
 
 @pytest.mark.parametrize("M,N,K", [(2, 3, 4), (7, 33, 132), (128, 256, 2048), (130, 200, 64), (64, 5632, 512),
-                                   (5, 9, 7), (300, 129, 260), (16, 2560, 2048)])
+                                   (5, 9, 7), (300, 129, 260), (16, 2560, 2048),
+                                   # two to four rows: the weight-streaming kernel (whole rows per wavefront); ragged N,
+                                   # K not a whole number of pieces, K that needs the 2-row tile, one unit per wavefront
+                                   (2, 2560, 2048), (3, 2047, 5632), (4, 11264, 2048), (4, 33, 8200), (2, 5, 1028),
+                                   (4, 4096, 11008)])
 def test_gemm_against_oracle(M, N, K):
     A = f32(RNG.normal(0, 1, (1, M, K)))
     W = f32(RNG.normal(0, 0.02, (N, K)))
@@ -112,8 +116,8 @@ def test_gemm_keeps_f32_accuracy_across_magnitudes():
     assert errb.max() <= 1e-6, errb.max()
 
 
-def test_gemm_bf16_weights():
-    M, N, K = 48, 300, 256
+@pytest.mark.parametrize("M,N,K", [(48, 300, 256), (3, 301, 1024), (4, 4096, 11008)])
+def test_gemm_bf16_weights(M, N, K):
     A = f32(RNG.normal(0, 1, (M, K)))
     bits = lo.f32_to_bf16(f32(RNG.normal(0, 0.02, (N, K))))
     C = ops.matmul(dev(A), dev(bits)).data()
