@@ -403,7 +403,7 @@ __global__ __launch_bounds__(256, (F == 4 ? 1 : 2)) void gemm_bf16x3_tile_kernel
 // accumulation order of the single-row product (src/ops/matmul.rs:42-69 applied to each row of A).  The MS rows of A
 // lie in LDS for the whole launch, staged once per workgroup (K padded with zeros to whole pieces); more rows of A than
 // MS: tiles of MS over gridDim.y (W is then streamed once per tile).
-#define SK_WAVES 8
+#define SK_WAVES 4  // (8 wavefronts per workgroup leave a round of workgroups uneven over the compute units: 1.48 against 1.44 ms)
 #define SK_THREADS (SK_WAVES * 64)
 template <int MS, bool BF16, int EPI>
 __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(GemmArgs a, int kpad) {
@@ -794,9 +794,9 @@ size_t gemm_workspace_bytes(const lumen_ctx *ctx, int M, int N, int K, int w_bf1
 template <int MS, bool BF16>
 static int launch_gemm_skinny(lumen_ctx *ctx, const GemmArgs &a, int kpad) {
     const size_t lds = (size_t)MS * kpad * sizeof(float);
-    // one round of workgroups: as many as fit the compute units' LDS side by side, two at most (16 wavefronts)
+    // one round of workgroups: as many as fit the compute units' LDS side by side, 16 wavefronts at most
     int per_cu = (int)((size_t)(160 * 1024) / (lds + 512));
-    if (per_cu > 2) per_cu = 2;
+    if (per_cu > 16 / SK_WAVES) per_cu = 16 / SK_WAVES;
     if (per_cu < 1) per_cu = 1;
     const int nunits = (a.N + 1) / 2;
     int blocks = (nunits + SK_WAVES - 1) / SK_WAVES;
@@ -822,18 +822,30 @@ static int launch_gemm_skinny(lumen_ctx *ctx, const GemmArgs &a, int kpad) {
     return LUMEN_OK;
 }
 
+// rows of A per tile of the few-row kernel for this product, 0: the tile kernels take it
+static int gemm_skinny_rows(const GemmArgs &a, int *kpad_out) {
+    const bool aligned = (((uintptr_t)a.A | (uintptr_t)a.W) & 15) == 0;
+    const bool fast = (a.K % (a.w_bf16 ? 8 : 4) == 0) && aligned && a.K > 0;  // rows of 16-byte pieces
+    if (!fast || a.M <= 0 || a.M > GEMM_SKINNY_MAX_M || (a.epi == EPI_SWIGLU && (a.N & 1))) return 0;
+    const int piece = 64 * (a.w_bf16 ? 8 : 4) * 4;
+    const int kpad = (a.K + piece - 1) / piece * piece;
+    int ms = a.M <= 2 ? 2 : 4;
+    if ((size_t)ms * kpad * sizeof(float) > 150 * 1024) ms = 2;
+    if ((size_t)ms * kpad * sizeof(float) > 150 * 1024) return 0;
+    if (kpad_out) *kpad_out = kpad;
+    return ms;
+}
+
 int launch_gemm(lumen_ctx *ctx, const GemmArgs &a) {
     if (a.M <= 0 || a.N <= 0) return LUMEN_OK;
     const bool aligned = (((uintptr_t)a.A | (uintptr_t)a.W) & 15) == 0;
     const bool fast = (a.K % (a.w_bf16 ? 8 : 4) == 0) && aligned && a.K > 0;  // rows of 16-byte pieces
-    if (fast && a.M <= GEMM_SKINNY_MAX_M && (a.epi != EPI_SWIGLU || !(a.N & 1))) {
+    int kpad = 0;
+    const int ms = gemm_skinny_rows(a, &kpad);
+    if (ms) {
         // two to four rows of A: the weights are streamed the way the single-row product streams them, once per MS rows
         // of A (4, or 2 where 4 rows of K padded to whole pieces do not fit LDS)
-        const int piece = 64 * (a.w_bf16 ? 8 : 4) * 4;
-        const int kpad = (a.K + piece - 1) / piece * piece;
-        int ms = a.M <= 2 ? 2 : 4;
-        if ((size_t)ms * kpad * sizeof(float) > 150 * 1024) ms = 2;
-        if ((size_t)ms * kpad * sizeof(float) <= 150 * 1024) {
+        {
             if (a.splits_used) *a.splits_used = 1;
             int rc;
             if (a.w_bf16) rc = ms == 4 ? launch_gemm_skinny<4, true>(ctx, a, kpad) : launch_gemm_skinny<2, true>(ctx, a, kpad);
