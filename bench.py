@@ -44,6 +44,9 @@ def main():
                          "Llama-2-7B shape with bf16 weights (--prompt 512 --steps 40 --max-seq 1024).  The bench line "
                          "the driver reads is the default one; the others carry no cpu_baseline")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip the long-context, Qwen3-0.6B-shape and Llama-2-7B-shape decode records that the default "
+                         "run appends (other_configs) after the headline measurement")
     ap.add_argument("--mode", choices=["graph", "eager"], default="graph",
                     help="how decode steps are issued: a HIP graph replay per token (default) or kernel by kernel "
                          "(for rocprofv3 --kernel-trace, which cannot follow graph replays here)")
@@ -69,31 +72,66 @@ def main():
 
     import numpy as np
 
-    from lumen_amd import _lib, synth
-    from lumen_amd.models import LlamaModel
+    from lumen_amd import synth
 
     base = {"tinyllama-1.1b": synth.TINYLLAMA_1B, "qwen3-0.6b": synth.QWEN3_0P6B, "llama2-7b-bf16": synth.LLAMA2_7B}[args.model]
     cfg = dict(base, max_seq_len=args.max_seq)
-    headline = args.model == "tinyllama-1.1b"
+    headline = args.model == "tinyllama-1.1b" and args.prompt == 128 and args.max_seq == 2048
     if not headline:
         args.no_cpu_baseline = True
+        args.no_other_configs = True
+    out, model, params, prompt = decode_bench(args.model, cfg, args.prompt, args.steps, args.warmup, args.mode,
+                                              keep_host=not args.no_cpu_baseline, headline=headline)
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfg, params, prompt, args.cpu_tokens, model)
+    del model, params
+    if not args.no_other_configs:
+        # the other decode configurations of the benchmark, same library, same protocol, after the headline's timed
+        # region: long context (cache 3976-4008 rows), the Qwen3-0.6B shape, the Llama-2-7B shape with bf16 weights
+        out["other_configs"] = []
+        for name, ocfg, n_prompt in (("tinyllama-1.1b", dict(synth.TINYLLAMA_1B_LONG), 3968),
+                                     ("qwen3-0.6b", dict(synth.QWEN3_0P6B), 256),
+                                     ("llama2-7b-bf16", dict(synth.LLAMA2_7B), 512)):
+            steps = min(args.steps, (ocfg["max_seq_len"] - n_prompt - min(args.warmup, 8) - 8) // 2)
+            o, m, _, _ = decode_bench(name, ocfg, n_prompt, steps, min(args.warmup, 8), args.mode, keep_host=False, headline=False)
+            del m
+            out["other_configs"].append({
+                "workload": o["config"]["workload"], "dtype": o["dtype"], "steps": steps, "ms_per_step": o["ms_per_step"],
+                "tokens_per_s": o["value"], "kv_len_during_timing": o["config"]["kv_len_during_timing"],
+                "bytes_per_token": o["step_roofline"]["bytes_per_token"], "frac_of_8TBps": o["step_roofline"]["frac_of_8TBps"],
+                "kernels": o["kernels"], "kernel_instances": o["kernel_instances"],
+                "prefill_ms": o["prefill"]["ms"], "graph_picks_equal_eager_picks": o["self_check"]["graph_picks_equal_eager_picks"],
+                "setup_s": o["setup_s"]})
+    print(json.dumps(out))
+
+
+MODEL_NAMES = {"tinyllama-1.1b": "TinyLlama-1.1B", "qwen3-0.6b": "Qwen3-0.6B", "llama2-7b-bf16": "Llama-2-7B"}
+
+
+def decode_bench(model_name, cfg, n_prompt, steps, warmup, mode, keep_host, headline):
+    """One decode measurement: build the random-init model, prompt pass, warm-up, EXACTLY `steps` greedy tokens
+    between two events on the library's stream, then the per-kernel passes.  Returns (record, model, params, prompt)."""
+    import numpy as np
+
+    from lumen_amd import _lib, synth
+    from lumen_amd.models import LlamaModel
+
     w_bf16 = cfg.get("weight_dtype") == "bf16"
-    need = args.prompt + args.warmup + 3 * args.steps + 8
+    need = n_prompt + warmup + 2 * steps + 8
     if need > cfg["max_seq_len"]:
-        sys.exit("bench.py: prompt + warmup + 3*steps = %d exceeds max_seq_len %d" % (need, cfg["max_seq_len"]))
+        sys.exit("bench.py: prompt + warmup + 2*steps = %d exceeds max_seq_len %d" % (need, cfg["max_seq_len"]))
 
     t0 = time.time()
     model = LlamaModel(cfg)
-    model.set_decode_mode(args.mode)
-    keep_host = not args.no_cpu_baseline
+    model.set_decode_mode(mode)
     params = {}
-    for name, a in synth.iter_params(cfg, seed=0):
-        if w_bf16 and a.ndim == 2 and "embed" not in name:
-            a = synth.bf16_round(a)  # bf16-stored weights: the values the reference would widen at load time
+    # bf16-stored weights: the values the reference would widen at load time
+    to_bits = (lambda name, a: synth.bf16_round(a) if a.ndim == 2 and "embed" not in name else a) if w_bf16 else None
+    for name, a in synth.iter_params_threaded(cfg, seed=0, workers=12, transform=to_bits):
         model.set_param(name, a)
         if keep_host:
             params[name] = a
-    prompt = synth.make_tokens(args.prompt, cfg["vocab_size"], seed=0)
+    prompt = synth.make_tokens(n_prompt, cfg["vocab_size"], seed=0)
     t_setup = time.time() - t0
 
     # prefill (outside the timed decode region; reported separately).  The first pass sizes the
@@ -109,37 +147,42 @@ def main():
     first = int(np.argmax(last))
 
     # warmup, then EXACTLY --steps decoded tokens between two events on the library's stream
-    if args.warmup:
-        w = model.decode_greedy(first, args.warmup)
+    if warmup:
+        w = model.decode_greedy(first, warmup)
         first = int(w[-1])
     len0 = model.kv_len
     ctx.synchronize()
     wall0 = time.perf_counter()
     ctx.timer_start()
-    picks = model.decode_greedy(first, args.steps)
+    picks = model.decode_greedy(first, steps)
     ms = ctx.timer_stop()
     wall = time.perf_counter() - wall0
-    ms_per_step = ms / args.steps
+    ms_per_step = ms / steps
     tok_s = 1000.0 / ms_per_step
-    mean_len = len0 + (args.steps + 1) / 2.0
+    mean_len = len0 + (steps + 1) / 2.0
     step_bytes = model.decode_bytes(int(round(mean_len)))
 
-    # Per-kernel durations, live: a second pass of the same length with every launch between two HIP
-    # events on the library's stream (eager launches of the same kernels).  An event pair adds a fixed
-    # cost to what it brackets; it is measured here as well -- a third pass launches the same kernels
-    # one by one WITHOUT events, and (bracketed total - plain total) / launches is that cost -- and
-    # taken off, so that the figures are kernel durations (they agree with the rocprofv3 trace).
-    prof = model.decode_profile(int(picks[-1]), args.steps)
+    # The timed pass checks itself: the same steps again from the same cache state, launched kernel by kernel
+    # instead of replayed from the graph, must pick the same tokens.  (That pass is also the plain eager timing.)
+    model.set_kv_len(len0)
     model.set_decode_mode("eager")
     ctx.timer_start()
-    model.decode_greedy(int(picks[-1]), args.steps)
+    picks_eager = model.decode_greedy(first, steps)
     eager_ms = ctx.timer_stop()
-    model.set_decode_mode(args.mode)
+    model.set_decode_mode(mode)
+    if not np.array_equal(picks, picks_eager):
+        raise SystemExit("bench: the timed pass picked %s, eager launches of the same steps %s" % (picks.tolist(), picks_eager.tolist()))
+
+    # Per-kernel durations, live: a further pass of the same length with every launch between two HIP
+    # events on the library's stream (eager launches of the same kernels).  An event pair adds a fixed
+    # cost to what it brackets; (bracketed total - plain eager total) / launches is that cost, and it is
+    # taken off, so that the figures are kernel durations (they agree with the rocprofv3 trace).
+    prof = model.decode_profile(int(picks[-1]), steps)
     n_launches = sum(n for _, n in prof.values())
     bracketed_ms = sum(s_ms for s_ms, _ in prof.values())
     event_overhead_ms = max(0.0, (bracketed_ms - eager_ms) / max(n_launches, 1))
     H, I = cfg["hidden_size"], cfg["intermediate_size"]
-    # dominant kernel: RMSNorm + gate|up GEMV + SwiGLU, W [2I, H] f32 read once per launch
+    # dominant kernel: RMSNorm + gate|up GEMV + SwiGLU, W [2I, H] read once per launch
     esz = 2.0 if w_bf16 else 4.0
     mlp_fused = prof["mlp_fused"][1] > 0  # narrow models: gate|up and down are one launch
     gu_ms, gu_n = prof["mlp_fused"] if mlp_fused else prof["norm_gateup_gemv"]
@@ -151,10 +194,8 @@ def main():
     for name, (s_ms, n) in prof.items():
         if n:
             kernels[name] = {"avg_us": round(1e3 * (s_ms / n - event_overhead_ms), 3),
-                             "launches_per_step": n // args.steps}
+                             "launches_per_step": n // steps}
 
-    # decode attention: K and V rows of every KV head, read once per launch (mean cache length of the timed
-    # region); with short caches attention and o_proj are one launch, which also streams W_o [H, H]
     # Kernel instances: the names the launchers recorded during that profile pass.  The dominant one must be what the
     # library's own dispatch reports for [2I, H] (lumen_gemv_kernel_name reads the decision launch_gemv takes), and
     # the committed counter figures are only quoted when they were taken on that same instance.
@@ -163,6 +204,8 @@ def main():
     picked = _lib.gemv_kernel_name(ctx.num_cus, 2 * I, H, w_bf16, True, _lib.GEMV_EPI_SWIGLU)
     if not mlp_fused and gu_kernel != picked:
         raise SystemExit("bench: gate|up launched %r but the dispatch reports %r" % (gu_kernel, picked))
+    # decode attention: K and V rows of every KV head, read once per launch (mean cache length of the timed
+    # region); with short caches attention and o_proj are one launch, which also streams W_o [H, H]
     hq, hkv = cfg["num_attention_heads"], cfg["num_key_value_heads"]
     D = cfg.get("head_dim") or H // hq
     fused_attn = prof["attn_oproj_fused"][1] > 0
@@ -179,14 +222,14 @@ def main():
             at_what = "RMSNorm + q|k|v + RoPE, decode attention, o_proj + residual"
     out = {
         "metric": "batch-1 decode tokens/s", "value": round(tok_s, 2), "unit": "tokens/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 weights, f32 accumulate" if w_bf16 else "f32", "data": "synthetic",
         "config": {"workload": "%s-shaped model %s random-init seed 0, batch 1, prompt %d random ids, "
                                "greedy decode, static KV cache max_seq_len %d"
-                               % ({"tinyllama-1.1b": "TinyLlama-1.1B", "qwen3-0.6b": "Qwen3-0.6B", "llama2-7b-bf16": "Llama-2-7B"}[args.model],
-                                  "bf16 weights" if w_bf16 else "fp32", args.prompt, cfg["max_seq_len"]),
+                               % (MODEL_NAMES[model_name], "bf16 weights" if w_bf16 else "fp32", n_prompt, cfg["max_seq_len"]),
                    "layers": cfg["num_hidden_layers"], "hidden": H, "heads": "%dq/%dkv" % (hq, hkv), "head_dim": D,
-                   "intermediate": I, "vocab": cfg["vocab_size"], "kv_len_during_timing": [len0, len0 + args.steps]},
+                   "intermediate": I, "vocab": cfg["vocab_size"], "kv_len_during_timing": [len0, len0 + steps]},
         "roofline": {"bound": "hbm", "kernel": "%s (RMSNorm + gate|up GEMV [%d,%d] + SwiGLU%s)"
                                % (gu_kernel, 2 * I, H, ", down [%d,%d] + residual" % (H, I) if mlp_fused else ""),
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -201,14 +244,12 @@ def main():
                       "avg_launch_us": round(at_avg_ms * 1e3, 3), "achieved_GBps": round(at_bytes / (at_avg_ms * 1e-3) / 1e9, 1),
                       "frac_of_8TBps": round(at_bytes / (at_avg_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
         "kernels": kernels, "kernel_instances": names,
-        "prefill": dict(prefill_report(cfg, args.prompt, prefill_ms), passes_ms=[round(x, 3) for x in prefill_all_ms]),
-        "decode_mode": args.mode, "eager_ms_per_step": round(eager_ms / args.steps, 5),
+        "prefill": dict(prefill_report(cfg, n_prompt, prefill_ms), passes_ms=[round(x, 3) for x in prefill_all_ms]),
+        "decode_mode": mode, "eager_ms_per_step": round(eager_ms / steps, 5),
+        "self_check": {"graph_picks_equal_eager_picks": True, "steps": steps},
         "wall_s_timed_region": round(wall, 4), "setup_s": round(t_setup, 1),
     }
-
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(cfg, params, prompt, args.cpu_tokens)
-    print(json.dumps(out))
+    return out, model, params, prompt
 
 
 def prefill_report(cfg, S, ms):
@@ -381,9 +422,11 @@ def prefill_bench(args):
     print(json.dumps(out))
 
 
-def cpu_baseline(cfg, params, prompt, n_tokens):
+def cpu_baseline(cfg, params, prompt, n_tokens, model):
     """The C restatement of Lumen's CPU path (row-parallel M=1 GEMV, head-parallel online-softmax
-    attention) on the host cores: prefill the same prompt, then time n_tokens greedy decode steps."""
+    attention) on the host cores: prefill the same prompt, then time n_tokens greedy decode steps.
+    Its logits then check the GPU path of this very process: the same prompt and the same tokens through
+    `model` (prompt pass, then one decode step per token), every row within 1e-4 or the run stops."""
     import numpy as np
 
     from oracle import lumen_oracle as lo
@@ -391,16 +434,28 @@ def cpu_baseline(cfg, params, prompt, n_tokens):
     ora = lo.Llama(cfg, params)
     rc, logits = ora.forward(prompt)
     assert rc == lo.LO_OK
+    ref_rows = [logits[-1].copy()]
     tok = lo.argmax(logits[-1])
+    toks = [tok]
     t0 = time.perf_counter()
     for _ in range(n_tokens):
         rc, lg = ora.forward(np.array([tok]))
         tok = lo.argmax(lg[0])
+        ref_rows.append(lg[0].copy())
+        toks.append(tok)
     dt = time.perf_counter() - t0
+    model.reset_kv_caches()
+    worst = 0.0
+    for t, ref in enumerate(ref_rows):
+        got = model.forward(prompt if t == 0 else np.array([toks[t - 1]]), all_rows=False)
+        worst = max(worst, float(np.abs(got.astype(np.float64) - ref).max() / np.abs(ref).max()))
+    if not worst <= 1e-4:
+        raise SystemExit("bench: GPU logits differ from the CPU restatement's by %.3g (tolerance 1e-4)" % worst)
     return {"value": round(n_tokens / dt, 3), "unit": "tokens/s", "cores": lo.get_threads(), "kind": "port",
             "sample": "%d greedy decode tokens after the same %d-token prompt, same weights; C restatement of "
                       "Lumen's CPU algorithms (gcc -O3 -march=x86-64-v3 -ffp-contract=off, OpenMP), Rust toolchain "
-                      "unavailable" % (n_tokens, len(prompt))}
+                      "unavailable" % (n_tokens, len(prompt)),
+            "gpu_logits_vs_cpu": {"rows": len(ref_rows), "max_rel_err": worst, "tolerance": 1e-4}}
 
 
 if __name__ == "__main__":

@@ -760,6 +760,7 @@ class LlamaEngine {
         return out;
     }
     void reset_kv_caches() { check(lumen_llama_reset(h_)); }  // llama.rs:172-176
+    void set_kv_len(size_t n) { check(lumen_llama_set_kv_len(h_, (int)n)); }  // KVCacheInner.len, a public field (:28)
     size_t kv_len() const {
         int n = 0;
         check(lumen_llama_kv_len(h_, &n));

@@ -333,12 +333,20 @@ int lumen_llama_profile_kernel_name(const lumen_llama *model, int kernel_class, 
  * wavefront still exits -- and the timing of the o_proj workgroups: pre_sleep, their weight requests go out that
  * many tenths of a microsecond after the workgroup's start; poll_delay, their first poll follows that many tenths
  * later; poll_gap, pause between polls in units of 256 clocks (kept per form; the call sets those of the form in
- * use after it).  A negative argument leaves that setting as it is.
+ * use after it).  A negative argument leaves that setting as it is.  Limits (beyond them LUMEN_ERR_INVALID):
+ * spin_limit <= 2^22, pre_sleep and poll_delay <= 1000 (100 us), poll_gap <= 16 -- so a wait that cannot end costs
+ * about 10 s at the very worst (a few seconds with the defaults) before its workgroup flags it and exits.
+ * A single-token lumen_llama_forward without a logits pointer does not synchronise: a wait given up inside it is
+ * reported by the next call that does (forward with logits, decode_greedy, decode_profile).
  * enable = 1 or 2 on a shape that form does not cover -> LUMEN_ERR_UNSUPPORTED. */
 int lumen_llama_set_handover(lumen_llama *model, int enable, int64_t spin_limit, int pre_sleep, int poll_delay, int poll_gap);
 int lumen_llama_get_decode_mode(const lumen_llama *model, int *mode_out);
 int lumen_llama_reset(lumen_llama *model);                      /* reset_kv_caches, llama.rs:172-176 */
 int lumen_llama_kv_len(const lumen_llama *model, int *len_out);
+/* len of every layer's cache at once (a public field of the reference's KVCacheInner, self_attention.rs:28): go
+ * back to an earlier length -- the rows beyond it are overwritten by the steps that follow -- e.g. to decode the
+ * same positions again.  Outside [0, current length] -> LUMEN_ERR_KV_OVERFLOW (rows never written cannot be claimed). */
+int lumen_llama_set_kv_len(lumen_llama *model, int len);
 int lumen_llama_cache_download(lumen_llama *model, int layer, float *k_host, float *v_host);
 /* bytes of weights + KV prefix one decode step at cache length len must read */
 int lumen_llama_decode_bytes(const lumen_llama *model, int len, double *bytes_out);

@@ -188,7 +188,8 @@ __device__ __forceinline__ bool attn_decode_slice(const AttnDecodeArgs &a, int r
         }
     }
     if (nact == 1 || a.defer_merge) return true;  // one slice, or the consumer folds them
-    // every wavefront's stores are ordered before thread 0's arrival by the barrier (see handover_arrive)
+    // every wavefront's stores are acknowledged before the barrier, hence before thread 0's arrival (see handover_arrive)
+    handover_stores_done();
     __syncthreads();
     if (t == 0) {
         int *counter = a.counters + (size_t)bb * a.hq + hq;

@@ -446,6 +446,9 @@ int launch_attn_oproj(lumen_ctx *ctx, const AttnOprojArgs &a) {
                           (a.slice_rows & (a.slice_rows - 1)) || a.slice_rows % attn_decode_trip_rows(a.attn.d)))
         LUMEN_FAIL(LUMEN_ERR_INVALID, "attention -> o_proj chain: %d slices (at most %d, with a buffer for their states)", a.nslices,
                    ATTN_CHAIN_MAX_SLICES);
+    if (!handover_timing_ok(a.spin_limit, a.pre_sleep, a.poll_delay, a.poll_gap))
+        LUMEN_FAIL(LUMEN_ERR_INVALID, "attention -> o_proj chain: wait limits out of range (%u polls, pauses %d / %d / %d)",
+                   a.spin_limit, a.pre_sleep, a.poll_delay, a.poll_gap);
     if ((size_t)a.attn.max_seq * a.attn.d * sizeof(float) >= ((size_t)1 << 32))
         LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "attention -> o_proj chain: a KV head of %d rows x %d exceeds 4 GiB", a.attn.max_seq, a.attn.d);
     if (a.attn.d == 64) return a.w_bf16 ? launch_ao<64, true>(ctx, a) : launch_ao<64, false>(ctx, a);

@@ -815,7 +815,8 @@ static int launch_gemm_skinny(lumen_ctx *ctx, const GemmArgs &a, int kpad) {
     switch (a.epi) {
         case EPI_STORE: SK_LAUNCH(EPI_STORE); break;
         case EPI_RESIDUAL: SK_LAUNCH(EPI_RESIDUAL); break;
-        default: SK_LAUNCH(EPI_SWIGLU); break;
+        case EPI_SWIGLU: SK_LAUNCH(EPI_SWIGLU); break;
+        default: LUMEN_FAIL(LUMEN_ERR_INVALID, "few-row product: epilogue %d", a.epi);
     }
 #undef SK_LAUNCH
     LUMEN_CHECK_LAUNCH();
@@ -827,6 +828,7 @@ static int gemm_skinny_rows(const GemmArgs &a, int *kpad_out) {
     const bool aligned = (((uintptr_t)a.A | (uintptr_t)a.W) & 15) == 0;
     const bool fast = (a.K % (a.w_bf16 ? 8 : 4) == 0) && aligned && a.K > 0;  // rows of 16-byte pieces
     if (!fast || a.M <= 0 || a.M > GEMM_SKINNY_MAX_M || (a.epi == EPI_SWIGLU && (a.N & 1))) return 0;
+    if (a.epi != EPI_STORE && a.epi != EPI_RESIDUAL && a.epi != EPI_SWIGLU) return 0;  // (the three epilogues it has)
     const int piece = 64 * (a.w_bf16 ? 8 : 4) * 4;
     const int kpad = (a.K + piece - 1) / piece * piece;
     int ms = a.M <= 2 ? 2 : 4;
@@ -838,6 +840,8 @@ static int gemm_skinny_rows(const GemmArgs &a, int *kpad_out) {
 
 int launch_gemm(lumen_ctx *ctx, const GemmArgs &a) {
     if (a.M <= 0 || a.N <= 0) return LUMEN_OK;
+    if (a.epi != EPI_STORE && a.epi != EPI_RESIDUAL && a.epi != EPI_SWIGLU)  // (the switches below read SwiGLU into "else")
+        LUMEN_FAIL(LUMEN_ERR_INVALID, "GEMM: epilogue %d (store, residual or SwiGLU)", a.epi);
     const bool aligned = (((uintptr_t)a.A | (uintptr_t)a.W) & 15) == 0;
     const bool fast = (a.K % (a.w_bf16 ? 8 : 4) == 0) && aligned && a.K > 0;  // rows of 16-byte pieces
     int kpad = 0;

@@ -461,6 +461,7 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W
             __hip_atomic_store(a.amax_val + blockIdx.x, best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(a.amax_idx + blockIdx.x, best_idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
+        handover_stores_done();
         __syncthreads();
         if (threadIdx.x == 0) {
             const int old = handover_arrive(a.amax_counter);

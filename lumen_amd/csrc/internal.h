@@ -269,6 +269,17 @@ struct AttnOprojArgs {
     unsigned long long *t0_tagged;  // one word: the first workgroup's clock reading at its start
 };
 #define ATTN_CHAIN_MAX_SLICES 16
+// Limits of the waits inside the chained launches, enforced by lumen_llama_set_handover and by the launchers: a
+// pause is at most 100 us, a wait at most 2^22 polls of at most 16 x 256 clocks plus a trip to memory each -- about
+// 10 s in the worst case, a few seconds with the default settings -- after which the waiting workgroup flags the
+// failure and exits.
+#define HANDOVER_MAX_TENTHS 1000
+#define HANDOVER_MAX_GAP 16
+#define HANDOVER_MAX_SPINS (1u << 22)
+static inline bool handover_timing_ok(unsigned spin_limit, int pre_sleep, int poll_delay, int poll_gap) {
+    return spin_limit <= HANDOVER_MAX_SPINS && pre_sleep >= 0 && pre_sleep <= HANDOVER_MAX_TENTHS && poll_delay >= 0 &&
+           poll_delay <= HANDOVER_MAX_TENTHS && poll_gap >= 0 && poll_gap <= HANDOVER_MAX_GAP;
+}
 bool attn_oproj_supported(int hq, int hkv, int d, int N, int K, int w_bf16);
 bool qkv_attn_oproj_supported(int hq, int hkv, int d, int N, int K, int w_bf16, int qk_norm);
 int launch_attn_oproj(lumen_ctx *ctx, const AttnOprojArgs &a);

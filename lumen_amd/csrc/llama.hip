@@ -686,11 +686,16 @@ extern "C" int lumen_llama_set_handover(lumen_llama *m, int enable, int64_t spin
     if (enable > 1 && !qkv_attn_oproj_supported(m->cfg.num_attention_heads, m->cfg.num_key_value_heads, m->D, m->cfg.hidden_size,
                                                 m->qd, m->bf16, m->cfg.qk_norm))
         LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "the q|k|v -> attention -> o_proj launch does not cover this model shape");
+    if (spin_limit > (int64_t)HANDOVER_MAX_SPINS || pre_sleep > HANDOVER_MAX_TENTHS || poll_delay > HANDOVER_MAX_TENTHS ||
+        poll_gap > HANDOVER_MAX_GAP)
+        LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_set_handover: spin_limit at most %u, pre_sleep and poll_delay at most %d "
+                                      "(tenths of a microsecond), poll_gap at most %d", HANDOVER_MAX_SPINS,
+                   HANDOVER_MAX_TENTHS, HANDOVER_MAX_GAP);
     if (enable >= 0) {
         m->chain_ao = enable > 2 ? 2 : enable;
         m->chain_ao_on = enable > 0;  // (enable 0 also takes the MLP chain of narrow models apart)
     }
-    if (spin_limit >= 0) m->spin_limit = spin_limit > 0xffffffffLL ? 0xffffffffu : (unsigned)spin_limit;
+    if (spin_limit >= 0) m->spin_limit = (unsigned)spin_limit;
     if (pre_sleep >= 0) m->chain_pre[m->chain_ao] = pre_sleep;
     if (poll_delay >= 0) m->chain_delay[m->chain_ao] = poll_delay;
     if (poll_gap >= 0) m->chain_gap[m->chain_ao] = poll_gap;
@@ -870,6 +875,8 @@ extern "C" int lumen_llama_forward(lumen_llama *m, const float *ids_host, int s,
         LUMEN_TRY(lumen_download(m->ctx, logits_host, m->logits, sizeof(float) * (size_t)m->cfg.vocab_size));
         return check_handover(m);
     }
+    // (no logits wanted: the step stays in flight, and a wait that gave up inside it is reported by the next call
+    // that synchronises -- lumen_llama_forward with logits, lumen_llama_decode_greedy, lumen_llama_decode_profile)
     return LUMEN_OK;
 }
 
@@ -953,6 +960,7 @@ extern "C" int lumen_llama_decode_profile(lumen_llama *m, int first_id, int n, d
             lumen_set_error("decode_profile step %d: %s", t, hipGetErrorString(e));
             rc = LUMEN_ERR_HIP;
         }
+        if (rc == LUMEN_OK) rc = check_handover(m);  // (figures of a step whose wait gave up would mean nothing)
     }
     return rc;
 }
@@ -968,6 +976,15 @@ extern "C" int lumen_llama_profile_kernel_name(const lumen_llama *m, int kernel_
 extern "C" int lumen_llama_reset(lumen_llama *m) {
     if (!m) LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_reset: null model");
     m->len = 0;  // KVCacheInner::reset, self_attention.rs:41-43: data stays
+    return sync_pos_to_device(m);
+}
+
+extern "C" int lumen_llama_set_kv_len(lumen_llama *m, int len) {
+    if (!m) LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_set_kv_len: null model");
+    if (len < 0 || len > m->len)
+        LUMEN_FAIL(LUMEN_ERR_KV_OVERFLOW, "llama_set_kv_len: %d outside [0, %d]", len, m->len);
+    HIP_TRY(hipSetDevice(m->ctx->device));
+    m->len = len;
     return sync_pos_to_device(m);
 }
 

@@ -226,6 +226,9 @@ int launch_mlp_chain(lumen_ctx *ctx, const MlpChainArgs &a) {
         LUMEN_FAIL(LUMEN_ERR_INVALID, "MLP chain: null argument");
     if ((((uintptr_t)a.Wgu | (uintptr_t)a.Wdown | (uintptr_t)a.h | (uintptr_t)a.norm_w) & 15) != 0)
         LUMEN_FAIL(LUMEN_ERR_INVALID, "MLP chain: operands must be 16-byte aligned");
+    if (!handover_timing_ok(a.spin_limit, a.pre_sleep, a.poll_delay, a.poll_gap))
+        LUMEN_FAIL(LUMEN_ERR_INVALID, "MLP chain: wait limits out of range (%u polls, pauses %d / %d / %d)", a.spin_limit,
+                   a.pre_sleep, a.poll_delay, a.poll_gap);
     return a.w_bf16 ? launch_mc<true>(ctx, a) : launch_mc<false>(ctx, a);
 }
 

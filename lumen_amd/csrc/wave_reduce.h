@@ -52,6 +52,10 @@ __device__ __forceinline__ float wave_max(float v) {
 #ifndef LUMEN_HANDOVER_ORDER
 #define LUMEN_HANDOVER_ORDER __ATOMIC_RELAXED
 #endif
+// In front of the barrier that precedes handover_arrive: this wavefront's partial stores are acknowledged (written
+// through to the memory side) before it enters the barrier.  The compiler emits this wait in front of s_barrier
+// anyway; stating it here keeps the hand-over independent of that.
+__device__ __forceinline__ void handover_stores_done() { __builtin_amdgcn_s_waitcnt(0); }
 __device__ __forceinline__ int handover_arrive(int *counter) {
     return __hip_atomic_fetch_add(counter, 1, LUMEN_HANDOVER_ORDER, __HIP_MEMORY_SCOPE_AGENT);
 }

@@ -119,6 +119,11 @@ class LlamaModel:
         check(lib.lumen_llama_kv_len(self.handle, C.byref(n)))
         return n.value
 
+    def set_kv_len(self, length):
+        """Back to an earlier cache length (KVCacheInner.len is a public field, self_attention.rs:28): the rows beyond
+        it are overwritten by the steps that follow."""
+        check(lib.lumen_llama_set_kv_len(self.handle, int(length)))
+
     def cache(self, layer):
         cfg = self.config
         d = cfg.head_dim or cfg.hidden_size // cfg.num_attention_heads

@@ -79,6 +79,27 @@ def iter_params(cfg, seed=0, std=0.02, gains_one=True):
         yield name, make_param(name, shape, seed, std, gains_one)
 
 
+def iter_params_threaded(cfg, seed=0, std=0.02, gains_one=True, workers=8, transform=None):
+    """iter_params with the tensors generated (and passed through `transform(name, array)`, e.g. a bf16 rounding) by a
+    pool of threads a few tensors ahead of the consumer; same bytes, same order (every tensor has its own stream)."""
+    from collections import deque
+    from concurrent.futures import ThreadPoolExecutor
+
+    def job(name, shape):
+        a = make_param(name, shape, seed, std, gains_one)
+        return name, (transform(name, a) if transform else a)
+
+    todo = iter(param_shapes(cfg).items())
+    with ThreadPoolExecutor(max(1, workers)) as pool:
+        ahead = deque()
+        for name, shape in todo:
+            ahead.append(pool.submit(job, name, shape))
+            if len(ahead) >= 2 * workers:
+                yield ahead.popleft().result()
+        while ahead:
+            yield ahead.popleft().result()
+
+
 def make_params(cfg, seed=0, std=0.02, gains_one=True):
     return dict(iter_params(cfg, seed, std, gains_one))
 

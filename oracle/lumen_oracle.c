@@ -550,6 +550,21 @@ int lo_llama_kv_len(const lo_llama *m) { return m->caches[0]->len; }
 const float *lo_llama_cache_k(const lo_llama *m, int layer) { return m->caches[layer]->k; }
 const float *lo_llama_cache_v(const lo_llama *m, int layer) { return m->caches[layer]->v; }
 
+/* KVCacheInner's k, v and len are public fields (self_attention.rs:24-31): a caller may fill a cache with rows
+ * computed elsewhere and go on from there.  k, v: [1, Hkv, max_seq, D]; only rows [0, len) are copied. */
+int lo_llama_set_kv(lo_llama *m, int layer, const float *k, const float *v, int len) {
+    if (layer < 0 || layer >= m->cfg.num_hidden_layers) return LO_ERR_CACHE_COUNT;
+    lo_kv_cache *c = m->caches[layer];
+    if (len < 0 || len > c->max_seq) return LO_ERR_KV_OVERFLOW;
+    for (int h = 0; h < c->h_kv; ++h) {
+        const size_t off = (size_t)h * c->max_seq * c->d;
+        memcpy(c->k + off, k + off, sizeof(float) * (size_t)len * c->d);
+        memcpy(c->v + off, v + off, sizeof(float) * (size_t)len * c->d);
+    }
+    c->len = len;
+    return LO_OK;
+}
+
 int lo_llama_forward(lo_llama *m, const float *ids, int s, float *logits) {
     const lo_llama_config *cfg = &m->cfg;
     const int H = cfg->hidden_size, I = cfg->intermediate_size, V = cfg->vocab_size;

@@ -135,6 +135,8 @@ void lo_llama_reset(lo_llama *m);
 int lo_llama_kv_len(const lo_llama *m);
 const float *lo_llama_cache_k(const lo_llama *m, int layer);
 const float *lo_llama_cache_v(const lo_llama *m, int layer);
+/* fills a layer's cache with rows computed elsewhere (k, v [1, Hkv, max_seq, D], rows [0, len)) and sets its length */
+int lo_llama_set_kv(lo_llama *m, int layer, const float *k, const float *v, int len);
 /* ids as f32 like the reference (main.rs:143-152); logits [S, V] for all
  * positions (llama.rs:205) */
 int lo_llama_forward(lo_llama *m, const float *ids, int s, float *logits);

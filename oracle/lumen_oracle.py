@@ -96,6 +96,7 @@ _sig("lo_llama_reset", None, C.c_void_p)
 _sig("lo_llama_kv_len", C.c_int, C.c_void_p)
 _sig("lo_llama_cache_k", _f, C.c_void_p, C.c_int)
 _sig("lo_llama_cache_v", _f, C.c_void_p, C.c_int)
+_sig("lo_llama_set_kv", C.c_int, C.c_void_p, C.c_int, _f, _f, C.c_int)
 _sig("lo_llama_forward", C.c_int, C.c_void_p, _f, C.c_int, _f)
 
 
@@ -310,6 +311,15 @@ class Llama:
         d = cfg.get("head_dim") or cfg["hidden_size"] // cfg["num_attention_heads"]
         return np.ctypeslib.as_array(_lib.lo_llama_cache_v(self._m, layer),
                                      shape=(1, cfg["num_key_value_heads"], cfg["max_seq_len"], d))
+
+    def set_kv(self, layer, k, v, length):
+        """Fills a layer's cache with rows computed elsewhere (k, v [1, Hkv, max_seq, D]) and sets its length:
+        the fields of KVCacheInner are public (self_attention.rs:24-31)."""
+        k, v = np.ascontiguousarray(k, np.float32), np.ascontiguousarray(v, np.float32)
+        cfg = self.cfg
+        d = cfg.get("head_dim") or cfg["hidden_size"] // cfg["num_attention_heads"]
+        assert k.shape == v.shape == (1, cfg["num_key_value_heads"], cfg["max_seq_len"], d)
+        return _lib.lo_llama_set_kv(self._m, layer, _p(k), _p(v), int(length))
 
     def forward(self, ids):
         """ids: sequence of token ids (cast to f32 like main.rs:143-152).

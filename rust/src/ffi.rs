@@ -126,6 +126,7 @@ extern "C" {
     pub fn lumen_llama_get_decode_mode(model: *const lumen_llama, mode_out: *mut c_int) -> c_int;
     pub fn lumen_llama_reset(model: *mut lumen_llama) -> c_int;
     pub fn lumen_llama_kv_len(model: *const lumen_llama, len_out: *mut c_int) -> c_int;
+    pub fn lumen_llama_set_kv_len(model: *mut lumen_llama, len: c_int) -> c_int;
     pub fn lumen_llama_cache_download(model: *mut lumen_llama, layer: c_int, k_host: *mut c_float, v_host: *mut c_float) -> c_int;
     pub fn lumen_llama_decode_bytes(model: *const lumen_llama, len: c_int, bytes_out: *mut f64) -> c_int;
 }

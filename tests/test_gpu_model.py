@@ -494,20 +494,36 @@ def test_tinyllama_1b_shape_prefill_128_decode_teacher_forced():
 
 
 def _stream_build(cfg, seed, bf16=False):
-    """Full-width shapes: tensors are generated one at a time and shared by the GPU model and the oracle."""
+    """Full-width shapes: tensors are generated a few at a time (by a pool of threads) and shared by the GPU model
+    and the oracle; bf16-stored weights go to the GPU as bits and to the oracle as the same values widened."""
     gcfg = dict(cfg, weight_dtype="bf16") if bf16 else dict(cfg)
     gpu = LlamaModel(gcfg)
     params = {}
-    for name, a in synth.iter_params(cfg, seed=seed):
-        if bf16 and a.ndim == 2:
-            bits = synth.bf16_round(a)
-            a = synth.bf16_widen(bits)
+
+    def to_bf16(name, a):
+        if a.ndim != 2:
+            return a
+        bits = synth.bf16_round(a)
+        return bits, synth.bf16_widen(bits)
+
+    for name, a in synth.iter_params_threaded(cfg, seed=seed, workers=12, transform=to_bf16 if bf16 else None):
+        if isinstance(a, tuple):
+            bits, a = a
             gpu.set_param(name, a if name == "model.embed_tokens.weight" and not cfg.get("tie_embeddings") else bits)
         else:
             gpu.set_param(name, a)
         params[name] = a
     ocfg = {k: v for k, v in cfg.items() if k != "weight_dtype"}
     return gpu, lo.Llama(ocfg, params)
+
+
+def _seed_checker_with_gpu_cache(gpu, ora, length):
+    """The checker goes on from the rows the GPU's prompt pass left: its own prompt pass at these sizes would take
+    minutes.  (What the rows hold is then checked through what the checker computes FROM them.)"""
+    for layer in range(gpu.config.num_hidden_layers):
+        k, v = gpu.cache(layer)
+        assert ora.set_kv(layer, k, v, length) == lo.LO_OK
+    assert ora.kv_len == length
 
 
 def _prefill_decode_check(gpu, ora, vocab, n_prompt, n_dec, tol, seed):
@@ -582,3 +598,85 @@ def test_wide_model_prompt_of_4000_rows_on_the_large_gemm_tiles(bf16, tol):
     gpu, ora = _stream_build(cfg, seed=6, bf16=bf16)
     _prefill_decode_check(gpu, ora, cfg["vocab_size"], 4000, 2, tol, seed=6)
 
+
+
+@pytest.mark.slow
+def test_long_context_tinyllama_shape_at_full_depth_to_the_last_row():
+    """Config 3 as configured: all 22 layers, 3968-token prompt, decode to row 4095 of the 4096-row cache.
+    The checker does not repeat the prompt pass (minutes on the CPU): its caches are filled with the first 3967
+    rows the GPU's prompt pass wrote, and from there everything is its own arithmetic --
+    * its decode step for prompt token 3967 against the LAST ROW of the GPU's prompt pass (matrix-core kernels),
+    * 16 teacher-forced decode steps and ONE greedy call of 112 steps up to the last row (GEMV / attention kernels),
+      every step's logits within 1e-4,
+    * the cache rows both sides appended in the last layer."""
+    cfg = dict(synth.TINYLLAMA_1B_LONG)
+    gpu, ora = _stream_build(cfg, seed=0)
+    n_prompt, n_forced = 3968, 16
+    ids = synth.make_tokens(n_prompt + n_forced, cfg["vocab_size"], seed=0)
+    last = gpu.forward(ids[:n_prompt], all_rows=False)
+    _seed_checker_with_gpu_cache(gpu, ora, n_prompt - 1)
+    _, r = ora.forward(ids[n_prompt - 1:n_prompt])
+    assert max_rel(last, r[0]) <= 1e-4, max_rel(last, r[0])
+    check_argmax(last, r[0], 1e-4)
+    worst = 0.0
+    for t in range(n_prompt, n_prompt + n_forced):
+        g = gpu.forward(ids[t:t + 1], all_rows=False)
+        _, r = ora.forward(ids[t:t + 1])
+        worst = max(worst, max_rel(g, r[0]))
+        check_argmax(g, r[0], 1e-4)
+    assert worst <= 1e-4, worst
+    _greedy_call_checked(gpu, ora, lo.argmax(r[0]), cfg["max_seq_len"] - n_prompt - n_forced, 1e-4)
+    assert gpu.kv_len == ora.kv_len == cfg["max_seq_len"]
+    k, v = gpu.cache(cfg["num_hidden_layers"] - 1)
+    lo_k, lo_v = ora.cache_k(cfg["num_hidden_layers"] - 1), ora.cache_v(cfg["num_hidden_layers"] - 1)
+    assert max_rel(k[:, :, n_prompt - 1:], lo_k[:, :, n_prompt - 1:]) <= 1e-4
+    assert max_rel(v[:, :, n_prompt - 1:], lo_v[:, :, n_prompt - 1:]) <= 1e-4
+    with pytest.raises(_lib.LumenError) as e:
+        gpu.decode_greedy(1, 1)
+    assert e.value.status == _lib.ERR_KV_OVERFLOW
+
+
+@pytest.mark.slow
+def test_llama2_7b_shape_bf16_weights_at_full_depth():
+    """Config 5 as configured: all 32 layers (13 GB of bf16 weights on the GPU, the same values widened to f32 --
+    26 GB of host memory -- for the checker), 512-token prompt, decode across 512 -> 576 cached rows.
+    * checker (caches filled with the GPU's first 511 rows, then its own arithmetic): its decode step for prompt
+      token 511 against the last row of the GPU's prompt pass, and 12 steps of ONE greedy call, within 2e-2;
+    * the two GPU paths against each other at every one of 64 steps: logits of decode step t (GEMV / attention
+      kernels) against the last row of a prompt pass over the same t + 1 tokens (matrix-core kernels);
+    * graph replay against eager launches of the same 64 steps: the same bits."""
+    cfg = dict(synth.LLAMA2_7B)
+    cfg.pop("weight_dtype")
+    gpu, ora = _stream_build(cfg, seed=5, bf16=True)
+    n_prompt, n = 512, 64
+    ids = synth.make_tokens(n_prompt, cfg["vocab_size"], seed=5)
+    last = gpu.forward(ids, all_rows=False)
+    _seed_checker_with_gpu_cache(gpu, ora, n_prompt - 1)
+    _, r = ora.forward(ids[n_prompt - 1:])
+    assert max_rel(last, r[0]) <= 2e-2, max_rel(last, r[0])
+    check_argmax(last, r[0], 2e-2)
+    first = int(np.argmax(last))
+    picks, logits = gpu.decode_greedy(first, n, want_logits=True)
+    assert gpu.kv_len == n_prompt + n
+    tok, worst = first, 0.0
+    for t in range(12):
+        _, r = ora.forward(np.array([tok]))
+        worst = max(worst, max_rel(logits[t], r[0]))
+        check_argmax(logits[t], r[0], 2e-2)
+        tok = int(picks[t])
+    assert worst <= 2e-2, worst
+    # eager launches of the same steps
+    gpu.set_decode_mode("eager")
+    gpu.reset_kv_caches()
+    assert np.array_equal(gpu.forward(ids, all_rows=False), last)
+    picks_e, logits_e = gpu.decode_greedy(first, n, want_logits=True)
+    gpu.set_decode_mode("graph")
+    assert np.array_equal(picks_e, picks) and np.array_equal(logits_e, logits)
+    # decode step t against a prompt pass over the same t + 1 tokens
+    seq = np.concatenate([ids, [first], picks]).astype(np.int32)
+    cross = 0.0
+    for t in range(n):
+        gpu.reset_kv_caches()
+        row = gpu.forward(seq[:n_prompt + t + 1], all_rows=False)
+        cross = max(cross, max_rel(logits[t], row))
+    assert cross <= 1e-3, cross

@@ -104,3 +104,25 @@ def test_overflow_and_oob_status():
     assert m.forward(ids[:1])[0] == lo.LO_ERR_KV_OVERFLOW  # self_attention.rs:144-149
     m.reset()
     assert m.forward(np.array([TINY["vocab_size"]]))[0] == lo.LO_ERR_EMBED_OOB  # embedding.rs:55
+
+
+def test_a_cache_filled_from_outside_continues_bit_exactly():
+    """lo_llama_set_kv: a second model whose caches are filled with the first one's rows (and nothing of its own
+    prompt pass) decodes the same bits; rows beyond the given length are not taken; bad arguments are refused."""
+    params = synth.make_params(TINY, seed=9, std=0.1, gains_one=False)
+    a, b = lo.Llama(TINY, params), lo.Llama(TINY, params)
+    ids = synth.make_tokens(30, TINY["vocab_size"], seed=9)
+    a.forward(ids[:21])
+    for layer in range(TINY["num_hidden_layers"]):
+        k, v = a.cache_k(layer).copy(), a.cache_v(layer).copy()
+        k[:, :, 21:], v[:, :, 21:] = 7.0, 7.0   # must not be copied
+        assert b.set_kv(layer, k, v, 21) == lo.LO_OK
+        assert np.array_equal(b.cache_k(layer), a.cache_k(layer)) and np.array_equal(b.cache_v(layer), a.cache_v(layer))
+    assert b.kv_len == 21
+    for t in range(21, 30):
+        _, la = a.forward(ids[t:t + 1])
+        _, lb = b.forward(ids[t:t + 1])
+        assert np.array_equal(la, lb)
+    k = a.cache_k(0)
+    assert b.set_kv(TINY["num_hidden_layers"], k, k, 1) == lo.LO_ERR_CACHE_COUNT
+    assert b.set_kv(0, k, k, TINY["max_seq_len"] + 1) == lo.LO_ERR_KV_OVERFLOW
