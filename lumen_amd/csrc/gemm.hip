@@ -412,7 +412,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(GemmArgs a, int
     constexpr int R = 2, U = 4;
     constexpr int PIECE = SWEEP * U;
     constexpr int ESZ = BF16 ? 2 : 4;
-    extern __shared__ __align__(16) float As[];  // [MS][kpad]
+    LUMEN_DYNAMIC_LDS(float, As);  // [MS][kpad]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int M = a.M, N = a.N, K = a.K;
     const int m0 = blockIdx.y * MS;

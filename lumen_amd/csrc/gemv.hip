@@ -244,7 +244,7 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W
     // are in scalar registers when a wavefront starts and its first loads do not wait for a read of the
     // argument block.  XB: how x is staged -- 1 piece at a time, 4 at a time, or 0: requested ahead of the
     // weights (request_early).
-    extern __shared__ __align__(16) float xs[];
+    LUMEN_DYNAMIC_LDS(float, xs);
     constexpr int VEC = BF16 ? 8 : 4;          // elements per 16-byte load
     constexpr int SWEEP = 64 * VEC;            // elements one wavefront covers per load
     constexpr int U = 8 / R;                   // loads in flight per lane per row

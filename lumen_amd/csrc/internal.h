@@ -11,6 +11,11 @@
 
 #include "../../include/lumen_hip.h"
 
+// The dynamically sized LDS array of a kernel (one per kernel, sized by the launch)
+#ifndef LUMEN_DYNAMIC_LDS
+#define LUMEN_DYNAMIC_LDS(type, name) extern __shared__ __align__(16) type name[]
+#endif
+
 // ---------------------------------------------------------------- errors
 void lumen_set_error(const char *fmt, ...);
 
