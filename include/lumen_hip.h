@@ -345,9 +345,14 @@ int lumen_llama_reset(lumen_llama *model);                      /* reset_kv_cach
 int lumen_llama_kv_len(const lumen_llama *model, int *len_out);
 /* len of every layer's cache at once (a public field of the reference's KVCacheInner, self_attention.rs:28): go
  * back to an earlier length -- the rows beyond it are overwritten by the steps that follow -- e.g. to decode the
- * same positions again.  Outside [0, current length] -> LUMEN_ERR_KV_OVERFLOW (rows never written cannot be claimed). */
+ * same positions again, or say how many rows of caches filled with lumen_llama_cache_upload are valid.
+ * Outside [0, max_seq_len] -> LUMEN_ERR_KV_OVERFLOW. */
 int lumen_llama_set_kv_len(lumen_llama *model, int len);
 int lumen_llama_cache_download(lumen_llama *model, int layer, float *k_host, float *v_host);
+/* the other direction: a layer's cache rows from host memory, k and v [1, H_kv, max_seq, D] (k, v and len are public
+ * fields of the reference's KVCacheInner, self_attention.rs:24-31: a caller may fill a cache itself and then say
+ * how many rows are valid with lumen_llama_set_kv_len) */
+int lumen_llama_cache_upload(lumen_llama *model, int layer, const float *k_host, const float *v_host);
 /* bytes of weights + KV prefix one decode step at cache length len must read */
 int lumen_llama_decode_bytes(const lumen_llama *model, int len, double *bytes_out);
 

@@ -116,6 +116,7 @@ SIGNATURES = {
     "lumen_llama_kv_len": (_i, [_vp, C.POINTER(_i)]),
     "lumen_llama_set_kv_len": (_i, [_vp, _i]),
     "lumen_llama_cache_download": (_i, [_vp, _i, _vp, _vp]),
+    "lumen_llama_cache_upload": (_i, [_vp, _i, _vp, _vp]),
     "lumen_llama_decode_bytes": (_i, [_vp, _i, C.POINTER(C.c_double)]),
 }
 

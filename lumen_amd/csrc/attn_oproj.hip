@@ -95,6 +95,8 @@ __global__ __launch_bounds__(AO_THREADS) void attn_oproj_kernel(const void *Wo_h
                                                                 AttnOprojArgs a_mem) {
     constexpr int VEC = BF16 ? 8 : 4;
     constexpr int ESZ = BF16 ? 2 : 4;
+    constexpr int PW = 1;  // rotation pairs per wavefront of the q|k|v role, rows per wavefront of the o_proj role (two of
+                           // each -- half the workgroups in those roles -- measured slower: 0.895 against 0.845 ms per token)
     constexpr int K = NLO * 64 * VEC;  // o_proj row length = hq * D
     constexpr int KQ = NLQ * 64 * VEC;  // q|k|v row length = hidden
     constexpr int EPT = K / AO_THREADS;
@@ -113,16 +115,17 @@ __global__ __launch_bounds__(AO_THREADS) void attn_oproj_kernel(const void *Wo_h
         tagged_store(a_mem.t0_tagged, __uint_as_float(t_start), *step_dev_hot * a_mem.tag_mul + a_mem.tag_add);
     const int hq = hq_hot, hkv = hkv_slices_hot & 0xffff, S = hkv_slices_hot >> 16, N = N_hot;  // S: attention slices
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int n_o = (N + AO_WAVES - 1) / AO_WAVES;  // o_proj workgroups
+    const int n_o = (N + AO_WAVES * PW - 1) / (AO_WAVES * PW);  // o_proj workgroups
     constexpr int HALF = D / 2;
-    const int nunits = QKV ? (hq + 2 * hkv) * HALF : 0;  // rotation pairs; a multiple of 8: D / 2 is
-    const int nq = nunits / AO_WAVES;                    // q|k|v workgroups
+    const int nunits = QKV ? (hq + 2 * hkv) * HALF : 0;  // rotation pairs; a multiple of 16: D / 2 is
+    const int nq = nunits / (AO_WAVES * PW);             // q|k|v workgroups
     int blk = blockIdx.x;
     if (QKV && blk < nq) {
         // ---- RMSNorm + q|k|v + RoPE: one pair of rows (j, j + D/2) of one head per wavefront
         constexpr int XP = (KQ / 4 + AO_THREADS - 1) / AO_THREADS;  // 16-byte pieces of x a thread stages
-        const int unit = blk * AO_WAVES + wave;
-        const int head = unit / HALF, j = unit % HALF;
+        const int unit = (blk * AO_WAVES + wave) * PW;
+        const int hh = unit / HALF, j = unit % HALF;  // PW pairs j, j + 1 of one head: adjacent rows
+        const int head = hh;
         const float *x = x_hot;
         if (a_mem.row_sel) x += (long)(*a_mem.row_sel) * a_mem.row_stride;  // (first layer: a trip of its own)
         // x and the gains first: what is requested first arrives first, and the norm is what the multiplies wait for
@@ -137,19 +140,26 @@ __global__ __launch_bounds__(AO_THREADS) void attn_oproj_kernel(const void *Wo_h
                 ge[i] = *(const v4f *)(in_norm_hot + k);
             }
         }
-        v4u raw[2][NLQ];
+        v4u raw[PW][2][NLQ];
 #pragma unroll
-        for (int r = 0; r < 2; ++r) {
-            const char *rp = (const char *)Wqkv_hot + ((size_t)(head * D + j + r * HALF) * KQ + (size_t)lane * VEC) * ESZ;
+        for (int p = 0; p < PW; ++p)
 #pragma unroll
-            for (int i = 0; i < NLQ; ++i) raw[r][i] = __builtin_nontemporal_load((const v4u *)(rp + (size_t)i * 64 * VEC * ESZ));
-        }
+            for (int r = 0; r < 2; ++r) {
+                const char *rp = (const char *)Wqkv_hot + ((size_t)(head * D + j + p + r * HALF) * KQ + (size_t)lane * VEC) * ESZ;
+#pragma unroll
+                for (int i = 0; i < NLQ; ++i) raw[p][r][i] = __builtin_nontemporal_load((const v4u *)(rp + (size_t)i * 64 * VEC * ESZ));
+            }
         const int pos = *pos_dev_hot;
         const unsigned tag = *step_dev_hot * a_mem.tag_mul + a_mem.tag_add;
-        float cs = 1.f, sn = 0.f;
-        if (QKV == 1) {
-            cs = a_mem.attn.cos_t[(size_t)pos * D + j];
-            sn = a_mem.attn.sin_t[(size_t)pos * D + j];
+        float cs[PW], sn[PW];
+#pragma unroll
+        for (int p = 0; p < PW; ++p) {
+            cs[p] = 1.f;
+            sn[p] = 0.f;
+            if (QKV == 1) {
+                cs[p] = a_mem.attn.cos_t[(size_t)pos * D + j + p];
+                sn[p] = a_mem.attn.sin_t[(size_t)pos * D + j + p];
+            }
         }
         STAGE_T(1);
         // (x * inv_rms) * g, src/layers/norm/rms_norm.rs:45-58
@@ -177,31 +187,34 @@ __global__ __launch_bounds__(AO_THREADS) void attn_oproj_kernel(const void *Wo_h
         }
         __syncthreads();
         STAGE_T(2);
-        float acc0 = 0.f, acc1 = 0.f;
 #pragma unroll
-        for (int i = 0; i < NLQ; ++i) {
-            acc0 += ao_dot16<BF16>(raw[0][i], xs + (i * 64 + lane) * VEC);
-            acc1 += ao_dot16<BF16>(raw[1][i], xs + (i * 64 + lane) * VEC);
-        }
-        acc0 = wave_sum(acc0);
-        acc1 = wave_sum(acc1);
-        if (lane == 0) {
-            // half-split rotation at the token's position (src/layers/attention/encoding.rs:196-203)
-            float o1 = acc0, o2 = acc1;
-            if (QKV == 1 && head < hq + hkv) {
-#pragma clang fp contract(off)
-                o1 = acc0 * cs - acc1 * sn;
-                o2 = acc0 * sn + acc1 * cs;
+        for (int p = 0; p < PW; ++p) {
+            float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+            for (int i = 0; i < NLQ; ++i) {
+                acc0 += ao_dot16<BF16>(raw[p][0][i], xs + (i * 64 + lane) * VEC);
+                acc1 += ao_dot16<BF16>(raw[p][1][i], xs + (i * 64 + lane) * VEC);
             }
-            unsigned long long *t = a_mem.qkv_tagged + (size_t)head * D + j;
-            tagged_store(t, o1, tag);
-            tagged_store(t + HALF, o2, tag);
-            if (QKV == 1 && head >= hq) {  // key / value of the new token: cache row pos
-                float *cache = head < hq + hkv ? k_cache_hot : v_cache_hot;
-                const int hk = head < hq + hkv ? head - hq : head - hq - hkv;
-                float *dst = cache + ((size_t)hk * max_seq_hot + pos) * D;
-                dst[j] = o1;
-                dst[j + HALF] = o2;
+            acc0 = wave_sum(acc0);
+            acc1 = wave_sum(acc1);
+            if (lane == 0) {
+                // half-split rotation at the token's position (src/layers/attention/encoding.rs:196-203)
+                float o1 = acc0, o2 = acc1;
+                if (QKV == 1 && head < hq + hkv) {
+#pragma clang fp contract(off)
+                    o1 = acc0 * cs[p] - acc1 * sn[p];
+                    o2 = acc0 * sn[p] + acc1 * cs[p];
+                }
+                unsigned long long *t = a_mem.qkv_tagged + (size_t)head * D + j + p;
+                tagged_store(t, o1, tag);
+                tagged_store(t + HALF, o2, tag);
+                if (QKV == 1 && head >= hq) {  // key / value of the new token: cache row pos
+                    float *cache = head < hq + hkv ? k_cache_hot : v_cache_hot;
+                    const int hk = head < hq + hkv ? head - hq : head - hq - hkv;
+                    float *dst = cache + ((size_t)hk * max_seq_hot + pos) * D;
+                    dst[j + p] = o1;
+                    dst[j + p + HALF] = o2;
+                }
             }
         }
         STAGE_T_STORES_DONE(3);
@@ -301,7 +314,7 @@ __global__ __launch_bounds__(AO_THREADS) void attn_oproj_kernel(const void *Wo_h
     }
     if (blk < n_o) {
         // ---- o_proj: one row per wavefront, all of its weights requested at once (rows past N: clamped, not stored)
-        const int row = blk * AO_WAVES + wave;
+        const int row = (blk * AO_WAVES + wave) * PW;
         // (see the head of the file; counted from the launch's start where that is known: with long caches these
         // workgroups wait for a free slot first, and a pause counted from their own start would begin too late)
         unsigned t_ref = t_start;
@@ -310,16 +323,19 @@ __global__ __launch_bounds__(AO_THREADS) void attn_oproj_kernel(const void *Wo_h
             if ((unsigned)(w0 >> 32) == *step_dev_hot * a_mem.tag_mul + a_mem.tag_add) t_ref = (unsigned)w0;
         }
         handover_pause_until32(t_ref, a_mem.pre_sleep);
-        v4u raw[NLO];
-        {
-            const char *rp = (const char *)Wo_hot + ((size_t)min(row, N - 1) * K + (size_t)lane * VEC) * ESZ;
+        v4u raw[PW][NLO];
 #pragma unroll
-            for (int i = 0; i < NLO; ++i) raw[i] = __builtin_nontemporal_load((const v4u *)(rp + (size_t)i * 64 * VEC * ESZ));
+        for (int p = 0; p < PW; ++p) {
+            const char *rp = (const char *)Wo_hot + ((size_t)min(row + p, N - 1) * K + (size_t)lane * VEC) * ESZ;
+#pragma unroll
+            for (int i = 0; i < NLO; ++i) raw[p][i] = __builtin_nontemporal_load((const v4u *)(rp + (size_t)i * 64 * VEC * ESZ));
         }
         const unsigned tag = *step_dev_hot * a_mem.tag_mul + a_mem.tag_add;
         const float *residual = a_mem.residual;
         if (a_mem.row_sel) residual += (long)(*a_mem.row_sel) * a_mem.row_stride;
-        const float res = residual[min(row, N - 1)];
+        float res[PW];
+#pragma unroll
+        for (int p = 0; p < PW; ++p) res[p] = residual[min(row + p, N - 1)];
         STAGE_T(5);
         // the attention output: this thread's EPT words, polled until every one carries this launch's tag
         handover_pause_until(wall_clock64(), a_mem.poll_delay);
@@ -332,13 +348,16 @@ __global__ __launch_bounds__(AO_THREADS) void attn_oproj_kernel(const void *Wo_h
         }
         __syncthreads();
         STAGE_T(6);
-        float acc = 0.f;
 #pragma unroll
-        for (int i = 0; i < NLO; ++i) acc += ao_dot16<BF16>(raw[i], xs + (i * 64 + lane) * VEC);
-        acc = wave_sum(acc);
-        if (lane == 0 && row < N) {
-            const float hv = res + acc;  // src/ops/arithmetic.rs:48-51 via llama.rs:110
-            a_mem.y[row] = hv;
+        for (int p = 0; p < PW; ++p) {
+            float acc = 0.f;
+#pragma unroll
+            for (int i = 0; i < NLO; ++i) acc += ao_dot16<BF16>(raw[p][i], xs + (i * 64 + lane) * VEC);
+            acc = wave_sum(acc);
+            if (lane == 0 && row + p < N) {
+                const float hv = res[p] + acc;  // src/ops/arithmetic.rs:48-51 via llama.rs:110
+                a_mem.y[row + p] = hv;
+            }
         }
         STAGE_T_STORES_DONE(7);
     }
@@ -373,15 +392,15 @@ template <int D, bool BF16>
 static int launch_ao(lumen_ctx *ctx, const AttnOprojArgs &a) {
     const int nlo = ao_nl(a.K, BF16), nlq = a.Wqkv ? ao_nl(a.N, BF16) : 0;
     const int form = !a.Wqkv ? 0 : a.attn.q_norm_w ? 2 : 1;
-    const int nq = a.Wqkv ? (a.attn.hq + 2 * a.attn.hkv) * (D / 2) / AO_WAVES : 0;
     const int S = a.nslices > 1 ? a.nslices : 1;
+    const int nq = a.Wqkv ? (a.attn.hq + 2 * a.attn.hkv) * (D / 2) / AO_WAVES : 0;
     const int n_att = a.attn.hq * S + (S > 1 ? a.attn.hq : 0);  // attention workgroups, and those that fold the slices
     const int n_wg = nq + n_att + attn_oproj_workgroups(a.N);
     dim3 grid(n_wg), block(AO_THREADS);
     bool launched = false;
 #define AO_LAUNCH(NLQ, NLO, QKV)                                                                                                 \
     do {                                                                                                                         \
-        hipLaunchKernelGGL((attn_oproj_kernel<D, NLQ, NLO, BF16, QKV>), grid, block, 0, ctx->stream, a.Wo, a.attn.k_cache,       \
+        hipLaunchKernelGGL((attn_oproj_kernel<D, NLQ, NLO, BF16, QKV>), grid, block, 0, ctx->stream, a.Wo, a.attn.k_cache,   \
                            a.attn.v_cache, a.attn.q, a.attn.pos_dev, a.step_dev, a.attn.max_seq, a.attn.hq, a.attn.hkv | (S << 16), a.N, \
                            a.Wqkv, a.residual, a.in_norm_w, a);                                                                  \
         launched = true;                                                                                                         \

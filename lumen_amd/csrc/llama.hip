@@ -981,8 +981,8 @@ extern "C" int lumen_llama_reset(lumen_llama *m) {
 
 extern "C" int lumen_llama_set_kv_len(lumen_llama *m, int len) {
     if (!m) LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_set_kv_len: null model");
-    if (len < 0 || len > m->len)
-        LUMEN_FAIL(LUMEN_ERR_KV_OVERFLOW, "llama_set_kv_len: %d outside [0, %d]", len, m->len);
+    if (len < 0 || len > m->cfg.max_seq_len)
+        LUMEN_FAIL(LUMEN_ERR_KV_OVERFLOW, "llama_set_kv_len: %d outside [0, %d]", len, m->cfg.max_seq_len);
     HIP_TRY(hipSetDevice(m->ctx->device));
     m->len = len;
     return sync_pos_to_device(m);
@@ -1007,6 +1007,15 @@ extern "C" int lumen_llama_cache_download(lumen_llama *m, int layer, float *k_ho
     const size_t bytes = m->cache_stride * sizeof(float);
     LUMEN_TRY(lumen_download(m->ctx, k_host, m->k_slab + m->cache_stride * layer, bytes));
     return lumen_download(m->ctx, v_host, m->v_slab + m->cache_stride * layer, bytes);
+}
+
+extern "C" int lumen_llama_cache_upload(lumen_llama *m, int layer, const float *k_host, const float *v_host) {
+    if (!m || !k_host || !v_host) LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_cache_upload: null argument");
+    if (layer < 0 || layer >= m->cfg.num_hidden_layers)
+        LUMEN_FAIL(LUMEN_ERR_CACHE_COUNT, "KV cache index %d outside [0,%d)", layer, m->cfg.num_hidden_layers);
+    const size_t bytes = m->cache_stride * sizeof(float);
+    LUMEN_TRY(lumen_upload(m->ctx, m->k_slab + m->cache_stride * layer, k_host, bytes));
+    return lumen_upload(m->ctx, m->v_slab + m->cache_stride * layer, v_host, bytes);
 }
 
 extern "C" int lumen_llama_decode_bytes(const lumen_llama *m, int len, double *bytes_out) {

@@ -132,6 +132,15 @@ class LlamaModel:
         check(lib.lumen_llama_cache_download(self.handle, layer, k.ctypes.data, v.ctypes.data))
         return k, v
 
+    def set_cache(self, layer, k, v):
+        """A layer's cache rows from host arrays [1, H_kv, max_seq, D] (public fields of KVCacheInner,
+        self_attention.rs:24-31); set_kv_len then says how many rows are valid."""
+        k, v = np.ascontiguousarray(k, np.float32), np.ascontiguousarray(v, np.float32)
+        cfg = self.config
+        d = cfg.head_dim or cfg.hidden_size // cfg.num_attention_heads
+        assert k.shape == v.shape == (1, cfg.num_key_value_heads, cfg.max_seq_len, d)
+        check(lib.lumen_llama_cache_upload(self.handle, int(layer), k.ctypes.data, v.ctypes.data))
+
     # -- forward ----------------------------------------------------------------
     def forward(self, input_ids, caches=None, _pos=0, all_rows=True):
         """llama.rs:181-206.  input_ids: token ids (any numeric dtype; they travel as f32 like

@@ -128,6 +128,7 @@ extern "C" {
     pub fn lumen_llama_kv_len(model: *const lumen_llama, len_out: *mut c_int) -> c_int;
     pub fn lumen_llama_set_kv_len(model: *mut lumen_llama, len: c_int) -> c_int;
     pub fn lumen_llama_cache_download(model: *mut lumen_llama, layer: c_int, k_host: *mut c_float, v_host: *mut c_float) -> c_int;
+    pub fn lumen_llama_cache_upload(model: *mut lumen_llama, layer: c_int, k_host: *const c_float, v_host: *const c_float) -> c_int;
     pub fn lumen_llama_decode_bytes(model: *const lumen_llama, len: c_int, bytes_out: *mut f64) -> c_int;
 }
 
