@@ -349,7 +349,7 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W
     else stage_x<PRO, (XB > 0 ? XB : 1)>(xs, xin, norm_w_hot, a.eps, K, kpad, nwaves);
     STAGE_T(2);
     float best = -INFINITY;
-    int best_idx = 0x7fffffff;
+    int best_idx = 0xffffff;  // (rows are below 2^24: the launcher checks)
 
     float acc[R];
 #pragma unroll
@@ -441,12 +441,19 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W
     STAGE_T(4);
     STAGE_T_STORES_DONE(5);
     if (EPI == EPI_ARGMAX) {
-        // greedy pick fused into the lm_head product: per-workgroup candidates go through memory with
-        // agent-scope accesses, the last workgroup to arrive folds them (lowest index wins ties)
+        // Greedy pick fused into the lm_head product.  Every workgroup leaves its candidate as ONE 8-byte word
+        // {value bits, tag << 24 | row}, stored with a single agent-scope atomic store; the workgroup with the highest
+        // index -- dispatched last, so every other one is resident or finished when it starts to wait -- polls the
+        // words of all workgroups until each carries this launch's tag, and folds them (lowest row wins ties).
+        // Value, row and tag are one atomic object: a reader that sees the tag has the candidate, whatever the order
+        // of other accesses (no counter, no fence).  The tag is 1 + (*epoch mod 255); every workgroup writes its word
+        // in every launch and the folding workgroup advances *epoch when it is done, so a word left by the launch
+        // before never carries the tag of this one.  The wait is bounded: after spin_limit polls the workgroup flags
+        // the failure in *err_dev, folds what it has and exits.
         __shared__ float am_v[GEMV_MAX_WAVES];
         __shared__ int am_i[GEMV_MAX_WAVES];
-        __shared__ int am_last;
         const int wave = threadIdx.x >> 6;
+        const unsigned tag = 1u + *a.amax_epoch % 255u;
         if (lane == 0) {
             am_v[wave] = best;
             am_i[wave] = best_idx;
@@ -458,28 +465,36 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W
                     best = am_v[w];
                     best_idx = am_i[w];
                 }
-            __hip_atomic_store(a.amax_val + blockIdx.x, best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(a.amax_idx + blockIdx.x, best_idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // (a workgroup without a row, or with NaNs only, leaves the row 0xffffff: never picked)
+            const unsigned long long word = ((unsigned long long)((tag << 24) | ((unsigned)best_idx & 0xffffffu)) << 32) |
+                                            (unsigned long long)__float_as_uint(best);
+            __hip_atomic_store(a.amax_word + blockIdx.x, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        handover_stores_done();
-        __syncthreads();
-        if (threadIdx.x == 0) {
-            const int old = handover_arrive(a.amax_counter);
-            am_last = (old == nblocks - 1);
-            if (am_last) __hip_atomic_store(a.amax_counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        __syncthreads();
-        if (!am_last) return;
+        if ((int)blockIdx.x != nblocks - 1) return;
         float bv = -INFINITY;
-        int bi = 0x7fffffff;
+        int bi = 0xffffff;
+        bool gave_up = false;
         for (int i = threadIdx.x; i < nblocks; i += nwaves * 64) {
-            const float v = __hip_atomic_load(a.amax_val + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const int ix = __hip_atomic_load(a.amax_idx + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            unsigned long long w;
+            unsigned spins = 0;
+            for (;;) {
+                w = __hip_atomic_load(a.amax_word + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if ((unsigned)(w >> 56) == tag) break;
+                if (++spins > a.spin_limit) {  // never in a healthy launch
+                    gave_up = true;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(2);
+            }
+            if ((unsigned)(w >> 56) != tag) continue;
+            const float v = __uint_as_float((unsigned)w);
+            const int ix = (int)((unsigned)(w >> 32) & 0xffffffu);
             if (v > bv || (v == bv && ix < bi)) {
                 bv = v;
                 bi = ix;
             }
         }
+        if (gave_up) __hip_atomic_store(a.err_dev, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) {
             const float ov = __shfl_xor(bv, off, 64);
@@ -501,7 +516,7 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W
                     bv = am_v[w];
                     bi = am_i[w];
                 }
-            if (bi == 0x7fffffff) bi = 0;  // all NaN: index 0 like a sequential scan
+            if (bi >= N) bi = 0;  // all NaN: index 0 like a sequential scan
             *a.tok_out = bi;
             if (a.pos_inc) {
                 const int pos = *a.pos_inc;
@@ -509,6 +524,7 @@ __global__ __launch_bounds__(GEMV_MAX_WAVES * 64) void gemv_kernel(const void *W
                 *a.pos_inc = pos + 1;
             }
             if (a.step_inc) *a.step_inc += 1;
+            *a.amax_epoch += 1;
         }
     }
 }
@@ -670,6 +686,13 @@ int launch_gemv(lumen_ctx *ctx, const GemvArgs &a) {
     }
     if ((a.epi == EPI_SWIGLU || a.epi == EPI_ROPE_QKV) && (a.N & 1))
         LUMEN_FAIL(LUMEN_ERR_SHAPE, "paired-row epilogue needs an even row count, got %d", a.N);
+    if (a.epi == EPI_ARGMAX) {
+        if (!a.amax_word || !a.amax_epoch || !a.err_dev || !a.tok_out || ((uintptr_t)a.amax_word & 7))
+            LUMEN_FAIL(LUMEN_ERR_INVALID, "arg-max epilogue: needs a candidate buffer, a launch counter and an error flag");
+        if (a.N >= (1 << 24))  // a candidate's row shares a word with its tag
+            LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED, "arg-max epilogue: %d rows (at most %d)", a.N, (1 << 24) - 1);
+        if (a.spin_limit > HANDOVER_MAX_SPINS) LUMEN_FAIL(LUMEN_ERR_INVALID, "arg-max epilogue: poll limit %u", a.spin_limit);
+    }
     const int threads = p.threads, blocks = p.blocks;
     const size_t lds = p.lds;
     dim3 grid(blocks);

@@ -108,11 +108,12 @@ struct GemvArgs {
     const int *row_sel;
     long row_stride;
     int x_sel, residual_sel;
-    // EPI_ARGMAX: y still receives the N values; the index of the first maximum goes to *tok_out
-    // and *pos_inc is incremented, by the last workgroup to finish
-    float *amax_val;   // [gridDim.x]
-    int *amax_idx;     // [gridDim.x]
-    int *amax_counter; // zero between launches
+    // EPI_ARGMAX (N < 2^24): y still receives the N values; the index of the first maximum goes to *tok_out and
+    // *pos_inc is incremented, by the workgroup with the highest index, which waits for the others' candidates
+    unsigned long long *amax_word;  // [gridDim.x] candidates {value, tag << 24 | row}, zero before the first launch
+    unsigned *amax_epoch;           // launches so far (the tag is made of it; advanced by the kernel)
+    int *err_dev;                   // set to 1 when the wait for the candidates ran into spin_limit
+    unsigned spin_limit;
     int *tok_out, *pos_inc;
     int *tok_hist;     // optional [max_seq + 1]: the pick is also stored at index *pos_inc + 1
     unsigned *step_inc;  // optional: decode step counter, incremented together with *pos_inc

@@ -70,9 +70,8 @@ struct lumen_llama {
     int chain_slice_trips = 0;                     // > 0: trips per slice fixed (measurements), else chosen by length
     unsigned long long *part_tagged = nullptr;     // [Hq][ATTN_CHAIN_MAX_SLICES][D + 2]
     int decode_mode = LUMEN_DECODE_GRAPH;
-    float *amax_val = nullptr;
-    int *amax_idx = nullptr;
-    int *amax_counter = nullptr;
+    unsigned long long *amax_word = nullptr;  // per-workgroup candidates of the lm_head product's arg-max
+    unsigned *amax_epoch = nullptr;
     // prefill buffers (grown on demand, kept)
     int pf_cap = 0, pf_logit_cap = 0;
     float *p_x = nullptr, *p_h = nullptr, *p_n = nullptr, *p_qkv = nullptr, *p_qrot = nullptr, *p_attn = nullptr,
@@ -254,13 +253,13 @@ extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg,
     }
     {
         const size_t nb = (size_t)std::max(gemv_max_blocks(ctx), ctx->num_cus);
-        M_TRY(dmalloc_t(m, &m->amax_val, nb));
-        M_TRY(dmalloc_t(m, &m->amax_idx, nb));
-        M_TRY(dmalloc_t(m, &m->amax_counter, 4));
-        if (hipMemsetAsync(m->amax_counter, 0, 4 * sizeof(int), ctx->stream) != hipSuccess ||
+        M_TRY(dmalloc_t(m, &m->amax_word, nb));
+        M_TRY(dmalloc_t(m, &m->amax_epoch, 4));
+        if (hipMemsetAsync(m->amax_word, 0, nb * sizeof(unsigned long long), ctx->stream) != hipSuccess ||
+            hipMemsetAsync(m->amax_epoch, 0, 4 * sizeof(unsigned), ctx->stream) != hipSuccess ||
             hipStreamSynchronize(ctx->stream) != hipSuccess) {
             lumen_llama_destroy(m);
-            LUMEN_FAIL(LUMEN_ERR_HIP, "llama_create: clearing the arg-max counter failed");
+            LUMEN_FAIL(LUMEN_ERR_HIP, "llama_create: clearing the arg-max candidates failed");
         }
     }
     m->decode_mode = LUMEN_DECODE_GRAPH;
@@ -618,7 +617,7 @@ static int enqueue_decode_step(lumen_llama *m, StepProbe *pr = nullptr) {
     g.w_bf16 = (m->lm_head == (void *)m->embed) ? 0 : (int)m->bf16;
     g.pro = PRO_RMSNORM; g.norm_w = m->final_norm; g.eps = c.rms_norm_eps;
     // the greedy pick is folded in: it becomes the next token id and the position counter advances
-    g.epi = EPI_ARGMAX; g.amax_val = m->amax_val; g.amax_idx = m->amax_idx; g.amax_counter = m->amax_counter;
+    g.epi = EPI_ARGMAX; g.amax_word = m->amax_word; g.amax_epoch = m->amax_epoch; g.err_dev = m->d_err; g.spin_limit = m->spin_limit;
     g.tok_out = m->d_tok; g.pos_inc = m->d_pos; g.tok_hist = m->tok_hist; g.step_inc = m->d_step;
     pr->before(KC_LMHEAD);
     const int rc = launch_gemv(ctx, g);
@@ -718,13 +717,12 @@ extern "C" int lumen_llama_get_decode_mode(const lumen_llama *m, int *mode_out) 
 
 // after a synchronisation: did a wait inside the attention -> o_proj chain run into its limit?
 static int check_handover(lumen_llama *m) {
-    if (!m->chain_ao && !(m->chain_mlp && m->chain_ao_on)) return LUMEN_OK;
     int err = 0;
     HIP_TRY(hipMemcpy(&err, m->d_err, sizeof(int), hipMemcpyDeviceToHost));
     if (!err) return LUMEN_OK;
     HIP_TRY(hipMemset(m->d_err, 0, sizeof(int)));
-    LUMEN_FAIL(LUMEN_ERR_HIP, "decode: a workgroup gave up waiting for a value handed over inside a chained "
-                              "launch (poll limit %u); the results of this call are invalid, reset the model", m->spin_limit);
+    LUMEN_FAIL(LUMEN_ERR_HIP, "decode: a workgroup gave up waiting for a value handed over inside a launch (poll "
+                              "limit %u); the results of this call are invalid, reset the model", m->spin_limit);
 }
 
 static int sync_pos_to_device(lumen_llama *m) {
