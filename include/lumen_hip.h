@@ -209,12 +209,17 @@ int lumen_attn_decode_prerotated_f32(lumen_kv_cache *cache, const float *q_rot_d
 /* The same decode step for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments,
  * same results, bit for bit, as lumen_attn_decode_f32, but the scratch that the slices of a long cache need
- * (per query head and slice a partial state of head_dim + 2 floats, plus one arrival counter per query head)
+ * (per query head and slice a partial state of head_dim + 2 values, each an 8-byte word {value, tag of the launch})
  * comes from a fixed 4 MiB array inside the library's device image instead of a hipMalloc at the first call:
- * this entry point calls no allocator.  batch x heads > 1024, or partial states beyond the array
- * (batch x heads x slices x (head_dim + 2) x 4 bytes > 4 MiB - 4 KiB; slices = ceil(max_seq / (16384 / head_dim))
- * rounded up to a power of two, 64 at most) -> LUMEN_ERR_UNSUPPORTED.  All calls on one GPU share that GPU's
- * array: calls that overlap in time on one GPU (two contexts, two streams) race; calls in stream order do not. */
+ * this entry point calls no allocator.  The launch count the tags are made of sits in the same array and is
+ * advanced by a one-thread kernel in front of the launch, so a call recorded into a graph is sound at every replay.
+ * Partial states beyond the array (batch x heads x slices x (head_dim + 2) x 8 bytes > 4 MiB - 256 bytes; slices =
+ * ceil(max_seq / (16384 / head_dim)) rounded up to a power of two, 64 at most) -> LUMEN_ERR_UNSUPPORTED.  All calls
+ * on one GPU share that GPU's array: calls that overlap in time on one GPU (two contexts, two streams) race; calls
+ * in stream order do not.
+ * Both entry points merge the slices inside the launch: the workgroup of a head's last slice waits (bounded) for
+ * the others' states; a wait that runs out is reported by the next lumen_ctx_synchronize / lumen_download on the
+ * context as LUMEN_ERR_HIP. */
 int lumen_attn_decode_static_f32(lumen_kv_cache *cache, lumen_rope *rope, const float *q3_dev,
                                  const float *k3_dev, const float *v3_dev, float *out_dev,
                                  int h, float scale, int causal);

@@ -48,8 +48,8 @@ __device__ __forceinline__ void long_slices(int pos, int nslices, int &nact, int
 }
 
 // One query head (r of KV group hk) over slice `slice` of nact: rows [slice * chunk, ...) of the cache.
-// The partial state (ctx[D], m, l) goes to a.part[head][slice]; the last workgroup of the head to
-// arrive (a.counters[head]) folds the nact partials: slice weights exp2(m_s - M) from wavefront 0
+// The partial state (ctx[D], m, l) goes to a.part_tagged[head][slice] as tagged words; the workgroup of the
+// last slice in use folds the nact partials: slice weights exp2(m_s - M) from wavefront 0
 // (lane s takes slice s), the D context elements by THREADS / D thread groups that each take every
 // (THREADS / D)-th slice, their sums added in group order.  !PRE: every workgroup rotates its own
 // query head; the last slice also rotates the new key, takes the new row from LDS, and its first
@@ -58,7 +58,7 @@ template <int D, int WAVES, bool PRE>
 __device__ __forceinline__ bool attn_decode_slice(const AttnDecodeArgs &a, int r, int nrep, int hk, int bb, int pos_new,
                                                   int slice, int nslices, bool fixed, int short_rows, float *q_rot,
                                                   float *k_new, float *v_new, float *sm, float *sl, float *sacc,
-                                                  float *w_lds, int *s_last) {
+                                                  float *w_lds) {
     constexpr int LPR = D / 4, RPW = 64 / LPR, RPI = WAVES * RPW, UB = ShortTrip<D>::loads, THREADS = WAVES * 64;
     constexpr int TRIP = RPI * UB, GROUPS = THREADS / D, JMAX = (64 + GROUPS - 1) / GROUPS;
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
@@ -172,44 +172,72 @@ __device__ __forceinline__ bool attn_decode_slice(const AttnDecodeArgs &a, int r
     wave_merge_publish<D, 1>(st, sm, sl, sacc);
     __syncthreads();
     float *out_head = a.out + ((size_t)bb * a.hq + hq) * D;
-    float *part_head = a.part + ((size_t)bb * a.hq + hq) * nslices * (D + 2);
+    const size_t part_off = ((size_t)bb * a.hq + hq) * nslices * (D + 2);
+    // a slice's state travels as tagged 8-byte words {value, tag} (attn_short_device.h) unless the consumer is a
+    // later launch (defer_merge: plain values in a.part)
+    unsigned long long *part_head = a.part_tagged + part_off;
+    const unsigned tag = (a.tag_dev ? *a.tag_dev : 0u) * a.tag_mul + a.tag_add;
     for (int dd = t; dd < D; dd += THREADS) {
         float mm, ls, cx;
         wave_fold<D, 1, WAVES>(sm, sl, sacc, 0, dd, mm, ls, cx);
         if (nact == 1 && !a.defer_merge) {
             out_head[dd] = cx * (1.0f / (ls + 1e-9f));  // self_attention.rs:287-290
-        } else {
-            float *pp = part_head + (size_t)slice * (D + 2);
-            part_store(pp + dd, cx);
+        } else if (a.defer_merge) {
+            float *pp = a.part + part_off + (size_t)slice * (D + 2);
+            pp[dd] = cx;
             if (dd == 0) {
-                part_store(pp + D, mm);
-                part_store(pp + D + 1, ls);
+                pp[D] = mm;
+                pp[D + 1] = ls;
+            }
+        } else {
+            unsigned long long *pp = part_head + (size_t)slice * (D + 2);
+            tagged_store(pp + dd, cx, tag);
+            if (dd == 0) {
+                tagged_store(pp + D, mm, tag);
+                tagged_store(pp + D + 1, ls, tag);
             }
         }
     }
     if (nact == 1 || a.defer_merge) return true;  // one slice, or the consumer folds them
-    // every wavefront's stores are acknowledged before the barrier, hence before thread 0's arrival (see handover_arrive)
-    handover_stores_done();
-    __syncthreads();
-    if (t == 0) {
-        int *counter = a.counters + (size_t)bb * a.hq + hq;
-        const int old = handover_arrive(counter);
-        *s_last = (old == nact - 1);
-        if (*s_last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __syncthreads();
-    if (!*s_last) return true;
-    // fold: context partials of this thread's element and slices first (one trip to memory) ...
+    // The workgroup of the last slice in use folds the slices of its head.  It has the highest index among them,
+    // so it is dispatched last and the others are resident or finished while it waits; it polls their words (and
+    // its own) until every one carries this launch's tag: a word that does has its value, whatever the order of
+    // other accesses.  The wait is bounded (spin_limit polls, then *err_dev = 1 and the fold goes on with what it has).
+    if (slice != nact - 1) return true;
+    // fold: context partials of this thread's element and slices, and the slice weights' inputs by wavefront 0
     const int dd = t % D, grp = t / D;
-    float cv[JMAX];
-    if (grp < GROUPS) {
+    unsigned long long wv[JMAX], wm = 0, wl = 0;
+    {
+        unsigned spins = 0;
+        bool ok;
+        do {
+            ok = true;
+            if (grp < GROUPS) {
 #pragma unroll
-        for (int j = 0; j < JMAX; ++j) cv[j] = part_load(part_head + (size_t)min(grp + j * GROUPS, nact - 1) * (D + 2) + dd);
+                for (int j = 0; j < JMAX; ++j) {
+                    wv[j] = tagged_load(part_head + (size_t)min(grp + j * GROUPS, nact - 1) * (D + 2) + dd);
+                    ok = ok && (unsigned)(wv[j] >> 32) == tag;
+                }
+            }
+            if (wave == 0) {
+                const unsigned long long *pp = part_head + (size_t)min(lane, nact - 1) * (D + 2);
+                wm = tagged_load(pp + D);
+                wl = tagged_load(pp + D + 1);
+                ok = ok && (unsigned)(wm >> 32) == tag && (unsigned)(wl >> 32) == tag;
+            }
+            if (!ok) {
+                if (++spins > a.spin_limit) break;  // never in a healthy launch: give up so that the wavefront exits
+                __builtin_amdgcn_s_sleep(2);
+            }
+        } while (!ok);
+        if (!ok && a.err_dev) __hip_atomic_store(a.err_dev, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    float cv[JMAX];
+#pragma unroll
+    for (int j = 0; j < JMAX; ++j) cv[j] = __uint_as_float((unsigned)wv[j]);
     // ... then the slice weights, by wavefront 0
     if (wave == 0) {
-        const float *pp = part_head + (size_t)min(lane, nact - 1) * (D + 2);
-        float m = part_load(pp + D), l = part_load(pp + D + 1);
+        float m = __uint_as_float((unsigned)wm), l = __uint_as_float((unsigned)wl);
         if (lane >= nact) {
             m = -INFINITY;
             l = 0.f;
@@ -266,7 +294,6 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
     // wavefront states [WAVES][D]; the fold of a long cache reuses it for one partial sum per thread
     __shared__ __align__(16) float sacc[WAVES * (D > 64 ? D : 64)];
     __shared__ float sm[WAVES], sl[WAVES], w_lds[65];
-    __shared__ int s_last;
 
     const int split = blockIdx.x, hk = blockIdx.y, bb = blockIdx.z;
     const int NREP = NREP_T ? NREP_T : a.hq / a.hkv;  // query heads per KV head
@@ -294,33 +321,23 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
     // workgroup's rows do not depend on the position and are requested before it is read
     const bool fixed = a.max_seq <= nslices * ShortTrip<D>::loads * G::RPI;
 
-    // The form follows the position where it is known (pos_host), the caller's hint where it sits in
-    // device memory: then the hinted form starts before the position is read and hands over to the
-    // other one if the hint was wrong.  One call site per form: two would let the compiler keep the
-    // first one's loaded rows alive for the second across everything in between.
+    // The form follows the position: the launcher knows it (pos_host, or its own mirror of the device counter) and
+    // passes the form to run, so the first trip of rows is requested before the position itself is read.  A form
+    // that then finds the cache on the other side of the boundary has been launched wrongly: it writes nothing and
+    // flags the launch as failed (*err_dev), which the next synchronising call reports.
     int pos_new = a.pos_dev ? -1 : a.pos_host;  // == past_len, the new token's position
-    bool want_short = start_short != 0;
-#pragma unroll 1
-    for (int attempt = 0; attempt < 2; ++attempt) {
-        if (want_short) {
-            if (r < NREP && attn_decode_short<D, WAVES, PRE ? ATTN_SRC_CACHE : ATTN_SRC_RAW>(a, r, NREP, hk, bb, pos_new, SHORT_ROWS, q_rot, k_new, v_new, sm, sl, sacc))
-                return;
-            if (pos_new < 0) pos_new = *a.pos_dev;
-            if (pos_new + 1 <= SHORT_ROWS) return;  // short indeed: not one of the short form's workgroups
-            want_short = false;
-        } else {
-            if (pos_new < 0 && !fixed) pos_new = *a.pos_dev;
-            if (pos_new >= 0 && pos_new + 1 <= SHORT_ROWS) {
-                want_short = true;
-                continue;
-            }
-            if (attn_decode_slice<D, WAVES, PRE>(a, rr, NREP, hk, bb, pos_new, slice, nslices, fixed, SHORT_ROWS, q_rot, k_new,
-                                                 v_new, sm, sl, sacc, w_lds, &s_last))
-                return;
-            pos_new = *a.pos_dev;  // the slice form found a short cache
-            want_short = true;
-        }
+    // (slices longer than a trip depend on the position: it is read first then)
+    if (start_short == 0 && pos_new < 0 && !fixed) pos_new = *a.pos_dev;
+    bool done;
+    if (start_short != 0) {
+        if (r >= NREP) return;  // not one of the short form's workgroups
+        done = attn_decode_short<D, WAVES, PRE ? ATTN_SRC_CACHE : ATTN_SRC_RAW>(a, r, NREP, hk, bb, pos_new, SHORT_ROWS, q_rot, k_new,
+                                                                                 v_new, sm, sl, sacc);
+    } else {
+        done = attn_decode_slice<D, WAVES, PRE>(a, rr, NREP, hk, bb, pos_new, slice, nslices, fixed, SHORT_ROWS, q_rot, k_new, v_new,
+                                                sm, sl, sacc, w_lds);
     }
+    if (!done && a.err_dev && threadIdx.x == 0) __hip_atomic_store(a.err_dev, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // slices of a long cache: one trip of rows each (16384 / head_dim rows: eight 16-byte loads per lane,
@@ -638,8 +655,7 @@ extern "C" int lumen_kv_cache_destroy(lumen_kv_cache *c) {
         hipFree(c->k);
         hipFree(c->v);
     }
-    hipFree(c->part);
-    hipFree(c->counters);
+    hipFree(c->part_tagged);
     hipFree(c->q_rot);
     hipFree(c->d_pos);
     delete c;
@@ -701,22 +717,21 @@ extern "C" int lumen_kv_cache_get_view(const lumen_kv_cache *c, int cur, float *
 }
 
 static int ensure_split_scratch(lumen_kv_cache *c, int hq, int nsplit) {
-    if (c->part && c->part_heads >= hq) return LUMEN_OK;
+    if (c->part_tagged && c->part_heads >= hq) return LUMEN_OK;
     hipStreamSynchronize(c->ctx->stream);
-    hipFree(c->part);
-    hipFree(c->counters);
-    c->part = nullptr;
-    c->counters = nullptr;
-    HIP_TRY(hipMalloc((void **)&c->part, sizeof(float) * attn_decode_part_floats(c->b, hq, c->d, nsplit)));
-    HIP_TRY(hipMalloc((void **)&c->counters, sizeof(int) * (size_t)c->b * hq));
-    HIP_TRY(hipMemsetAsync(c->counters, 0, sizeof(int) * (size_t)c->b * hq, c->ctx->stream));
+    hipFree(c->part_tagged);
+    c->part_tagged = nullptr;
+    const size_t bytes = sizeof(unsigned long long) * attn_decode_part_floats(c->b, hq, c->d, nsplit);
+    HIP_TRY(hipMalloc((void **)&c->part_tagged, bytes));
+    HIP_TRY(hipMemsetAsync(c->part_tagged, 0, bytes, c->ctx->stream));  // (no word carries a tag yet)
     c->part_heads = hq;
     return LUMEN_OK;
 }
 
 // The decode step of SelfAttention::forward behind both entry points: checks, launch, len += 1.
 static int attn_decode_entry(lumen_kv_cache *c, lumen_rope *rope, const float *q3, const float *k3, const float *v3,
-                             float *out, int h, float scale, float *part, int *counters, int nsplit) {
+                             float *out, int h, float scale, unsigned long long *part_tagged, const unsigned *tag_dev,
+                             unsigned tag_add, int nsplit) {
     const int past_len = c->len, new_len = past_len + 1;
     AttnDecodeArgs a = {};
     a.q = q3; a.k_new = k3; a.v_new = v3; a.out = out;
@@ -724,7 +739,8 @@ static int attn_decode_entry(lumen_kv_cache *c, lumen_rope *rope, const float *q
     a.pos_dev = nullptr; a.pos_host = past_len;
     a.b = c->b; a.hq = h; a.hkv = c->h_kv; a.d = c->d; a.max_seq = c->max_seq; a.scale = scale;
     a.q_norm_w = nullptr; a.k_norm_w = nullptr; a.norm_eps = 0.f;
-    a.part = part; a.counters = counters; a.nsplit = nsplit;
+    a.part_tagged = part_tagged; a.tag_dev = tag_dev; a.tag_mul = 1; a.tag_add = tag_add; a.nsplit = nsplit;
+    a.spin_limit = HANDOVER_MAX_SPINS; a.err_dev = c->ctx->err_host;
     LUMEN_TRY(launch_attn_decode(c->ctx, a));
     c->len = new_len;
     return LUMEN_OK;
@@ -749,7 +765,9 @@ extern "C" int lumen_attn_decode_f32(lumen_kv_cache *c, lumen_rope *rope, const 
     LUMEN_TRY(check_attn_decode(c, rope, q3, k3, v3, out, h));
     const int nsplit = attn_decode_nsplit(c->max_seq, c->d);
     LUMEN_TRY(ensure_split_scratch(c, h, nsplit));
-    return attn_decode_entry(c, rope, q3, k3, v3, out, h, scale, c->part, c->counters, nsplit);
+    // (the tag of this launch comes from the host: every call is a launch of its own with its own arguments)
+    if (++c->merge_epoch == 0) c->merge_epoch = 1;
+    return attn_decode_entry(c, rope, q3, k3, v3, out, h, scale, c->part_tagged, nullptr, c->merge_epoch, nsplit);
 }
 
 // ------------------------------------------------ the fused decode step of SelfAttention::forward, as two operators
@@ -796,21 +814,25 @@ extern "C" int lumen_attn_decode_prerotated_f32(lumen_kv_cache *c, const float *
     a.q = q_rot; a.out = out; a.k_cache = c->k; a.v_cache = c->v;
     a.pos_dev = nullptr; a.pos_host = c->len;
     a.b = c->b; a.hq = h; a.hkv = c->h_kv; a.d = c->d; a.max_seq = c->max_seq; a.scale = scale;
-    a.part = c->part; a.counters = c->counters; a.nsplit = nsplit; a.pre_rotated = 1;
+    if (++c->merge_epoch == 0) c->merge_epoch = 1;
+    a.part_tagged = c->part_tagged; a.tag_mul = 1; a.tag_add = c->merge_epoch; a.nsplit = nsplit; a.pre_rotated = 1;
+    a.spin_limit = HANDOVER_MAX_SPINS; a.err_dev = c->ctx->err_host;
     LUMEN_TRY(launch_attn_decode(c->ctx, a));
     c->len += 1;
     return LUMEN_OK;
 }
 
 // ------------------------------------------------ decode attention that allocates nothing
-// The slices of a long cache hand their partial states (ctx[D], m, l per query head and slice) and one arrival
-// counter per query head from workgroup to workgroup through device memory.  lumen_attn_decode_f32 keeps that
-// scratch on the cache object and allocates it at the first call; this variant takes it from a fixed array in
-// the library's own device image instead, so it never calls an allocator.  Every GPU holds its own copy of the
-// array for the life of the process; host code reaches it only through the address hipGetSymbolAddress gives on
-// that GPU (the array's name in host code is a host-side stand-in, not a device address).
-#define ATTN_STATIC_COUNTERS 1024                    // query heads x batch at most
-#define ATTN_STATIC_BYTES ((size_t)4 << 20)          // counters (first 4 KiB) + partial states
+// The slices of a long cache hand their partial states (ctx[D], m, l per query head and slice, as tagged 8-byte
+// words) from workgroup to workgroup through device memory.  lumen_attn_decode_f32 keeps that scratch on the cache
+// object and allocates it at the first call; this variant takes it from a fixed array in the library's own device
+// image instead, so it never calls an allocator.  Every GPU holds its own copy of the array for the life of the
+// process; host code reaches it only through the address hipGetSymbolAddress gives on that GPU (the array's name in
+// host code is a host-side stand-in, not a device address).  The first 256 bytes hold the count of launches the
+// tags are made of -- in device memory, advanced by a one-thread kernel in front of every launch, so that a call
+// recorded into a graph carries a new tag at every replay.
+#define ATTN_STATIC_HEAD 256                         // the launch count (4 bytes used)
+#define ATTN_STATIC_BYTES ((size_t)4 << 20)          // launch count + partial states
 static __device__ __align__(256) unsigned char scratch[ATTN_STATIC_BYTES];
 
 // called by lumen_ctx_create with the context's device current
@@ -823,8 +845,10 @@ int attn_static_scratch_init(lumen_ctx *ctx) {
     return LUMEN_OK;
 }
 
-__global__ __launch_bounds__(256) void clear_ints_kernel(int *p, int n) {
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) p[i] = 0;
+// the next launch's tag: 1, 2, ... (0 is what an untouched word carries)
+__global__ void next_epoch_kernel(unsigned *epoch) {
+    unsigned e = *epoch + 1u;
+    *epoch = e ? e : 1u;
 }
 
 extern "C" int lumen_attn_decode_static_f32(lumen_kv_cache *c, lumen_rope *rope, const float *q3, const float *k3,
@@ -834,20 +858,18 @@ extern "C" int lumen_attn_decode_static_f32(lumen_kv_cache *c, lumen_rope *rope,
     lumen_ctx *ctx = c->ctx;
     if (!ctx->attn_static) LUMEN_FAIL(LUMEN_ERR_HIP, "attn_decode_static: the context holds no static scratch address");
     const int nsplit = attn_decode_nsplit(c->max_seq, c->d);
-    const size_t heads = (size_t)c->b * h;
-    const size_t need = sizeof(int) * ATTN_STATIC_COUNTERS + sizeof(float) * attn_decode_part_floats(c->b, h, c->d, nsplit);
-    if (heads > ATTN_STATIC_COUNTERS || need > ctx->attn_static_bytes)
+    const size_t need = ATTN_STATIC_HEAD + sizeof(unsigned long long) * attn_decode_part_floats(c->b, h, c->d, nsplit);
+    if (need > ctx->attn_static_bytes)
         LUMEN_FAIL(LUMEN_ERR_UNSUPPORTED,
                    "attn_decode_static: batch %d x %d heads x %d slices x head_dim %d needs %zu bytes of partial states; "
-                   "the static scratch holds %zu bytes and %d heads (use lumen_attn_decode_f32)",
-                   c->b, h, nsplit, c->d, need, ctx->attn_static_bytes, ATTN_STATIC_COUNTERS);
-    int *counters = (int *)ctx->attn_static;
-    float *part = (float *)(ctx->attn_static + sizeof(int) * ATTN_STATIC_COUNTERS);
-    // the array keeps what the last call left: the arrival counters must start at zero (a fill kernel, not a
-    // memset node, so that the call may sit inside a stream capture); partial states are written before they are read
-    hipLaunchKernelGGL(clear_ints_kernel, dim3(1), dim3(256), 0, ctx->stream, counters, (int)heads);
+                   "the static scratch holds %zu bytes (use lumen_attn_decode_f32)",
+                   c->b, h, nsplit, c->d, need, ctx->attn_static_bytes);
+    unsigned *epoch = (unsigned *)ctx->attn_static;
+    unsigned long long *part_tagged = (unsigned long long *)(ctx->attn_static + ATTN_STATIC_HEAD);
+    // the array keeps what the last call left: words with older tags, which this launch's readers pass over
+    hipLaunchKernelGGL(next_epoch_kernel, dim3(1), dim3(1), 0, ctx->stream, epoch);
     LUMEN_CHECK_LAUNCH();
-    return attn_decode_entry(c, rope, q3, k3, v3, out, h, scale, part, counters, nsplit);
+    return attn_decode_entry(c, rope, q3, k3, v3, out, h, scale, part_tagged, epoch, 0, nsplit);
 }
 
 extern "C" int lumen_attn_prefill_f32(lumen_kv_cache *c, lumen_rope *rope, const float *q, const float *k,

@@ -282,13 +282,3 @@ __device__ __forceinline__ void norm_rope_heads(const float *raw, float *rot, in
         }
     }
 }
-
-// Partial results of a slice travel between workgroups through memory with agent-scope accesses
-// (they bypass the per-XCD L2 and the CU's L1, so neither a cache write-back nor an invalidate is
-// needed around the hand-over; the writer only has to wait for its stores before it signals).
-__device__ __forceinline__ void part_store(float *p, float v) {
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ float part_load(const float *p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}

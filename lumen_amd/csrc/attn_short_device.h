@@ -253,7 +253,6 @@ __device__ __forceinline__ bool attn_decode_short(const AttnDecodeArgs &a, int r
     wave_merge_publish<D, 1>(st, sm, sl, sacc);
     __syncthreads();
     STAGE_T(2);
-    float *part0 = a.part + ((size_t)bb * a.hq + hq) * a.nsplit * (D + 2);  // slice 0 of this head
     for (int dd = threadIdx.x; dd < D; dd += THREADS) {
         float mm, ls, cx;
         wave_fold<D, 1, WAVES>(sm, sl, sacc, 0, dd, mm, ls, cx);
@@ -265,6 +264,7 @@ __device__ __forceinline__ bool attn_decode_short(const AttnDecodeArgs &a, int r
                 tagged_store(pt + D + 1, ls, a.tag);
             }
         } else if (a.defer_merge) {  // the consumer divides
+            float *part0 = a.part + ((size_t)bb * a.hq + hq) * a.nsplit * (D + 2);  // slice 0 of this head
             part0[dd] = cx;
             if (dd == 0) {
                 part0[D] = mm;

@@ -41,6 +41,8 @@ extern "C" int lumen_ctx_create(int device, lumen_ctx **out) {
     HIP_TRY(hipEventCreate(&c->ev1));
     HIP_TRY(hipMalloc((void **)&c->d_scratch_int, 64 * sizeof(int)));
     HIP_TRY(hipHostMalloc(&c->bounce, LUMEN_BOUNCE_BYTES, hipHostMallocDefault));
+    HIP_TRY(hipHostMalloc((void **)&c->err_host, 64, hipHostMallocDefault));
+    *c->err_host = 0;
     // load the device code of every translation unit now rather than under the first prompt
     lumen_warm_attention(c->stream);
     lumen_warm_attn_oproj(c->stream);
@@ -74,6 +76,7 @@ extern "C" int lumen_ctx_destroy(lumen_ctx *ctx) {
     hipStreamSynchronize(ctx->stream);
     hipFree(ctx->d_scratch_int);
     if (ctx->bounce) hipHostFree(ctx->bounce);
+    if (ctx->err_host) hipHostFree(ctx->err_host);
     if (ctx->gemm_ws) hipFree(ctx->gemm_ws);
     hipEventDestroy(ctx->ev0);
     hipEventDestroy(ctx->ev1);
@@ -88,10 +91,18 @@ extern "C" int lumen_ctx_set_stream(lumen_ctx *ctx, void *hip_stream) {
     return LUMEN_OK;
 }
 
+// after a synchronisation: did a bounded wait inside an operator-level launch run out?
+static int check_wait_flag(lumen_ctx *ctx) {
+    if (!ctx->err_host || !*(volatile int *)ctx->err_host) return LUMEN_OK;
+    *(volatile int *)ctx->err_host = 0;
+    LUMEN_FAIL(LUMEN_ERR_HIP, "a workgroup gave up waiting for values handed over inside a launch; the results of the "
+                              "launches since the last synchronisation are invalid");
+}
+
 extern "C" int lumen_ctx_synchronize(lumen_ctx *ctx) {
     if (!ctx) LUMEN_FAIL(LUMEN_ERR_INVALID, "ctx is null");
     HIP_TRY(hipStreamSynchronize(ctx->stream));
-    return LUMEN_OK;
+    return check_wait_flag(ctx);
 }
 
 extern "C" int lumen_timer_start(lumen_ctx *ctx) {
@@ -140,11 +151,11 @@ extern "C" int lumen_download(lumen_ctx *ctx, void *dst_host, const void *src_de
         HIP_TRY(hipMemcpyAsync(ctx->bounce, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
         HIP_TRY(hipStreamSynchronize(ctx->stream));
         memcpy(dst_host, ctx->bounce, bytes);
-        return LUMEN_OK;
+        return check_wait_flag(ctx);
     }
     HIP_TRY(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
     HIP_TRY(hipStreamSynchronize(ctx->stream));
-    return LUMEN_OK;
+    return check_wait_flag(ctx);
 }
 
 extern "C" int lumen_ctx_num_cus(const lumen_ctx *ctx, int *num_cus_out) {

@@ -51,6 +51,9 @@ struct lumen_ctx {
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     int *d_scratch_int = nullptr;  // small device scratch (argmax result etc.)
     void *bounce = nullptr;        // pinned host memory that small downloads travel through (LUMEN_BOUNCE_BYTES)
+    // one int of pinned host memory the GPU can write: set to 1 by an operator-level launch whose bounded wait for
+    // another workgroup's values ran out; lumen_ctx_synchronize and lumen_download report and clear it
+    int *err_host = nullptr;
     float *gemm_ws = nullptr;      // split-K workspace of the prefill GEMM, grown on demand
     size_t gemm_ws_bytes = 0;
     // this device's address of the fixed scratch array behind lumen_attn_decode_static_f32
@@ -78,9 +81,10 @@ struct lumen_kv_cache {
     int len = 0;            // host mirror of the position counter
     float *k = nullptr, *v = nullptr;
     bool owns = true;       // false when k/v are slices of a model-wide slab
-    // decode-attention split-L scratch
-    float *part = nullptr;  // [b*h_q_max, nsplit, d + 2]
-    int *counters = nullptr;
+    // decode attention, sliced long cache: the slices' states on their way to the workgroup that folds them,
+    // tagged words [b*h_q_max, nsplit, d + 2], and the count of launches their tags are made of
+    unsigned long long *part_tagged = nullptr;
+    unsigned merge_epoch = 0;
     int part_heads = 0;
     int *d_pos = nullptr;    // device copy of len for lumen_qkv_rope_append_f32, allocated at its first call
     float *q_rot = nullptr;  // rotated queries of the prefill entry point, grown on demand
@@ -215,9 +219,13 @@ struct AttnDecodeArgs {
     float scale;
     const float *q_norm_w, *k_norm_w;  // per-head RMSNorm gains [D] or null
     float norm_eps;
-    float *part;        // split scratch
-    int *counters;      // one per (batch, query head), zero between launches
+    float *part;        // slice states for a consumer in a LATER launch (defer_merge), plain floats [b*hq][nsplit][d + 2]
     int nsplit;         // slices a long cache is cut into (attn_decode_nsplit)
+    // slices merged inside the launch: their states travel as tagged words in part_tagged [b*hq][nsplit][d + 2]
+    // (zero before the first launch); the tag is (*tag_dev, or 0 without one) * tag_mul + tag_add and must differ
+    // from launch to launch on one buffer and never be 0
+    const unsigned *tag_dev;
+    unsigned tag_mul, tag_add;
     int pre_rotated;    // q is already rotated and row pos of the cache already written (fused QKV GEMV)
     int expect_short;   // hint: the cache is short (a few hundred rows); a wrong hint only costs time
     // Leave the merge of a long cache's slices to the consumer: every workgroup stores its partial state
@@ -232,7 +240,7 @@ struct AttnDecodeArgs {
     // o_proj chain): the cache row of the new token is not read, nothing is rotated or stored here; null everywhere else
     const unsigned long long *qkv_tagged;
     // the chained launch with several workgroups per query head: slices launched, and where a slice leaves its
-    // state for the workgroup that folds them, [hq][tslices][d + 2] tagged words
+    // state for the workgroup that folds them, [hq][tslices][d + 2] tagged words (part_tagged, as above)
     int tslices, slice_shift;  // (a slice covers 1 << slice_shift rows)
     unsigned long long *part_tagged;
     unsigned spin_limit;  // polls before a wait for tagged words gives up (then *err_dev = 1)

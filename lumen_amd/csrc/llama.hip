@@ -40,8 +40,8 @@ struct lumen_llama {
     float *x = nullptr, *h = nullptr, *qkv = nullptr, *attn = nullptr, *act = nullptr, *logits = nullptr;
     int *d_tok = nullptr, *d_pos = nullptr;
     int *tok_hist = nullptr;  // [max_seq + 1]: greedy pick made at position p sits at index p + 1
-    float *part = nullptr;
-    int *counters = nullptr;
+    float *part = nullptr;                          // slice states for the o_proj product to fold (defer_merge)
+    unsigned long long *part_merge = nullptr;       // slice states folded inside the attention launch (tagged words)
     int nsplit = 1;     // slices of a long cache in the decode attention kernel
     bool defer_merge = false;  // the o_proj GEMV, not the attention kernel, may merge the slices of a long cache
     // short caches: attention and o_proj chained in one launch (attn_oproj.hip); its hand-over buffer, the decode
@@ -214,7 +214,7 @@ extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg,
     m->defer_merge = m->nsplit >= 2 && m->nsplit <= GEMV_FOLD_MAX_SLICES && !cfg->qk_norm &&
                      cfg->max_seq_len <= m->nsplit * attn_decode_trip_rows(D) && fold_bytes <= ((size_t)64 << 20);
     M_TRY(dmalloc_t(m, &m->part, attn_decode_part_floats(1, Hq, D, m->nsplit)));
-    M_TRY(dmalloc_t(m, &m->counters, (size_t)Hq));
+    M_TRY(dmalloc_t(m, &m->part_merge, attn_decode_part_floats(1, Hq, D, m->nsplit)));
     // (q/k-norm models rotate inside the attention role: only the three-role form serves them)
     m->chain_ao = qkv_attn_oproj_supported(Hq, Hkv, D, H, m->qd, m->bf16, cfg->qk_norm)                 ? 2
                   : (!cfg->qk_norm && attn_oproj_supported(Hq, Hkv, D, H, m->qd, m->bf16)) ? 1
@@ -244,7 +244,7 @@ extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg,
         lumen_llama_destroy(m);
         LUMEN_FAIL(LUMEN_ERR_HIP, "llama_create: clearing the hand-over state failed");
     }
-    if (hipMemsetAsync(m->counters, 0, sizeof(int) * Hq, ctx->stream) != hipSuccess ||
+    if (hipMemsetAsync(m->part_merge, 0, sizeof(unsigned long long) * attn_decode_part_floats(1, Hq, D, m->nsplit), ctx->stream) != hipSuccess ||
         hipMemsetAsync(m->d_tok, 0, 4 * sizeof(int), ctx->stream) != hipSuccess ||
         hipMemsetAsync(m->d_pos, 0, 4 * sizeof(int), ctx->stream) != hipSuccess ||
         hipStreamSynchronize(ctx->stream) != hipSuccess) {
@@ -538,7 +538,10 @@ static int enqueue_decode_step(lumen_llama *m, StepProbe *pr = nullptr) {
         a.cos_t = m->cos_dev; a.sin_t = m->sin_dev; a.pos_dev = m->d_pos; a.pos_host = 0;
         a.b = 1; a.hq = c.num_attention_heads; a.hkv = c.num_key_value_heads; a.d = m->D; a.max_seq = c.max_seq_len;
         a.scale = m->scale; a.q_norm_w = w.q_norm; a.k_norm_w = w.k_norm; a.norm_eps = c.rms_norm_eps;
-        a.part = m->part; a.counters = m->counters; a.nsplit = m->nsplit; a.pre_rotated = fuse_rope;
+        a.part = m->part; a.nsplit = m->nsplit; a.pre_rotated = fuse_rope;
+        // (slices merged inside the attention launch: tagged words, the tag made of the step counter like the chains')
+        a.part_tagged = m->part_merge; a.tag_dev = m->d_step; a.tag_mul = (unsigned)c.num_hidden_layers; a.tag_add = (unsigned)l + 1u;
+        a.spin_limit = m->spin_limit; a.err_dev = m->d_err;
         a.expect_short = expect_short_cache(m);
         // (a graph is captured anew when the cache crosses the short / long boundary, so the choices below are the
         // same for every launch of a step)

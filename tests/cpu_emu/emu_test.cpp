@@ -4,9 +4,10 @@
 // in its three forms (with a q|k|v role, attention + o_proj only, separate launches), with one and with several
 // attention workgroups per head (slices + fold), rotated and un-rotated (q/k-norm) hand-over, f32 and bf16 weights;
 // the gate|up -> down chain; the few-row product of short prompts with ragged shapes and all three epilogues; the
-// streaming vector-matrix product and the stand-alone decode attention those forms fall back to.
+// streaming vector-matrix product and the stand-alone decode attention those forms fall back to, the latter also
+// at operator level over a sliced cache (slices merged inside the launch).
 //
-//   emu_test [case ...]      cases: chain sliced qknorm bf16 skinny (default: all)
+//   emu_test [case ...]      cases: chain sliced qknorm bf16 skinny attn (default: all)
 #include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -282,6 +283,66 @@ static void case_skinny(lumen_ctx *ctx) {
     }
 }
 
+// the operator-level decode attention over a sliced cache: slices merged inside the launch (tagged words polled by
+// the workgroup of the last slice), through the allocating entry point and through the one with the fixed scratch
+static void case_attn(lumen_ctx *ctx) {
+    printf("attn: lumen_attn_decode_f32 / lumen_attn_decode_static_f32, 4/2 heads of 64, 700 and 40 cached rows\n");
+    const int h = 4, hkv = 2, d = 64, max_seq = 1024;
+    const float scale = 0.125f;
+    lumen_rope *rope = nullptr;
+    OK(lumen_rope_create(ctx, d, max_seq, 10000.f, &rope));
+    std::vector<float> cs((size_t)max_seq * d), sn((size_t)max_seq * d);
+    lo_rope_table(cs.data(), sn.data(), d, max_seq, 10000.f);
+    for (int filled : {700, 40}) {
+        lumen_kv_cache *ca = nullptr, *cb = nullptr;
+        OK(lumen_kv_cache_create(ctx, 1, hkv, max_seq, d, &ca));
+        OK(lumen_kv_cache_create(ctx, 1, hkv, max_seq, d, &cb));
+        lo_kv_cache *co = lo_kv_cache_new(1, hkv, max_seq, d);
+        std::vector<float> k0 = randn((size_t)hkv * filled * d, 1.f), v0 = randn((size_t)hkv * filled * d, 1.f);
+        void *dk, *dv;
+        OK(lumen_malloc(ctx, k0.size() * 4, &dk));
+        OK(lumen_malloc(ctx, v0.size() * 4, &dv));
+        OK(lumen_upload(ctx, dk, k0.data(), k0.size() * 4));
+        OK(lumen_upload(ctx, dv, v0.data(), v0.size() * 4));
+        for (lumen_kv_cache *c : {ca, cb}) {
+            OK(lumen_kv_cache_update(c, (const float *)dk, (const float *)dv, filled, 0));
+            OK(lumen_kv_cache_set_len(c, filled));
+        }
+        for (int hk = 0; hk < hkv; ++hk) {
+            memcpy(co->k + (size_t)hk * max_seq * d, k0.data() + (size_t)hk * filled * d, sizeof(float) * filled * d);
+            memcpy(co->v + (size_t)hk * max_seq * d, v0.data() + (size_t)hk * filled * d, sizeof(float) * filled * d);
+        }
+        co->len = filled;
+        void *dq, *dkn, *dvn, *dout;
+        OK(lumen_malloc(ctx, (size_t)h * d * 4, &dq));
+        OK(lumen_malloc(ctx, (size_t)hkv * d * 4, &dkn));
+        OK(lumen_malloc(ctx, (size_t)hkv * d * 4, &dvn));
+        OK(lumen_malloc(ctx, (size_t)h * d * 4, &dout));
+        for (int step = 0; step < 2; ++step) {
+            std::vector<float> q = randn((size_t)h * d, 1.f), kn = randn((size_t)hkv * d, 1.f), vn = randn((size_t)hkv * d, 1.f);
+            std::vector<float> ref((size_t)h * d), got((size_t)h * d), got_static((size_t)h * d);
+            OK(lumen_upload(ctx, dq, q.data(), q.size() * 4));
+            OK(lumen_upload(ctx, dkn, kn.data(), kn.size() * 4));
+            OK(lumen_upload(ctx, dvn, vn.data(), vn.size() * 4));
+            OK(lumen_attn_decode_f32(ca, rope, (const float *)dq, (const float *)dkn, (const float *)dvn, (float *)dout, h, scale, 1));
+            OK(lumen_download(ctx, got.data(), dout, got.size() * 4));
+            OK(lumen_attn_decode_static_f32(cb, rope, (const float *)dq, (const float *)dkn, (const float *)dvn, (float *)dout, h, scale, 1));
+            OK(lumen_download(ctx, got_static.data(), dout, got_static.size() * 4));
+            CHECK(lo_attn_decode_f32(co, q.data(), kn.data(), vn.data(), ref.data(), h, cs.data(), sn.data(), max_seq, scale, 1) == LO_OK, "checker");
+            const double e = max_rel(got.data(), ref.data(), ref.size());
+            printf("  %d cached rows: max rel err %.2e, fixed-scratch entry %s\n", filled + step, e,
+                   memcmp(got.data(), got_static.data(), got.size() * 4) ? "DIFFERS" : "bit-equal");
+            CHECK(e <= 2e-5, "attn %d rows: %.3g", filled + step, e);
+            CHECK(!memcmp(got.data(), got_static.data(), got.size() * 4), "fixed-scratch entry differs at %d rows", filled + step);
+        }
+        for (void *p : {dk, dv, dq, dkn, dvn, dout}) OK(lumen_free(ctx, p));
+        OK(lumen_kv_cache_destroy(ca));
+        OK(lumen_kv_cache_destroy(cb));
+        lo_kv_cache_free(co);
+    }
+    OK(lumen_rope_destroy(rope));
+}
+
 // The harness checks itself: a product whose output array is one element short must be stopped by the sanitizer.
 static void selfcheck_oob(lumen_ctx *ctx) {
     const int N = 64, K = 256;
@@ -306,7 +367,7 @@ int main(int argc, char **argv) {
         return 0;  // (reached only if nothing stopped the program: the test expects a sanitizer report instead)
     }
     struct { const char *name; void (*fn)(lumen_ctx *); } cases[] = {
-        {"chain", case_chain}, {"sliced", case_sliced}, {"qknorm", case_qknorm}, {"bf16", case_bf16}, {"skinny", case_skinny}};
+        {"chain", case_chain}, {"sliced", case_sliced}, {"qknorm", case_qknorm}, {"bf16", case_bf16}, {"skinny", case_skinny}, {"attn", case_attn}};
     for (const auto &c : cases) {
         bool run = argc <= 1;
         for (int i = 1; i < argc; ++i) run = run || !strcmp(argv[i], c.name);

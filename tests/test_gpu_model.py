@@ -311,12 +311,12 @@ def _greedy_call_checked(gpu, ora, first, n, tol):
     (dict(hidden_size=256, num_attention_heads=2, num_key_value_heads=1, max_seq_len=700, intermediate_size=704), 236, False),  # head_dim 128: 256 rows
     (dict(hidden_size=256, num_attention_heads=2, num_key_value_heads=1, max_seq_len=700, intermediate_size=704, qk_norm=True, head_dim=128), 236, True),
 ], ids=["d64-nrep4-defer", "d64-nrep8-defer", "d64-qknorm", "d128", "d128-qknorm"])
-def test_one_greedy_call_replays_a_graph_across_the_attention_boundary(cfg_extra, n_prompt, same_bits):
-    """A single decode_greedy call captures its graph once, on the short side of the attention boundary (512 cached
-    rows, 256 for head_dim 128), and keeps replaying it on the long side: the captured launches then carry a stale
-    hint and the kernel hands over to the sliced form by itself.  Every step of such a call is held to the checker,
-    and to the eager launches of the same steps (whose hint is right at every step; where the eager steps leave the
-    merge of the slices to o_proj the two differ in summation order, elsewhere they are bit-equal)."""
+def test_one_greedy_call_crosses_the_attention_boundary(cfg_extra, n_prompt, same_bits):
+    """A single decode_greedy call that starts on the short side of the attention boundary (512 cached rows, 256
+    for head_dim 128) and ends on the long side: the step's graph is recorded anew at the step that crosses it (the
+    recorded launches carry the form to run), inside the one call.  Every step of such a call is held to the
+    checker, and to the eager launches of the same steps (where the eager steps leave the merge of the slices to
+    o_proj the two differ in summation order, elsewhere they are bit-equal)."""
     cfg = dict(vocab_size=900, hidden_size=512, intermediate_size=1408, num_hidden_layers=2, rms_norm_eps=1e-5,
                rope_theta=10000.0)
     cfg.update(cfg_extra)

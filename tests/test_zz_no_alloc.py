@@ -1,6 +1,6 @@
 """GPU check of lumen_attn_decode_static_f32, the decode-attention entry point that allocates nothing: its
-scratch (partial states and arrival counters of a sliced long cache) is a fixed array in the library's device
-image.  It must give the same bits as lumen_attn_decode_f32 -- outputs and appended cache rows -- on calls in a
+scratch (the partial states of a sliced long cache, as tagged words, and the launch count their tags are made
+of) is a fixed array in the library's device image.  It must give the same bits as lumen_attn_decode_f32 -- outputs and appended cache rows -- on calls in a
 row that share the array, the later ones smaller than the first, and refuse what the array cannot hold."""
 import math
 
@@ -63,7 +63,7 @@ def test_static_scratch_decode_attention_matches_the_allocating_entry_point():
 
 
 def test_static_scratch_refuses_what_it_cannot_hold():
-    d, max_seq = 128, 8192  # 64 slices x 130 floats x 4 bytes = 33 KB per head: 256 heads do not fit 4 MiB
+    d, max_seq = 128, 8192  # 64 slices x 130 words x 8 bytes = 66 KB per head: 256 heads do not fit 4 MiB
     rope = RotaryEmbedding(d, max_seq, 10000.0)
     c = KVCacheInner(1, 2, max_seq, d)
     q, kv = dev(np.zeros((1, 256, d), np.float32)), dev(np.zeros((1, 2, d), np.float32))
