@@ -51,6 +51,9 @@ def main():
                     help="how decode steps are issued: a HIP graph replay per token (default) or kernel by kernel "
                          "(for rocprofv3 --kernel-trace, which cannot follow graph replays here)")
     ap.add_argument("--cpu-tokens", type=int, default=48)
+    ap.add_argument("--resident", action="store_true",
+                    help="--workload gemv: every launch reads the SAME copy of W (what the caches hold counts: the "
+                         "figure is no longer HBM bandwidth); default: >= 1.2 GB of copies in rotation")
     ap.add_argument("--workload", choices=["decode", "gemv", "gemm", "prefill", "copy"], default="decode",
                     help="decode: the headline batch-1 decode benchmark; gemv: the isolated M=1 GEMV shapes; "
                          "gemm: the prompt-pass GEMM shapes against the fp32 matrix-core peak; prefill: one long "
@@ -327,7 +330,7 @@ def gemv_microbench(args):
         rng = np.random.default_rng(K * 100003 + N)
         W = (rng.standard_normal((N, K), dtype=np.float32) * np.float32(0.02))
         x = rng.standard_normal(K, dtype=np.float32)
-        ncopies = max(2, int(np.ceil(1.2e9 / W.nbytes)))
+        ncopies = 1 if args.resident else max(2, int(np.ceil(1.2e9 / W.nbytes)))
         slab = Tensor.empty((ncopies, N, K), np.float32, ctx)
         for c in range(ncopies):
             check(lib.lumen_upload(ctx.handle, slab.ptr + c * W.nbytes, W.ctypes.data, W.nbytes))
@@ -345,7 +348,10 @@ def gemv_microbench(args):
                      "weight_copies": ncopies})
         del slab
     print(json.dumps({"metric": "M=1 GEMV HBM GB/s", "unit": "GB/s", "n_gpus": 1, "dtype": "f32", "data": "synthetic",
-                      "layout": "[N,K] row-major (out,in)", "shapes": rows}))
+                      "layout": "[N,K] row-major (out,in)",
+                      "weights": "one copy, cache-resident (not an HBM figure)" if args.resident else
+                                 "copies in rotation (>= 1.2 GB): every launch reads from HBM",
+                      "shapes": rows}))
 
 
 GEMM_SHAPES = [(128, 2048, 2048), (128, 2560, 2048), (128, 11264, 2048), (128, 2048, 5632), (512, 2048, 2048),

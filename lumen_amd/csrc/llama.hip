@@ -502,118 +502,133 @@ static int chain_plan_key(const lumen_llama *m) {
     return s ? s * 65536 + rows : 0;
 }
 
+// One decoder layer of a decode step, LlamaDecoderLayer::forward_infer for S == 1 (src/models/llama.rs:104-116):
+// three launches (two for narrow models, five where no chain applies).  x_in [H] is the layer input -- or, with
+// row_sel, row *row_sel of the table x_in points at (the embedding gather of llama.rs:191 folded into the first
+// layer) --, y_out [H] its output (may be x_in); k_cache / v_cache the layer's cache [Hkv, max_seq, D]; the new
+// token's position is *m->d_pos; tag_slot < tag_mul tells the launches of one step apart (their hand-over tags are
+// *d_step * tag_mul + tag_slot + 1).
+static int enqueue_decoder_layer(lumen_llama *m, const LayerW &w, float *k_cache, float *v_cache, const float *x_in,
+                                 const int *row_sel, float *y_out, unsigned tag_mul, unsigned tag_slot, StepProbe *pr) {
+    lumen_ctx *ctx = m->ctx;
+    const lumen_llama_config &c = m->cfg;
+    const int H = c.hidden_size, I = c.intermediate_size;
+    // RoPE + KV append ride on the q|k|v product unless q/k need a per-head norm first.
+    const bool fuse_rope = !c.qk_norm;
+    GemvArgs g = {};
+    // input_layernorm + q|k|v projections, llama.rs:107, self_attention.rs:106-108
+    g.W = w.wqkv; g.x = x_in; g.y = m->qkv; g.N = m->qkvd; g.K = H; g.w_bf16 = m->bf16;
+    g.pro = PRO_RMSNORM; g.norm_w = w.in_norm; g.eps = c.rms_norm_eps; g.epi = EPI_STORE;
+    if (row_sel) { g.row_sel = row_sel; g.row_stride = H; g.x_sel = 1; }
+    if (fuse_rope) {
+        g.epi = EPI_ROPE_QKV; g.cos_t = m->cos_dev; g.sin_t = m->sin_dev; g.pos = m->d_pos;
+        g.k_cache = k_cache; g.v_cache = v_cache;
+        g.hq = c.num_attention_heads; g.hkv = c.num_key_value_heads; g.D = m->D; g.max_seq = c.max_seq_len;
+    }
+    int slice_rows = 0;
+    const int slices = chain_slices(m, &slice_rows);
+    const bool chain_short = slices > 0;
+    const bool chain_qkv = chain_short && m->chain_ao > 1;
+    if (!chain_qkv) {
+        pr->before(KC_QKV);
+        LUMEN_TRY(launch_gemv(ctx, g));
+        pr->after();
+    }
+    AttnDecodeArgs a = {};
+    a.q = m->qkv; a.k_new = m->qkv + m->qd; a.v_new = m->qkv + m->qd + m->kvd; a.out = m->attn;
+    a.k_cache = k_cache; a.v_cache = v_cache;
+    a.cos_t = m->cos_dev; a.sin_t = m->sin_dev; a.pos_dev = m->d_pos; a.pos_host = 0;
+    a.b = 1; a.hq = c.num_attention_heads; a.hkv = c.num_key_value_heads; a.d = m->D; a.max_seq = c.max_seq_len;
+    a.scale = m->scale; a.q_norm_w = w.q_norm; a.k_norm_w = w.k_norm; a.norm_eps = c.rms_norm_eps;
+    a.part = m->part; a.nsplit = m->nsplit; a.pre_rotated = fuse_rope;
+    // (slices merged inside the attention launch: tagged words, the tag made of the step counter like the chains')
+    a.part_tagged = m->part_merge; a.tag_dev = m->d_step; a.tag_mul = tag_mul; a.tag_add = tag_slot + 1u;
+    a.spin_limit = m->spin_limit; a.err_dev = m->d_err;
+    a.expect_short = expect_short_cache(m);
+    // (a graph is captured anew when the cache crosses the short / long boundary, so the choices below are the
+    // same for every launch of a step)
+    if (chain_short) {
+        // short caches: (q|k|v,) attention and o_proj + residual chained in one launch
+        AttnOprojArgs f = {};
+        f.attn = a;
+        f.attn.out_tagged = m->x_tagged;
+        f.Wo = w.wo; f.residual = x_in; f.y = m->h; f.N = H; f.K = m->qd; f.w_bf16 = m->bf16;
+        if (row_sel) { f.row_sel = row_sel; f.row_stride = H; }
+        f.x_tagged = m->x_tagged; f.step_dev = m->d_step;
+        f.tag_mul = tag_mul; f.tag_add = tag_slot + 1u;
+        f.err_dev = m->d_err; f.spin_limit = m->spin_limit;
+        f.pre_sleep = m->chain_pre[m->chain_ao]; f.poll_delay = m->chain_delay[m->chain_ao]; f.poll_gap = m->chain_gap[m->chain_ao];
+        // (the fold of the slices is one more hand-over in front of o_proj, and two-trip slices take a trip longer:
+        // polling earlier only puts polls in the way of those hand-overs; measured optima, 1.7 / 3.7 us)
+        if (slices > 1) f.poll_delay += slice_rows > attn_decode_trip_rows(m->D) ? 37 : 17;
+        f.nslices = slices; f.slice_rows = slice_rows; f.part_tagged = m->part_tagged;
+        f.t0_tagged = m->part_tagged + (size_t)c.num_attention_heads * ATTN_CHAIN_MAX_SLICES * (m->D + 2);  // (one word behind the states)
+        if (chain_qkv) {
+            f.Wqkv = w.wqkv; f.in_norm_w = w.in_norm; f.norm_eps = c.rms_norm_eps; f.qkv_tagged = m->qkv_tagged;
+        }
+        pr->before(KC_ATTN_OPROJ);
+        LUMEN_TRY(launch_attn_oproj(ctx, f));
+        pr->after();
+    } else {
+        const bool defer = m->defer_merge && !a.expect_short;
+        a.defer_merge = defer;
+        pr->before(KC_ATTN);
+        LUMEN_TRY(launch_attn_decode(ctx, a));
+        pr->after();
+        // o_proj + residual, self_attention.rs:303, llama.rs:110
+        g = {};
+        g.W = w.wo; g.x = m->attn; g.y = m->h; g.N = H; g.K = m->qd; g.w_bf16 = m->bf16;
+        g.pro = PRO_NONE; g.epi = EPI_RESIDUAL; g.residual = x_in;
+        if (defer) {
+            g.pro = PRO_ATTN_FOLD; g.attn_part = m->part; g.attn_pos = m->d_pos; g.attn_nslices = m->nsplit; g.attn_d = m->D;
+            g.attn_trip = attn_decode_trip_rows(m->D); g.attn_short_rows = attn_decode_short_rows(m->D);
+        }
+        if (row_sel) { g.row_sel = row_sel; g.row_stride = H; g.residual_sel = 1; }
+        pr->before(KC_OPROJ);
+        LUMEN_TRY(launch_gemv(ctx, g));
+        pr->after();
+    }
+    if (m->chain_mlp && m->chain_ao_on) {
+        // narrow models: post_attention_layernorm + gate|up + silu*up + down + residual as one launch
+        MlpChainArgs mc = {};
+        mc.Wgu = w.wgu; mc.h = m->h; mc.norm_w = w.post_norm; mc.eps = c.rms_norm_eps; mc.Wdown = w.wdown; mc.y = y_out;
+        mc.N = H; mc.I = I; mc.w_bf16 = m->bf16; mc.act_tagged = m->act_tagged; mc.step_dev = m->d_step;
+        mc.tag_mul = tag_mul; mc.tag_add = tag_slot + 1u;
+        mc.err_dev = m->d_err; mc.spin_limit = m->spin_limit;
+        mc.pre_sleep = m->mlp_pre; mc.poll_delay = m->mlp_delay; mc.poll_gap = m->mlp_gap;
+        pr->before(KC_MLP);
+        LUMEN_TRY(launch_mlp_chain(ctx, mc));
+        pr->after();
+        return LUMEN_OK;
+    }
+    // post_attention_layernorm + gate|up + silu*up, llama.rs:113, :60-63
+    g = {};
+    g.W = w.wgu; g.x = m->h; g.y = m->act; g.N = 2 * I; g.K = H; g.w_bf16 = m->bf16;
+    g.pro = PRO_RMSNORM; g.norm_w = w.post_norm; g.eps = c.rms_norm_eps; g.epi = EPI_SWIGLU;
+    pr->before(KC_GATEUP);
+    LUMEN_TRY(launch_gemv(ctx, g));
+    pr->after();
+    // down_proj + residual, llama.rs:64, :115
+    g = {};
+    g.W = w.wdown; g.x = m->act; g.y = y_out; g.N = H; g.K = I; g.w_bf16 = m->bf16;
+    g.pro = PRO_NONE; g.epi = EPI_RESIDUAL; g.residual = m->h;
+    pr->before(KC_DOWN);
+    LUMEN_TRY(launch_gemv(ctx, g));
+    pr->after();
+    return LUMEN_OK;
+}
+
 static int enqueue_decode_step(lumen_llama *m, StepProbe *pr = nullptr) {
     StepProbe none;
     if (!pr) pr = &none;
     lumen_ctx *ctx = m->ctx;
     const lumen_llama_config &c = m->cfg;
-    const int H = c.hidden_size, I = c.intermediate_size, V = c.vocab_size;
-    // Embedding::forward (llama.rs:191) is folded into the first layer: its GEMVs read row *d_tok of
-    // the table directly.  RoPE + KV append ride on the q|k|v product unless q/k need a per-head norm first.
-    const bool fuse_rope = !c.qk_norm;
-    for (int l = 0; l < c.num_hidden_layers; ++l) {
-        const LayerW &w = m->layers[l];
-        GemvArgs g = {};
-        // input_layernorm + q|k|v projections, llama.rs:107, self_attention.rs:106-108
-        g.W = w.wqkv; g.x = m->x; g.y = m->qkv; g.N = m->qkvd; g.K = H; g.w_bf16 = m->bf16;
-        g.pro = PRO_RMSNORM; g.norm_w = w.in_norm; g.eps = c.rms_norm_eps; g.epi = EPI_STORE;
-        if (l == 0) { g.x = m->embed; g.row_sel = m->d_tok; g.row_stride = H; g.x_sel = 1; }
-        if (fuse_rope) {
-            g.epi = EPI_ROPE_QKV; g.cos_t = m->cos_dev; g.sin_t = m->sin_dev; g.pos = m->d_pos;
-            g.k_cache = m->k_slab + m->cache_stride * l; g.v_cache = m->v_slab + m->cache_stride * l;
-            g.hq = c.num_attention_heads; g.hkv = c.num_key_value_heads; g.D = m->D; g.max_seq = c.max_seq_len;
-        }
-        int slice_rows = 0;
-        const int slices = chain_slices(m, &slice_rows);
-        const bool chain_short = slices > 0;
-        const bool chain_qkv = chain_short && m->chain_ao > 1;
-        if (!chain_qkv) {
-            pr->before(KC_QKV);
-            LUMEN_TRY(launch_gemv(ctx, g));
-            pr->after();
-        }
-        AttnDecodeArgs a = {};
-        a.q = m->qkv; a.k_new = m->qkv + m->qd; a.v_new = m->qkv + m->qd + m->kvd; a.out = m->attn;
-        a.k_cache = m->k_slab + m->cache_stride * l; a.v_cache = m->v_slab + m->cache_stride * l;
-        a.cos_t = m->cos_dev; a.sin_t = m->sin_dev; a.pos_dev = m->d_pos; a.pos_host = 0;
-        a.b = 1; a.hq = c.num_attention_heads; a.hkv = c.num_key_value_heads; a.d = m->D; a.max_seq = c.max_seq_len;
-        a.scale = m->scale; a.q_norm_w = w.q_norm; a.k_norm_w = w.k_norm; a.norm_eps = c.rms_norm_eps;
-        a.part = m->part; a.nsplit = m->nsplit; a.pre_rotated = fuse_rope;
-        // (slices merged inside the attention launch: tagged words, the tag made of the step counter like the chains')
-        a.part_tagged = m->part_merge; a.tag_dev = m->d_step; a.tag_mul = (unsigned)c.num_hidden_layers; a.tag_add = (unsigned)l + 1u;
-        a.spin_limit = m->spin_limit; a.err_dev = m->d_err;
-        a.expect_short = expect_short_cache(m);
-        // (a graph is captured anew when the cache crosses the short / long boundary, so the choices below are the
-        // same for every launch of a step)
-        if (chain_short) {
-            // short caches: (q|k|v,) attention and o_proj + residual chained in one launch
-            AttnOprojArgs f = {};
-            f.attn = a;
-            f.attn.out_tagged = m->x_tagged;
-            f.Wo = w.wo; f.residual = m->x; f.y = m->h; f.N = H; f.K = m->qd; f.w_bf16 = m->bf16;
-            if (l == 0) { f.residual = m->embed; f.row_sel = m->d_tok; f.row_stride = H; }
-            f.x_tagged = m->x_tagged; f.step_dev = m->d_step;
-            f.tag_mul = (unsigned)c.num_hidden_layers; f.tag_add = (unsigned)l + 1u;
-            f.err_dev = m->d_err; f.spin_limit = m->spin_limit;
-            f.pre_sleep = m->chain_pre[m->chain_ao]; f.poll_delay = m->chain_delay[m->chain_ao]; f.poll_gap = m->chain_gap[m->chain_ao];
-            // (the fold of the slices is one more hand-over in front of o_proj, and two-trip slices take a trip longer:
-            // polling earlier only puts polls in the way of those hand-overs; measured optima, 1.7 / 3.7 us)
-            if (slices > 1) f.poll_delay += slice_rows > attn_decode_trip_rows(m->D) ? 37 : 17;
-            f.nslices = slices; f.slice_rows = slice_rows; f.part_tagged = m->part_tagged;
-            f.t0_tagged = m->part_tagged + (size_t)c.num_attention_heads * ATTN_CHAIN_MAX_SLICES * (m->D + 2);  // (one word behind the states)
-            if (chain_qkv) {
-                f.Wqkv = w.wqkv; f.in_norm_w = w.in_norm; f.norm_eps = c.rms_norm_eps; f.qkv_tagged = m->qkv_tagged;
-            }
-            pr->before(KC_ATTN_OPROJ);
-            LUMEN_TRY(launch_attn_oproj(ctx, f));
-            pr->after();
-        } else {
-            const bool defer = m->defer_merge && !a.expect_short;
-            a.defer_merge = defer;
-            pr->before(KC_ATTN);
-            LUMEN_TRY(launch_attn_decode(ctx, a));
-            pr->after();
-            // o_proj + residual, self_attention.rs:303, llama.rs:110
-            g = {};
-            g.W = w.wo; g.x = m->attn; g.y = m->h; g.N = H; g.K = m->qd; g.w_bf16 = m->bf16;
-            g.pro = PRO_NONE; g.epi = EPI_RESIDUAL; g.residual = m->x;
-            if (defer) {
-                g.pro = PRO_ATTN_FOLD; g.attn_part = m->part; g.attn_pos = m->d_pos; g.attn_nslices = m->nsplit; g.attn_d = m->D;
-                g.attn_trip = attn_decode_trip_rows(m->D); g.attn_short_rows = attn_decode_short_rows(m->D);
-            }
-            if (l == 0) { g.residual = m->embed; g.row_sel = m->d_tok; g.row_stride = H; g.residual_sel = 1; }
-            pr->before(KC_OPROJ);
-            LUMEN_TRY(launch_gemv(ctx, g));
-            pr->after();
-        }
-        if (m->chain_mlp && m->chain_ao_on) {
-            // narrow models: post_attention_layernorm + gate|up + silu*up + down + residual as one launch
-            MlpChainArgs mc = {};
-            mc.Wgu = w.wgu; mc.h = m->h; mc.norm_w = w.post_norm; mc.eps = c.rms_norm_eps; mc.Wdown = w.wdown; mc.y = m->x;
-            mc.N = H; mc.I = I; mc.w_bf16 = m->bf16; mc.act_tagged = m->act_tagged; mc.step_dev = m->d_step;
-            mc.tag_mul = (unsigned)c.num_hidden_layers; mc.tag_add = (unsigned)l + 1u;
-            mc.err_dev = m->d_err; mc.spin_limit = m->spin_limit;
-            mc.pre_sleep = m->mlp_pre; mc.poll_delay = m->mlp_delay; mc.poll_gap = m->mlp_gap;
-            pr->before(KC_MLP);
-            LUMEN_TRY(launch_mlp_chain(ctx, mc));
-            pr->after();
-            continue;
-        }
-        // post_attention_layernorm + gate|up + silu*up, llama.rs:113, :60-63
-        g = {};
-        g.W = w.wgu; g.x = m->h; g.y = m->act; g.N = 2 * I; g.K = H; g.w_bf16 = m->bf16;
-        g.pro = PRO_RMSNORM; g.norm_w = w.post_norm; g.eps = c.rms_norm_eps; g.epi = EPI_SWIGLU;
-        pr->before(KC_GATEUP);
-        LUMEN_TRY(launch_gemv(ctx, g));
-        pr->after();
-        // down_proj + residual, llama.rs:64, :115
-        g = {};
-        g.W = w.wdown; g.x = m->act; g.y = m->x; g.N = H; g.K = I; g.w_bf16 = m->bf16;
-        g.pro = PRO_NONE; g.epi = EPI_RESIDUAL; g.residual = m->h;
-        pr->before(KC_DOWN);
-        LUMEN_TRY(launch_gemv(ctx, g));
-        pr->after();
-    }
+    const int H = c.hidden_size, V = c.vocab_size;
+    // Embedding::forward (llama.rs:191) is folded into the first layer: its launches read row *d_tok of the table
+    for (int l = 0; l < c.num_hidden_layers; ++l)
+        LUMEN_TRY(enqueue_decoder_layer(m, m->layers[l], m->k_slab + m->cache_stride * l, m->v_slab + m->cache_stride * l,
+                                        l == 0 ? m->embed : m->x, l == 0 ? m->d_tok : nullptr, m->x,
+                                        (unsigned)c.num_hidden_layers, (unsigned)l, pr));
     // final norm + lm_head, llama.rs:202-205
     GemvArgs g = {};
     g.W = m->lm_head; g.x = m->x; g.y = m->logits; g.N = V; g.K = H;
