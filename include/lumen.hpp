@@ -693,6 +693,33 @@ inline int32_t sample_top_p(const std::vector<float> &logits, float temperature,
     return pick;
 }
 
+// LlamaDecoderLayer::forward_infer for ONE token as one operator call (llama.rs:104-116 behind
+// lumen_decoder_layer_decode_f32): the launches of the model-level decode step -- three per layer where the chained
+// launch covers the shape -- for an integration that replaces the reference layer by layer.  One object serves every
+// layer of a stack; weights in the fused layouts (q|k|v rows one after the other, gate / up rows interleaved:
+// lumen_interleave_rows).  No counterpart in the reference.
+class DecoderLayerStep {
+  public:
+    DecoderLayerStep(const lumen_llama_config &cfg, ContextPtr ctx = nullptr) : ctx_(ctx ? std::move(ctx) : Context::global()) {
+        check(lumen_decoder_layer_create(ctx_->handle(), &cfg, &h_));
+    }
+    ~DecoderLayerStep() {
+        if (h_) lumen_decoder_layer_destroy(h_);
+    }
+    DecoderLayerStep(const DecoderLayerStep &) = delete;
+    DecoderLayerStep &operator=(const DecoderLayerStep &) = delete;
+    // y = layer(x) for the token at position cache.len; the cache length advances by one
+    void decode(KVCacheInner &cache, const Tensor &wqkv, const Tensor &wo, const Tensor &wgu, const Tensor &wdown,
+                const Tensor &input_norm, const Tensor &post_norm, const Tensor &x, Tensor &y) {
+        check(lumen_decoder_layer_decode_f32(h_, cache.handle(), wqkv.ptr(), wo.ptr(), wgu.ptr(), wdown.ptr(), input_norm.ptr(),
+                                             post_norm.ptr(), nullptr, nullptr, x.ptr(), y.ptr()));
+    }
+
+  private:
+    ContextPtr ctx_;
+    lumen_decoder_layer *h_ = nullptr;
+};
+
 // ----------------------------------------------------------------------------- engine
 // No counterpart in the reference: the same network as LlamaModel with its weights in fused
 // layouts (q|k|v rows concatenated, gate/up rows interleaved), five kernels per layer and one

@@ -361,6 +361,31 @@ int lumen_llama_cache_upload(lumen_llama *model, int layer, const float *k_host,
 /* bytes of weights + KV prefix one decode step at cache length len must read */
 int lumen_llama_decode_bytes(const lumen_llama *model, int len, double *bytes_out);
 
+/* ---- layer level: LlamaDecoderLayer::forward_infer for ONE token (src/models/llama.rs:104-116) as one operator.
+ * y = h + down(silu(gate(n2)) * up(n2)), h = x + o_proj(attention(q|k|v(n1))), n1 = RMSNorm(x), n2 = RMSNorm(h), with
+ * RoPE and the append of the new row to `cache` -- the launches of the model-level decode step: three per layer
+ * (q|k|v + attention + o_proj chained in one, gate|up, down), two where gate|up + down chain as well, five where no
+ * chain covers the shape; the cache length advances by one.
+ * lumen_decoder_layer holds what such a step needs besides weights and cache (activations, RoPE tables, the words
+ * values travel in between workgroups, the position counter in device memory); one handle serves every layer of a
+ * stack that is called layer by layer.  cfg: hidden_size, intermediate_size, num_attention_heads,
+ * num_key_value_heads, head_dim, qk_norm, rms_norm_eps, max_seq_len, rope_theta, weight_dtype (vocab_size,
+ * num_hidden_layers and tie_embeddings are ignored).  Weights as the model keeps them: wqkv [(n_head + 2 n_kv_head) *
+ * head_dim, hidden] = the rows of w_q, w_k, w_v one after the other; wo [hidden, n_head * head_dim]; wgu
+ * [2 * intermediate, hidden] = gate / up rows interleaved (lumen_interleave_rows); wdown [hidden, intermediate]; f32 or
+ * bf16 bits by cfg.weight_dtype; norm gains f32, q_norm / k_norm [head_dim] exactly when cfg.qk_norm.
+ * x, y [hidden] f32 (may be the same array).  cache: batch 1, n_kv_head x max_seq_len x head_dim.
+ * Every call is a set of launches of its own whose arguments carry the call's tag: not for replay from a recorded
+ * graph (lumen_llama_* records its steps itself).  A wait inside a chained launch that runs out is reported by the
+ * next lumen_ctx_synchronize / lumen_download on the context.  Errors: KV overflow like lumen_attn_decode_f32. */
+typedef struct lumen_decoder_layer lumen_decoder_layer;
+int lumen_decoder_layer_create(lumen_ctx *ctx, const lumen_llama_config *cfg, lumen_decoder_layer **out);
+int lumen_decoder_layer_destroy(lumen_decoder_layer *layer);
+int lumen_decoder_layer_decode_f32(lumen_decoder_layer *layer, lumen_kv_cache *cache, const void *wqkv_dev,
+                                   const void *wo_dev, const void *wgu_dev, const void *wdown_dev,
+                                   const float *input_norm_dev, const float *post_norm_dev, const float *q_norm_dev,
+                                   const float *k_norm_dev, const float *x_dev, float *y_dev);
+
 #ifdef __cplusplus
 }
 #endif

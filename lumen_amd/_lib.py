@@ -118,6 +118,9 @@ SIGNATURES = {
     "lumen_llama_cache_download": (_i, [_vp, _i, _vp, _vp]),
     "lumen_llama_cache_upload": (_i, [_vp, _i, _vp, _vp]),
     "lumen_llama_decode_bytes": (_i, [_vp, _i, C.POINTER(C.c_double)]),
+    "lumen_decoder_layer_create": (_i, [_vp, C.POINTER(LlamaConfigStruct), _pp]),
+    "lumen_decoder_layer_destroy": (_i, [_vp]),
+    "lumen_decoder_layer_decode_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
 }
 
 

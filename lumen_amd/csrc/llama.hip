@@ -25,6 +25,8 @@ struct lumen_llama {
     lumen_llama_config cfg = {};
     int D = 0, qd = 0, kvd = 0, qkvd = 0;
     bool bf16 = false;
+    bool layer_only = false;  // the state of a decode step without a model (lumen_decoder_layer_*)
+    unsigned layer_epoch = 0;  // ... and the count of its launches, which their hand-over tags are made of
     size_t esz = 4;
     float scale = 0.f;
     float *embed = nullptr;    // [V,H] f32 (bf16 sources are widened: same values)
@@ -116,7 +118,10 @@ extern "C" int lumen_llama_destroy(lumen_llama *m) {
 static int ensure_prefill_buffers(lumen_llama *m, int s, bool all_rows);
 static int ensure_decode_graph(lumen_llama *m);
 
-extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg, lumen_llama **out) {
+// layer_only: the state of a decode step without a model around it -- activations, RoPE tables, hand-over words,
+// position counter, launch choices -- for the layer-level operator (lumen_decoder_layer_*): no weights, no caches, no
+// logits, no prompt-pass buffers, no recorded step.
+static int llama_create_impl(lumen_ctx *ctx, const lumen_llama_config *cfg, bool layer_only, lumen_llama **out) {
     if (!ctx || !cfg || !out) LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_create: null argument");
     *out = nullptr;
     const int H = cfg->hidden_size, I = cfg->intermediate_size, V = cfg->vocab_size, L = cfg->num_hidden_layers;
@@ -145,8 +150,10 @@ extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg,
     m->esz = m->bf16 ? 2 : 4;
     m->scale = 1.0f / sqrtf((float)D);  // self_attention.rs:89 (sqrt().recip())
     m->layers.resize(L);
+    m->layer_only = layer_only;
     int rc = LUMEN_OK;
 #define M_TRY(e) do { rc = (e); if (rc != LUMEN_OK) { lumen_llama_destroy(m); return rc; } } while (0)
+    if (!layer_only) {
     M_TRY(dmalloc_weight(m, (void **)&m->embed, (size_t)V * H * sizeof(float)));
     if (cfg->tie_embeddings && !m->bf16) {
         m->lm_head = m->embed;
@@ -173,6 +180,7 @@ extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg,
             M_TRY(fill_ones(m, w.k_norm, D));
         }
     }
+    }
     // one RoPE table for all layers (the reference builds an identical one per layer, self_attention.rs:78)
     {
         std::vector<float> c, s;
@@ -184,22 +192,24 @@ extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg,
     }
     // init_kv_caches(1), llama.rs:161-169: zero-filled [1,Hkv,max_seq,D] per layer
     m->cache_stride = (size_t)Hkv * cfg->max_seq_len * D;
-    M_TRY(dmalloc_t(m, &m->k_slab, m->cache_stride * L));
-    M_TRY(dmalloc_t(m, &m->v_slab, m->cache_stride * L));
-    if (hipMemsetAsync(m->k_slab, 0, m->cache_stride * L * sizeof(float), ctx->stream) != hipSuccess ||
-        hipMemsetAsync(m->v_slab, 0, m->cache_stride * L * sizeof(float), ctx->stream) != hipSuccess) {
-        lumen_llama_destroy(m);
-        LUMEN_FAIL(LUMEN_ERR_HIP, "llama_create: clearing the KV slab failed");
+    if (!layer_only) {
+        M_TRY(dmalloc_t(m, &m->k_slab, m->cache_stride * L));
+        M_TRY(dmalloc_t(m, &m->v_slab, m->cache_stride * L));
+        if (hipMemsetAsync(m->k_slab, 0, m->cache_stride * L * sizeof(float), ctx->stream) != hipSuccess ||
+            hipMemsetAsync(m->v_slab, 0, m->cache_stride * L * sizeof(float), ctx->stream) != hipSuccess) {
+            lumen_llama_destroy(m);
+            LUMEN_FAIL(LUMEN_ERR_HIP, "llama_create: clearing the KV slab failed");
+        }
     }
     M_TRY(dmalloc_t(m, &m->x, (size_t)H));
     M_TRY(dmalloc_t(m, &m->h, (size_t)H));
     M_TRY(dmalloc_t(m, &m->qkv, (size_t)m->qkvd));
     M_TRY(dmalloc_t(m, &m->attn, (size_t)m->qd));
     M_TRY(dmalloc_t(m, &m->act, (size_t)I));
-    M_TRY(dmalloc_t(m, &m->logits, (size_t)V));
+    if (!layer_only) M_TRY(dmalloc_t(m, &m->logits, (size_t)V));
     M_TRY(dmalloc_t(m, &m->d_tok, 4));
     M_TRY(dmalloc_t(m, &m->d_pos, 4));
-    M_TRY(dmalloc_t(m, &m->tok_hist, (size_t)cfg->max_seq_len + 1));
+    if (!layer_only) M_TRY(dmalloc_t(m, &m->tok_hist, (size_t)cfg->max_seq_len + 1));
     m->nsplit = attn_decode_nsplit(cfg->max_seq_len, D);
     // Where a cache is cut into 2 to 16 slices the o_proj GEMV can fold the slices' partial states while it
     // stages its input: an atomic and a second round of loads fewer inside the attention kernel.  With more
@@ -263,11 +273,18 @@ extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg,
         }
     }
     m->decode_mode = LUMEN_DECODE_GRAPH;
-    // buffers of a prompt pass of up to 512 rows now, not under the first prompt (longer prompts grow them)
-    M_TRY(ensure_prefill_buffers(m, std::min(cfg->max_seq_len, 512), false));
-    // ... and the decode step recorded and instantiated for a short cache (recorded again when the cache outgrows it)
-    M_TRY(ensure_decode_graph(m));
-    if (m->graph_exec) hipGraphUpload(m->graph_exec, ctx->stream);
+    if (layer_only) {
+        m->decode_mode = LUMEN_DECODE_EAGER;
+        // (its launches are not followed by a call of this library that synchronises: a wait that runs out is flagged
+        // where lumen_ctx_synchronize / lumen_download find it)
+        m->d_err = ctx->err_host;
+    } else {
+        // buffers of a prompt pass of up to 512 rows now, not under the first prompt (longer prompts grow them)
+        M_TRY(ensure_prefill_buffers(m, std::min(cfg->max_seq_len, 512), false));
+        // ... and the decode step recorded and instantiated for a short cache (recorded again when the cache outgrows it)
+        M_TRY(ensure_decode_graph(m));
+        if (m->graph_exec) hipGraphUpload(m->graph_exec, ctx->stream);
+    }
     if (hipStreamSynchronize(ctx->stream) != hipSuccess) {
         lumen_llama_destroy(m);
         LUMEN_FAIL(LUMEN_ERR_HIP, "llama_create: preparing the decode graph failed");
@@ -275,6 +292,10 @@ extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg,
 #undef M_TRY
     *out = m;
     return LUMEN_OK;
+}
+
+extern "C" int lumen_llama_create(lumen_ctx *ctx, const lumen_llama_config *cfg, lumen_llama **out) {
+    return llama_create_impl(ctx, cfg, false, out);
 }
 
 // ----------------------------------------------------------- parameter upload
@@ -986,6 +1007,70 @@ extern "C" int lumen_llama_profile_kernel_name(const lumen_llama *m, int kernel_
     if (kernel_class < 0 || kernel_class >= KC_COUNT)
         LUMEN_FAIL(LUMEN_ERR_INVALID, "llama_profile_kernel_name: class %d of %d", kernel_class, (int)KC_COUNT);
     snprintf(buf, (size_t)buf_len, "%s", m->prof_names[kernel_class].c_str());
+    return LUMEN_OK;
+}
+
+// ---------------------------------------------------------------- the layer-level operator
+struct lumen_decoder_layer {
+    lumen_llama *m = nullptr;
+};
+
+__global__ void set_pos_kernel(int *p, int v) { *p = v; }
+
+extern "C" int lumen_decoder_layer_create(lumen_ctx *ctx, const lumen_llama_config *cfg, lumen_decoder_layer **out) {
+    if (!ctx || !cfg || !out) LUMEN_FAIL(LUMEN_ERR_INVALID, "decoder_layer_create: null argument");
+    *out = nullptr;
+    lumen_llama_config c = *cfg;
+    c.vocab_size = 1;         // (no embedding, no lm_head here)
+    c.num_hidden_layers = 1;
+    c.tie_embeddings = 0;
+    lumen_llama *m = nullptr;
+    LUMEN_TRY(llama_create_impl(ctx, &c, true, &m));
+    lumen_decoder_layer *h = new lumen_decoder_layer();
+    h->m = m;
+    *out = h;
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_decoder_layer_destroy(lumen_decoder_layer *h) {
+    if (!h) return LUMEN_OK;
+    lumen_llama_destroy(h->m);
+    delete h;
+    return LUMEN_OK;
+}
+
+extern "C" int lumen_decoder_layer_decode_f32(lumen_decoder_layer *h, lumen_kv_cache *cache, const void *wqkv, const void *wo,
+                                              const void *wgu, const void *wdown, const float *input_norm, const float *post_norm,
+                                              const float *q_norm, const float *k_norm, const float *x, float *y) {
+    if (!h || !cache || !wqkv || !wo || !wgu || !wdown || !input_norm || !post_norm || !x || !y)
+        LUMEN_FAIL(LUMEN_ERR_INVALID, "decoder_layer_decode: null argument");
+    lumen_llama *m = h->m;
+    const lumen_llama_config &c = m->cfg;
+    if (cache->ctx != m->ctx) LUMEN_FAIL(LUMEN_ERR_INVALID, "decoder_layer_decode: the cache belongs to another context");
+    if (cache->b != 1 || cache->h_kv != c.num_key_value_heads || cache->d != m->D || cache->max_seq != c.max_seq_len)
+        LUMEN_FAIL(LUMEN_ERR_SHAPE, "decoder_layer_decode: cache [%d, %d, %d, %d] against a layer of %d kv heads x %d, %d rows",
+                   cache->b, cache->h_kv, cache->max_seq, cache->d, c.num_key_value_heads, m->D, c.max_seq_len);
+    if ((c.qk_norm != 0) != (q_norm != nullptr && k_norm != nullptr))
+        LUMEN_FAIL(LUMEN_ERR_INVALID, "decoder_layer_decode: q/k norm gains %s", c.qk_norm ? "missing" : "given to a layer without q/k norm");
+    if (cache->len + 1 > cache->max_seq)  // self_attention.rs:144-149
+        LUMEN_FAIL(LUMEN_ERR_KV_OVERFLOW, "KV cache overflow: new_len=%d > max_seq=%d", cache->len + 1, cache->max_seq);
+    HIP_TRY(hipSetDevice(m->ctx->device));
+    // the position lives in device memory (the launches read it there); it follows the cache's length, which
+    // changes once per token for a stack of layers that share this state
+    if (m->len != cache->len || m->layer_epoch == 0) {
+        m->len = cache->len;
+        hipLaunchKernelGGL(set_pos_kernel, dim3(1), dim3(1), 0, m->ctx->stream, m->d_pos, m->len);
+        LUMEN_CHECK_LAUNCH();
+    }
+    LayerW w;
+    w.wqkv = const_cast<void *>(wqkv); w.wo = const_cast<void *>(wo); w.wgu = const_cast<void *>(wgu); w.wdown = const_cast<void *>(wdown);
+    w.in_norm = const_cast<float *>(input_norm); w.post_norm = const_cast<float *>(post_norm);
+    w.q_norm = const_cast<float *>(q_norm); w.k_norm = const_cast<float *>(k_norm);
+    // the hand-over tags of this call's launches: every call its own (the step counter in device memory stays 0 here)
+    if (++m->layer_epoch >= 0xfffffff0u) m->layer_epoch = 1;
+    StepProbe none;
+    LUMEN_TRY(enqueue_decoder_layer(m, w, cache->k, cache->v, x, nullptr, y, 0u, m->layer_epoch, &none));
+    cache->len += 1;
     return LUMEN_OK;
 }
 

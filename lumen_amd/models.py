@@ -273,7 +273,19 @@ class LlamaDecoderLayer:
                                        None, 0.0, _lib.GEMV_EPI_RESIDUAL, hbuf.ptr))
         return out, cache
 
-    def forward_infer(self, x, cache):
+    def forward_token_layer_op(self, x, cache, op):
+        """forward_infer for S == 1 as ONE operator call (lumen_decoder_layer_decode_f32): the launches of the
+        model-level decode step, three per layer where the chained launch covers the shape."""
+        out = Tensor.empty(x.shape, np.float32, self.self_attn.ctx)
+        check(lib.lumen_decoder_layer_decode_f32(op.handle, cache.handle, self.w_qkv.ptr, self.self_attn.w_o.weight.ptr,
+                                                 self.w_gate_up.ptr, self.mlp.down_proj.weight.ptr,
+                                                 self.input_layernorm.weight.ptr, self.post_attention_layernorm.weight.ptr,
+                                                 None, None, x.ptr, out.ptr))
+        return out, cache
+
+    def forward_infer(self, x, cache, layer_op=None):
+        if layer_op is not None and x.shape[0] == 1 and x.shape[1] == 1:
+            return self.forward_token_layer_op(x, cache, layer_op)
         if getattr(self, "fused", False) and x.shape[0] == 1 and x.shape[1] == 1:
             return self.forward_token(x, cache)
         norm_x = self.input_layernorm.forward(x)
@@ -284,12 +296,37 @@ class LlamaDecoderLayer:
         return h + mlp_out, cache_out
 
 
+class DecoderLayerOp:
+    """The state a layer-level decode step needs besides weights and cache (lumen_decoder_layer): one serves all
+    layers of a stack."""
+
+    def __init__(self, config, ctx=None):
+        if isinstance(config, dict):
+            config = LlamaConfig.from_dict(config)
+        self.ctx = ctx or default_ctx()
+        c = _lib.LlamaConfigStruct(
+            config.vocab_size, config.hidden_size, config.intermediate_size, config.num_hidden_layers,
+            config.num_attention_heads, config.num_key_value_heads, config.rms_norm_eps, config.max_seq_len,
+            config.rope_theta, config.head_dim or 0, int(config.qk_norm), int(config.tie_embeddings),
+            _lib.DTYPE_BF16 if config.weight_dtype == "bf16" else _lib.DTYPE_F32)
+        h = C.c_void_p()
+        check(lib.lumen_decoder_layer_create(self.ctx.handle, C.byref(c), C.byref(h)))
+        self.handle = h
+
+    def __del__(self):
+        h, self.handle = getattr(self, "handle", None), None
+        if h:
+            lib.lumen_decoder_layer_destroy(h)
+
+
 class LayeredLlamaModel:
     """LlamaModel::forward (llama.rs:181-206) composed operator by operator.  fused=True (default): a single
     token (S == 1) takes the fused operators -- five launches per layer, and the final norm rides on the lm_head
-    product -- as the model-level decode step does; fused=False: one call per reference leaf, every time."""
+    product -- as the model-level decode step does; fused=False: one call per reference leaf, every time;
+    layer_op=True: a single token takes ONE operator call per layer (lumen_decoder_layer_decode_f32: the chained
+    launches of the model-level step, three per layer where they cover the shape)."""
 
-    def __init__(self, config, params, ctx=None, fused=True):
+    def __init__(self, config, params, ctx=None, fused=True, layer_op=False):
         if isinstance(config, dict):
             config = LlamaConfig.from_dict(config)
         if config.head_dim or config.qk_norm or config.tie_embeddings or config.weight_dtype != "f32":
@@ -301,7 +338,8 @@ class LayeredLlamaModel:
                        for i in range(config.num_hidden_layers)]
         self.norm = RMSNorm(config.hidden_size, config.rms_norm_eps, params["model.norm.weight"], self.ctx)
         self.lm_head = Linear(Tensor.from_array_no_grad(params["lm_head.weight"], self.ctx))
-        self.fused = bool(fused)
+        self.fused = bool(fused) or bool(layer_op)
+        self.layer_op = DecoderLayerOp(config, self.ctx) if layer_op else None
         if self.fused:
             for layer in self.layers:
                 layer.fuse()
@@ -323,7 +361,7 @@ class LayeredLlamaModel:
         ids = np.ascontiguousarray(input_ids, np.float32).reshape(1, -1)
         x = self.embed_tokens.forward(ids)
         for i, layer in enumerate(self.layers):
-            x, caches[i] = layer.forward_infer(x, caches[i])
+            x, caches[i] = layer.forward_infer(x, caches[i], self.layer_op)
         if self.fused and ids.shape[1] == 1:  # final norm + lm_head in one launch (llama.rs:202-205)
             w = self.lm_head.weight
             logits = Tensor.empty((1, 1, w.shape[0]), np.float32, self.ctx)

@@ -130,6 +130,9 @@ extern "C" {
     pub fn lumen_llama_cache_download(model: *mut lumen_llama, layer: c_int, k_host: *mut c_float, v_host: *mut c_float) -> c_int;
     pub fn lumen_llama_cache_upload(model: *mut lumen_llama, layer: c_int, k_host: *const c_float, v_host: *const c_float) -> c_int;
     pub fn lumen_llama_decode_bytes(model: *const lumen_llama, len: c_int, bytes_out: *mut f64) -> c_int;
+    pub fn lumen_decoder_layer_create(ctx: *mut lumen_ctx, cfg: *const lumen_llama_config, out: *mut *mut lumen_decoder_layer) -> c_int;
+    pub fn lumen_decoder_layer_destroy(layer: *mut lumen_decoder_layer) -> c_int;
+    pub fn lumen_decoder_layer_decode_f32(layer: *mut lumen_decoder_layer, cache: *mut lumen_kv_cache, wqkv_dev: *const c_void, wo_dev: *const c_void, wgu_dev: *const c_void, wdown_dev: *const c_void, input_norm_dev: *const c_float, post_norm_dev: *const c_float, q_norm_dev: *const c_float, k_norm_dev: *const c_float, x_dev: *const c_float, y_dev: *mut c_float) -> c_int;
 }
 
 /// status -> panic with the library's message: the reference's own error behaviour (Cargo.toml: panic = "abort")

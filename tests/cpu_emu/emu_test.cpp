@@ -7,7 +7,7 @@
 // streaming vector-matrix product and the stand-alone decode attention those forms fall back to, the latter also
 // at operator level over a sliced cache (slices merged inside the launch).
 //
-//   emu_test [case ...]      cases: chain sliced qknorm bf16 skinny attn (default: all)
+//   emu_test [case ...]      cases: chain sliced qknorm bf16 skinny attn layerop (default: all)
 #include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -343,6 +343,71 @@ static void case_attn(lumen_ctx *ctx) {
     OK(lumen_rope_destroy(rope));
 }
 
+// LlamaDecoderLayer::forward_infer for one token as ONE operator call per layer (lumen_decoder_layer_decode_f32): two
+// layers of the chain shape driven layer by layer, embedding row in, final norm + lm_head by the checker's own
+// operators, against the checker's whole-model step
+static void case_layerop(lumen_ctx *ctx) {
+    printf("layerop: lumen_decoder_layer_decode_f32, two layers of hidden 512, 8/2 heads of 64, intermediate 1024\n");
+    const int V = 96, H = 512, I = 1024, L = 2, hq = 8, hkv = 2, D = 64, max_seq = 256;
+    Model m = build(ctx, V, H, I, L, hq, hkv, 0, max_seq, false, false, false);
+    lumen_decoder_layer *op = nullptr;
+    OK(lumen_decoder_layer_create(ctx, &m.cfg, &op));
+    // the layers' weights laid out as the fused step wants them: q|k|v rows one after the other, gate / up interleaved
+    // (m.keep: embed, final norm, lm_head, then per layer wq wk wv wo gate up down input_norm post_norm)
+    struct Dev { void *wqkv, *wo, *wgu, *wdown, *n1, *n2; lumen_kv_cache *cache; } dev[2];
+    const size_t qd = (size_t)hq * D, kvd = (size_t)hkv * D;
+    for (int l = 0; l < L; ++l) {
+        const std::vector<float> *w = &m.keep[3 + (size_t)l * 9];
+        std::vector<float> qkv;
+        for (int i = 0; i < 3; ++i) qkv.insert(qkv.end(), w[i].begin(), w[i].end());
+        std::vector<float> gu((size_t)2 * I * H);
+        for (int i = 0; i < I; ++i) {
+            memcpy(&gu[(size_t)(2 * i) * H], &w[4][(size_t)i * H], sizeof(float) * H);
+            memcpy(&gu[(size_t)(2 * i + 1) * H], &w[5][(size_t)i * H], sizeof(float) * H);
+        }
+        auto up = [&](const std::vector<float> &v) {
+            void *d;
+            OK(lumen_malloc(ctx, v.size() * 4, &d));
+            OK(lumen_upload(ctx, d, v.data(), v.size() * 4));
+            return d;
+        };
+        CHECK(qkv.size() == (qd + 2 * kvd) * H, "q|k|v rows");
+        dev[l].wqkv = up(qkv); dev[l].wo = up(w[3]); dev[l].wgu = up(gu); dev[l].wdown = up(w[6]);
+        dev[l].n1 = up(w[7]); dev[l].n2 = up(w[8]);
+        OK(lumen_kv_cache_create(ctx, 1, hkv, max_seq, D, &dev[l].cache));
+    }
+    void *dx;
+    OK(lumen_malloc(ctx, (size_t)H * 4, &dx));
+    std::vector<float> x(H), nx(H), got(V), ref(V);
+    int tok = 11;
+    for (int t = 0; t < 3; ++t) {
+        OK(lumen_upload(ctx, dx, m.keep[0].data() + (size_t)tok * H, (size_t)H * 4));  // Embedding::forward
+        for (int l = 0; l < L; ++l)
+            OK(lumen_decoder_layer_decode_f32(op, dev[l].cache, dev[l].wqkv, dev[l].wo, dev[l].wgu, dev[l].wdown,
+                                              (const float *)dev[l].n1, (const float *)dev[l].n2, nullptr, nullptr,
+                                              (const float *)dx, (float *)dx));
+        OK(lumen_download(ctx, x.data(), dx, (size_t)H * 4));
+        lo_rmsnorm_f32(x.data(), m.keep[1].data(), nx.data(), 1, H, m.cfg.rms_norm_eps);
+        lo_gemv_f32(m.keep[2].data(), nx.data(), got.data(), V, H);
+        const float f = (float)tok;
+        lo_llama_forward(m.ora, &f, 1, ref.data());
+        const double e = max_rel(got.data(), ref.data(), ref.size());
+        printf("  token %d through %d layer calls: max rel err %.2e\n", t, L, e);
+        CHECK(e <= 1e-4, "layer operator, token %d: %.3g", t, e);
+        tok = (tok * 5 + 1) % V;
+    }
+    int len = 0;
+    OK(lumen_kv_cache_len(dev[1].cache, &len));
+    CHECK(len == 3, "cache length %d", len);
+    for (int l = 0; l < L; ++l) {
+        for (void *p : {dev[l].wqkv, dev[l].wo, dev[l].wgu, dev[l].wdown, dev[l].n1, dev[l].n2}) OK(lumen_free(ctx, p));
+        OK(lumen_kv_cache_destroy(dev[l].cache));
+    }
+    OK(lumen_free(ctx, dx));
+    OK(lumen_decoder_layer_destroy(op));
+    destroy(m);
+}
+
 // The harness checks itself: a product whose output array is one element short must be stopped by the sanitizer.
 static void selfcheck_oob(lumen_ctx *ctx) {
     const int N = 64, K = 256;
@@ -367,7 +432,7 @@ int main(int argc, char **argv) {
         return 0;  // (reached only if nothing stopped the program: the test expects a sanitizer report instead)
     }
     struct { const char *name; void (*fn)(lumen_ctx *); } cases[] = {
-        {"chain", case_chain}, {"sliced", case_sliced}, {"qknorm", case_qknorm}, {"bf16", case_bf16}, {"skinny", case_skinny}, {"attn", case_attn}};
+        {"chain", case_chain}, {"sliced", case_sliced}, {"qknorm", case_qknorm}, {"bf16", case_bf16}, {"skinny", case_skinny}, {"attn", case_attn}, {"layerop", case_layerop}};
     for (const auto &c : cases) {
         bool run = argc <= 1;
         for (int i = 1; i < argc; ++i) run = run || !strcmp(argv[i], c.name);

@@ -171,6 +171,38 @@ def test_layered_operator_path_matches_fused_path_and_oracle(fused_ops):
         _layered_checks(layered, fused, ora, ids, caches)
 
 
+@pytest.mark.parametrize("cfg_extra", [dict(), dict(intermediate_size=1024),
+                                       dict(hidden_size=128, intermediate_size=352, max_seq_len=200)],
+                         ids=["chain-3-launches", "chain+mlp-chain-2-launches", "no-chain-5-launches"])
+def test_layer_level_operator_matches_the_oracle_across_a_trip_boundary(cfg_extra):
+    """LlamaDecoderLayer::forward_infer for one token as ONE operator call per layer
+    (lumen_decoder_layer_decode_f32): the model-level step's launches behind a layer-granular interface.  Prompt
+    through the leaf operators, then single tokens through the layer operator, across 256 cached rows (a second trip
+    of rows), against the checker and against the model-level path."""
+    cfg = dict(CHAIN, max_seq_len=300)
+    cfg.update(cfg_extra)
+    params = synth.make_params(cfg, seed=61, std=0.1, gains_one=False)
+    layered = LayeredLlamaModel(cfg, params, layer_op=True)
+    ora = lo.Llama(cfg, params)
+    fused = LlamaModel(cfg)
+    fused.load_params(params)
+    n_prompt = 250 if cfg["max_seq_len"] >= 300 else 20
+    ids = synth.make_tokens(n_prompt + 12, cfg["vocab_size"], seed=61)
+    caches = layered.init_kv_caches(1)
+    with no_grad():
+        a = layered.forward(ids[:n_prompt], caches).data()[0]
+        _, r = ora.forward(ids[:n_prompt])
+        assert max_rel(a, r) <= 1e-4
+        fused.forward(ids[:n_prompt], all_rows=False)
+        for t in range(n_prompt, n_prompt + 12):
+            a = layered.forward(ids[t:t + 1], caches).data()[0, 0]
+            _, r = ora.forward(ids[t:t + 1])
+            assert max_rel(a, r[0]) <= 1e-4, t
+            assert max_rel(fused.forward(ids[t:t + 1], all_rows=False), a) <= 2e-5, t
+    assert caches[0].len == caches[-1].len == n_prompt + 12
+    layered.ctx.synchronize()  # (would report a hand-over wait that ran out)
+
+
 def _layered_checks(layered, fused, ora, ids, caches):
     a = layered.forward(ids[:15], caches).data()[0]
     rc, r = ora.forward(ids[:15])
