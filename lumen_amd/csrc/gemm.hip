@@ -548,6 +548,169 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(GemmArgs a, int
     }
 }
 
+// Prompts of five to 32 rows (a chat turn's new tokens, the tail of a chunked prompt): the product is bound by the
+// weights, and the tile kernels above take the same ~100 us per layer for 5 rows as for 128.  This kernel streams W once
+// and multiplies on the matrix cores without sharing anything between wavefronts: a wavefront owns 16 rows of W (a column
+// tile of C; N / 16 tiles spread evenly over the compute units where N / 32 would not) over a range of K and all
+// MT <= 2 row tiles of 16 rows of A.  It fetches 16 x 32 blocks of W (GS_DW blocks ahead: 16 KB per wavefront in flight,
+// what the single-row product keeps in flight) and 16 x 32 blocks of A (those come from L2) with coalesced 16-byte loads,
+// turns them into operand order through a wavefront-private LDS buffer (no barriers) and multiplies with the f32
+// matrix instruction (v_mfma_f32_16x16x4_f32: a sixteenth of the bf16 rate, but no splitting into bf16 parts on the
+// vector ALU, which is what bounded a bf16-part form of this kernel -- 31 us for the 92 MB gate|up matrix against 25; every
+// further row tile costs 20 us per layer in f32 matrix instructions, so beyond 32 rows the tile kernels are as fast).  The four wavefronts of a
+// workgroup take consecutive K ranges of ONE column tile and add their accumulators through LDS in wavefront order; ranges
+// are split further over gridDim.z like the tile kernels' (partial tiles of M x 16).
+#define GS_KW 32           // k per block of W (128 and 256, longer visits to a row, measured no faster: 23.6 and 35 against 24.7 us)
+#define GS_LW (GS_KW + 4)  // floats per LDS row of a staged block of W: rows start 4 banks apart, 8 rows cover all banks
+#define GS_LA 36           // ... of a 32-wide block of A
+#define GS_DW 8            // blocks of W in flight per wavefront (16 KB)
+#define GS_DA 2            // 32-wide blocks of A in flight
+typedef float v4acc __attribute__((ext_vector_type(4)));
+template <int MT, int EPI, bool PARTIAL>
+__global__ __launch_bounds__(256) void gemm_stream_kernel(GemmArgs a) {
+    constexpr int WP = GS_KW / 16;   // 16-byte pieces of a W block per lane: 16 rows x GS_KW / 4 pieces / 64 lanes
+    constexpr int SUB = GS_KW / 32;  // 32-wide blocks of A per block of W
+    constexpr int RL = 64 * 4 / GS_KW;  // rows of W one load instruction covers
+    __shared__ __align__(16) float stage_w[4][16 * GS_LW];
+    __shared__ __align__(16) float stage_a[4][MT][16 * GS_LA];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int c = lane & 15, g = lane >> 4;
+    const int bn = blockIdx.x * 16;
+    const int M = a.M, N = a.N, K = a.K;
+    const float *A = a.A;
+    const float *W = (const float *)a.W;
+    // blocks of GS_KW k: this workgroup's share [z per_wg, (z + 1) per_wg), this wavefront's quarter of it
+    const int nblk = (K + GS_KW - 1) / GS_KW;
+    const int per_wg = (nblk + (int)gridDim.z - 1) / (int)gridDim.z;
+    const int per_wave = (per_wg + 3) / 4;
+    const int wg0 = (int)blockIdx.z * per_wg;
+    const int d0 = min(wg0 + wave * per_wave, nblk);
+    const int d1 = min(min(d0 + per_wave, wg0 + per_wg), nblk);
+
+    v4acc acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[t] = v4acc{0.f, 0.f, 0.f, 0.f};
+
+    // W: piece i of this lane in a 16 x GS_KW block is row RL i + lane / (64 / RL), k offset 4 * (lane % (64 / RL)):
+    // the lanes of a row read GS_KW * 4 contiguous bytes.  A: piece i (0, 1) of a 16 x 32 block is row 8 i + lane / 8,
+    // k offset 4 * (lane % 8).  K is a multiple of 4: a piece is inside or outside as a whole.  Rows past the end are
+    // clamped (their products are never stored).
+    const int wrow = lane / (64 / RL), wk = (lane % (64 / RL)) * 4;
+    const int arow = lane >> 3, ak = (lane & 7) * 4;
+    const float *wp = W + (size_t)min(bn + wrow, N - 1) * K + wk;
+    const size_t wstep = (size_t)RL * K;  // (rows past N - 1: the loads of the last tile are clamped one by one below)
+    const bool wclamp = bn + 16 > N;
+    const float *ap[MT][2];
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) ap[t][i] = A + (size_t)min(t * 16 + arow + 8 * i, M - 1) * K + ak;
+    v4f vw[GS_DW][WP], va[GS_DA][MT][2];
+    auto fetch_w = [&](int slot, int d) {
+        const bool in = d * GS_KW + wk < K;
+#pragma unroll
+        for (int i = 0; i < WP; ++i) {
+            vw[slot][i] = v4f{0.f, 0.f, 0.f, 0.f};
+            const float *q = wclamp ? W + (size_t)min(bn + wrow + RL * i, N - 1) * K + wk : wp + i * wstep;
+            if (in) vw[slot][i] = __builtin_nontemporal_load((const v4f *)(q + (size_t)d * GS_KW));
+        }
+    };
+    auto fetch_a = [&](int slot, int e) {  // e: index of the 32-wide block of A
+        const bool in = e * 32 + ak < K;
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                va[slot][t][i] = v4f{0.f, 0.f, 0.f, 0.f};
+                if (in) va[slot][t][i] = *(const v4f *)(ap[t][i] + e * 32);
+            }
+    };
+    float *sw = stage_w[wave];
+    auto block = [&](int ws, int d) {
+#pragma unroll
+        for (int i = 0; i < WP; ++i) *(v4f *)(sw + (wrow + RL * i) * GS_LW + wk) = vw[ws][i];
+#pragma unroll
+        for (int u = 0; u < SUB; ++u) {
+            const int as = (ws * SUB + u) % GS_DA;
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+#pragma unroll
+                for (int i = 0; i < 2; ++i) *(v4f *)(stage_a[wave][t] + (arow + 8 * i) * GS_LA + ak) = va[as][t][i];
+            // The buffers are this wavefront's own and its LDS instructions execute in order: the reads below see the
+            // writes above without a workgroup barrier (the wave barrier emits no instruction; it keeps the compiler
+            // from moving LDS accesses across it).
+            __builtin_amdgcn_wave_barrier();
+            if (d * SUB + u + GS_DA < d1 * SUB) fetch_a(as, d * SUB + u + GS_DA);
+            // lane (c, g) takes the k = 16 j + 4 g + e of row c for both operands: instruction (j, e) multiplies four k
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const v4f wf = *(const v4f *)(sw + c * GS_LW + u * 32 + j * 16 + g * 4);
+                v4f af[MT];
+#pragma unroll
+                for (int t = 0; t < MT; ++t) af[t] = *(const v4f *)(stage_a[wave][t] + c * GS_LA + j * 16 + g * 4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+#pragma unroll
+                    for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[t][e], wf[e], acc[t], 0, 0, 0);
+            }
+            __builtin_amdgcn_wave_barrier();  // (the next block's writes come after these reads)
+        }
+    };
+    // block d + j of W sits in slot j % GS_DW; the 32-wide blocks of A rotate through GS_DA slots (a trip of the loop
+    // below is a whole number of turns of that ring); a slot is requested anew as soon as its block is used
+    static_assert((GS_DW * SUB) % GS_DA == 0, "the A ring must divide a trip of the loop");
+#pragma unroll
+    for (int j = 0; j < GS_DW; ++j)
+        if (d0 + j < d1) fetch_w(j, d0 + j);
+#pragma unroll
+    for (int j = 0; j < GS_DA; ++j)
+        if (d0 * SUB + j < d1 * SUB) fetch_a(j, d0 * SUB + j);
+    for (int d = d0; d < d1; d += GS_DW) {
+#pragma unroll
+        for (int j = 0; j < GS_DW; ++j)
+            if (d + j < d1) {
+                block(j, d + j);
+                if (d + j + GS_DW < d1) fetch_w(j, d + j + GS_DW);
+            }
+    }
+    // the four K ranges of the workgroup, added in wavefront order
+    __syncthreads();
+    float *red = &stage_w[0][0];  // [3][MT][4][64] floats
+    if (wave > 0) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) red[(((wave - 1) * MT + t) * 4 + r) * 64 + lane] = acc[t][r];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w = 0; w < 3; ++w)
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[t][r] += red[((w * MT + t) * 4 + r) * 64 + lane];
+    float *part = PARTIAL ? a.part + (size_t)blockIdx.z * M * N : nullptr;
+    const int col = bn + c;
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            // accumulator register r of lane (c, g): row 4 g + r of its 16 x 16 tile, column c
+            const int row = t * 16 + g * 4 + r;
+            const float v = acc[t][r];
+            if (PARTIAL) {
+                if (row < M && col < N) part[(size_t)row * N + col] = v;
+            } else if (EPI == EPI_SWIGLU) {
+                const float up = __shfl_xor(v, 1, 64);
+                if (!(col & 1) && row < M && col < N) a.C[(size_t)row * (N >> 1) + (col >> 1)] = silu_g(v) * up;
+            } else if (row < M && col < N) {
+                const size_t o = (size_t)row * N + col;
+                a.C[o] = (EPI == EPI_RESIDUAL) ? a.residual[o] + v : v;
+            }
+        }
+}
+
 #define GEMM_MAX_SPLITS 16
 // Adds the K splits of every output element in split order and applies the epilogue.
 template <int EPI>
@@ -764,6 +927,29 @@ static int gemm_big_splits(const lumen_ctx *ctx, const GemmArgs &a) {
     return best;
 }
 
+// up to 4 rows of A the weight-streaming kernel wins (TinyLlama shape: prompt pass of 2 tokens 2.45 -> 1.48 ms, of 4
+// tokens 2.46 -> 1.89 ms); at 8 rows the two are level, beyond that the multiply-adds and LDS reads per piece cost more
+// than the tile kernels' fixed 100 us per layer
+#ifndef GEMM_SKINNY_MAX_M
+#define GEMM_SKINNY_MAX_M 4
+#endif
+// The weight-streaming matrix-core kernel takes five to 32 rows of A with f32 weights.
+#define GEMM_STREAM_MAX_M 32
+static bool gemm_stream_applies(const GemmArgs &a) {
+    const bool aligned = (((uintptr_t)a.A | (uintptr_t)a.W) & 15) == 0;
+    return !a.w_bf16 && aligned && a.K > 0 && a.K % 4 == 0 && a.M > GEMM_SKINNY_MAX_M && a.M <= GEMM_STREAM_MAX_M &&
+           !(a.epi == EPI_SWIGLU && (a.N & 1));
+}
+// Workgroups along K per column tile of 16: about three workgroups per compute unit over the chip, at least four
+// blocks of K per wavefront, 16 splits at most (the split sum takes that many).
+static int gemm_stream_splits(const lumen_ctx *ctx, const GemmArgs &a) {
+    const long tiles = (a.N + 15) / 16, nblk = (a.K + GS_KW - 1) / GS_KW;
+    long s = (3L * ctx->num_cus + tiles / 2) / tiles;
+    while (s > 1 && nblk / (4 * s) < 4) --s;
+    if (s > GEMM_MAX_SPLITS) s = GEMM_MAX_SPLITS;
+    while (s > 1 && (size_t)s * a.M * a.N * sizeof(float) > ((size_t)256 << 20)) --s;
+    return s < 1 ? 1 : (int)s;
+}
 int gemm_reserve_workspace(lumen_ctx *ctx, size_t need) {
     if (ctx->gemm_ws_bytes >= need) return LUMEN_OK;
     HIP_TRY(hipStreamSynchronize(ctx->stream));
@@ -780,17 +966,15 @@ size_t gemm_workspace_bytes(const lumen_ctx *ctx, int M, int N, int K, int w_bf1
     GemmArgs a = {};
     a.M = M; a.N = N; a.K = K; a.w_bf16 = w_bf16;
     if (M <= 0 || N <= 0 || K <= 0 || K % (w_bf16 ? 8 : 4)) return 0;
+    if (M > GEMM_SKINNY_MAX_M && M <= GEMM_STREAM_MAX_M && !w_bf16) {  // (alignment is the caller's: assume the streaming kernel)
+        const int st = gemm_stream_splits(ctx, a);
+        return st > 1 ? (size_t)st * M * N * sizeof(float) : 0;
+    }
     int splits = gemm_big_splits(ctx, a);
     if (splits <= 0) splits = gemm_splits(ctx, a);
     return splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
 }
 
-// up to 4 rows of A the weight-streaming kernel wins (TinyLlama shape: prompt pass of 2 tokens 2.45 -> 1.48 ms, of 4
-// tokens 2.46 -> 1.89 ms); at 8 rows the two are level, beyond that the multiply-adds and LDS reads per piece cost more
-// than the tile kernels' fixed 100 us per layer
-#ifndef GEMM_SKINNY_MAX_M
-#define GEMM_SKINNY_MAX_M 4
-#endif
 template <int MS, bool BF16>
 static int launch_gemm_skinny(lumen_ctx *ctx, const GemmArgs &a, int kpad) {
     const size_t lds = (size_t)MS * kpad * sizeof(float);
@@ -838,6 +1022,16 @@ static int gemm_skinny_rows(const GemmArgs &a, int *kpad_out) {
     return ms;
 }
 
+
+template <int MT>
+static void launch_gemm_stream(const GemmArgs &g, int splits, hipStream_t s) {
+    dim3 grid((g.N + 15) / 16, 1, splits);
+    if (splits > 1) hipLaunchKernelGGL((gemm_stream_kernel<MT, EPI_STORE, true>), grid, dim3(256), 0, s, g);
+    else if (g.epi == EPI_STORE) hipLaunchKernelGGL((gemm_stream_kernel<MT, EPI_STORE, false>), grid, dim3(256), 0, s, g);
+    else if (g.epi == EPI_RESIDUAL) hipLaunchKernelGGL((gemm_stream_kernel<MT, EPI_RESIDUAL, false>), grid, dim3(256), 0, s, g);
+    else hipLaunchKernelGGL((gemm_stream_kernel<MT, EPI_SWIGLU, false>), grid, dim3(256), 0, s, g);
+}
+
 int launch_gemm(lumen_ctx *ctx, const GemmArgs &a) {
     if (a.M <= 0 || a.N <= 0) return LUMEN_OK;
     if (a.epi != EPI_STORE && a.epi != EPI_RESIDUAL && a.epi != EPI_SWIGLU)  // (the switches below read SwiGLU into "else")
@@ -873,15 +1067,20 @@ int launch_gemm(lumen_ctx *ctx, const GemmArgs &a) {
     }
     if (a.epi == EPI_SWIGLU && (a.N & 1)) LUMEN_FAIL(LUMEN_ERR_SHAPE, "SwiGLU epilogue needs an even column count, got %d", a.N);
     GemmArgs g = a;
-    int splits = gemm_big_splits(ctx, a);
+    const bool stream = gemm_stream_applies(a);
+    int splits = stream ? 0 : gemm_big_splits(ctx, a);
     const bool big = splits > 0;
-    if (!big) splits = gemm_splits(ctx, a);
+    if (stream) splits = gemm_stream_splits(ctx, a);
+    else if (!big) splits = gemm_splits(ctx, a);
     if (splits > 1) {
         LUMEN_TRY(gemm_reserve_workspace(ctx, (size_t)splits * a.M * a.N * sizeof(float)));
         g.part = ctx->gemm_ws;
     }
     dim3 grid((a.N + BN - 1) / BN, (a.M + BM - 1) / BM, splits);
-    if (big) {
+    if (stream) {
+        if (a.M <= 16) launch_gemm_stream<1>(g, splits, ctx->stream);
+        else launch_gemm_stream<2>(g, splits, ctx->stream);
+    } else if (big) {
         dim3 bgrid((a.N + GB_N - 1) / GB_N, (a.M + GB_M - 1) / GB_M, splits);
         if (a.w_bf16) launch_gemm_tile<true, 4>(g, bgrid, ctx->stream);
         else launch_gemm_tile<false, 4>(g, bgrid, ctx->stream);

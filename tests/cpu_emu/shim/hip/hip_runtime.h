@@ -106,6 +106,25 @@ static inline unsigned emu_perm(unsigned hi, unsigned lo, unsigned sel) {  // v_
 }
 #define __builtin_amdgcn_perm(hi, lo, sel) emu_perm((hi), (lo), (sel))
 #define __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, x, y, z) (emu::not_emulated("v_mfma_f32_32x32x16_bf16"), (c))
+// v_mfma_f32_16x16x4_f32: D[i][j] = C[i][j] + sum over k < 4 of A[i][k] B[k][j]; lane l gives A[l % 16][l / 16] and
+// B[l / 16][l % 16] and holds D[4 (l / 16) + r][l % 16] in element r.  (The order of the four products inside the
+// instruction is the hardware's; results are compared to a tolerance.)
+template <typename V>
+static inline V emu_mfma_16x16x4f32(float a, float b, V c) {
+    const int lane = (int)(threadIdx.x & 63), j = lane & 15, g = lane >> 4;
+    float bk[4];
+    for (int k = 0; k < 4; ++k) bk[k] = emu_bits_to<float>(emu::wave_exchange(emu_bits_of(b), k * 16 + j));
+    for (int r = 0; r < 4; ++r)
+        for (int k = 0; k < 4; ++k) {
+            const float aik = emu_bits_to<float>(emu::wave_exchange(emu_bits_of(a), k * 16 + 4 * g + r));
+            c[r] = fmaf(aik, bk[k], c[r]);
+        }
+    return c;
+}
+#define __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, x, y, z) emu_mfma_16x16x4f32((a), (b), (c))
+// On the GPU the lanes of a wavefront run in lockstep and the wave barrier only orders the compiler; here the lanes are
+// fibers of their own and have to meet.
+#define __builtin_amdgcn_wave_barrier() ((void)emu::wave_exchange(0u, 0))
 
 using std::max;
 using std::min;

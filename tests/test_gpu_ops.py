@@ -116,6 +116,28 @@ def test_gemm_keeps_f32_accuracy_across_magnitudes():
     assert errb.max() <= 1e-6, errb.max()
 
 
+@pytest.mark.parametrize("M,N,K", [(5, 40, 36), (17, 96, 4), (31, 2047, 2048), (32, 2560, 2048), (9, 100, 260),
+                                   (24, 11264, 2048), (32, 2048, 5632), (20, 31, 8196), (16, 48, 64)])
+def test_gemm_five_to_32_rows(M, N, K):
+    """Five to 32 rows of A with f32 weights: the weight-streaming matrix-core kernel (a wavefront per 16 rows of W and
+    range of K, blocks of 32 k, the last one partial; one or two row tiles of A, f32 matrix instructions; ranges of K
+    added inside the workgroup and, split further, in a second pass).  Values against the checker and the fp64 product, and -- rows of A and W
+    scaled over 24 decades -- every output relative to the size of its own terms, as for the tile kernels."""
+    A = f32(RNG.normal(0, 1, (M, K)))
+    W = f32(RNG.normal(0, 0.02, (N, K)))
+    C = ops.matmul(dev(A), dev(W)).data()
+    assert C.shape == (M, N)
+    assert max_rel(C, lo.gemm(A, W)) <= 1e-5
+    assert max_rel(C, A.astype(np.float64) @ W.T.astype(np.float64)) <= 1e-5
+    A2 = RNG.normal(0, 1, (M, K)) * 10.0 ** RNG.uniform(-3, 3, (M, K)) * 10.0 ** RNG.integers(-12, 13, (M, 1))
+    W2 = RNG.normal(0, 1, (N, K)) * 10.0 ** RNG.uniform(-3, 3, (N, K)) * 10.0 ** RNG.integers(-12, 13, (N, 1))
+    A2, W2 = f32(A2), f32(W2)
+    C2 = ops.matmul(dev(A2), dev(W2)).data()
+    a64, w64 = A2.astype(np.float64), W2.astype(np.float64)
+    err = np.abs(C2 - a64 @ w64.T) / (np.abs(a64) @ np.abs(w64).T)
+    assert np.isfinite(C2).all() and err.max() <= 1e-6, err.max()
+
+
 @pytest.mark.parametrize("M,N,K", [(48, 300, 256), (3, 301, 1024), (4, 4096, 11008)])
 def test_gemm_bf16_weights(M, N, K):
     A = f32(RNG.normal(0, 1, (M, K)))
