@@ -21,6 +21,7 @@
 // result does not depend on scheduling.
 #include "internal.h"
 #include "wave_reduce.h"
+#include "stage_times.h"
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
@@ -573,6 +574,7 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmArgs a) {
     constexpr int RL = 64 * 4 / GS_KW;  // rows of W one load instruction covers
     __shared__ __align__(16) float stage_w[4][16 * GS_LW];
     __shared__ __align__(16) float stage_a[4][MT][16 * GS_LA];
+    STAGE_T(0);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = lane & 15, g = lane >> 4;
     const int bn = blockIdx.x * 16;
@@ -665,16 +667,21 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmArgs a) {
 #pragma unroll
     for (int j = 0; j < GS_DA; ++j)
         if (d0 * SUB + j < d1 * SUB) fetch_a(j, d0 * SUB + j);
+    STAGE_T(1);
     for (int d = d0; d < d1; d += GS_DW) {
 #pragma unroll
         for (int j = 0; j < GS_DW; ++j)
             if (d + j < d1) {
                 block(j, d + j);
                 if (d + j + GS_DW < d1) fetch_w(j, d + j + GS_DW);
+                if (d + j == d0) STAGE_T(2);
+                if (d + j == d0 + 7) STAGE_T(3);
             }
     }
+    STAGE_T(4);
     // the four K ranges of the workgroup, added in wavefront order
     __syncthreads();
+    STAGE_T(5);
     float *red = &stage_w[0][0];  // [3][MT][4][64] floats
     if (wave > 0) {
 #pragma unroll
@@ -709,6 +716,7 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmArgs a) {
                 a.C[o] = (EPI == EPI_RESIDUAL) ? a.residual[o] + v : v;
             }
         }
+    STAGE_T_STORES_DONE(6);
 }
 
 #define GEMM_MAX_SPLITS 16
@@ -1080,6 +1088,9 @@ int launch_gemm(lumen_ctx *ctx, const GemmArgs &a) {
     if (stream) {
         if (a.M <= 16) launch_gemm_stream<1>(g, splits, ctx->stream);
         else launch_gemm_stream<2>(g, splits, ctx->stream);
+        stage_times_report(ctx, "weight-streaming prompt product", (a.N + 15) / 16 * splits,
+                           "start, [1] requests out, [2] first block done, [3] eighth block done, [4] blocks done, [5] after the "
+                           "barrier, [6] stores acknowledged");
     } else if (big) {
         dim3 bgrid((a.N + GB_N - 1) / GB_N, (a.M + GB_M - 1) / GB_M, splits);
         if (a.w_bf16) launch_gemm_tile<true, 4>(g, bgrid, ctx->stream);
