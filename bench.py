@@ -140,6 +140,19 @@ def decode_bench(model_name, cfg, n_prompt, steps, warmup, mode, keep_host, head
     # prefill (outside the timed decode region; reported separately).  The first pass sizes the
     # prompt buffers and the GEMM workspace; the second, from a reset cache, is the one timed.
     ctx = model.ctx
+    short_ms = {}
+    if headline:  # prompts of a few rows (a chat turn's new tokens): the weight-streaming prompt products
+        for n_short in (4, 16, 32):
+            if n_short >= n_prompt:
+                continue
+            best = None
+            for _ in range(3):
+                model.reset_kv_caches()
+                ctx.timer_start()
+                model.forward(prompt[:n_short], all_rows=False)
+                t = ctx.timer_stop()
+                best = t if best is None else min(best, t)
+            short_ms[str(n_short)] = round(best, 3)
     prefill_all_ms = []
     for _ in range(3):  # the third pass is the steady one (the first two still see allocator / loader warm-up)
         model.reset_kv_caches()
@@ -247,7 +260,8 @@ def decode_bench(model_name, cfg, n_prompt, steps, warmup, mode, keep_host, head
                       "avg_launch_us": round(at_avg_ms * 1e3, 3), "achieved_GBps": round(at_bytes / (at_avg_ms * 1e-3) / 1e9, 1),
                       "frac_of_8TBps": round(at_bytes / (at_avg_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
         "kernels": kernels, "kernel_instances": names,
-        "prefill": dict(prefill_report(cfg, n_prompt, prefill_ms), passes_ms=[round(x, 3) for x in prefill_all_ms]),
+        "prefill": dict(prefill_report(cfg, n_prompt, prefill_ms), passes_ms=[round(x, 3) for x in prefill_all_ms],
+                        **({"short_prompts_ms": short_ms} if short_ms else {})),
         "decode_mode": mode, "eager_ms_per_step": round(eager_ms / steps, 5),
         "self_check": {"graph_picks_equal_eager_picks": True, "steps": steps},
         "wall_s_timed_region": round(wall, 4), "setup_s": round(t_setup, 1),

@@ -395,7 +395,7 @@ __global__ __launch_bounds__(256, (F == 4 ? 1 : 2)) void gemm_bf16x3_tile_kernel
     store_wave_tiles<EPI, PARTIAL, F>(a, acc, bm, bn, wm, wn, lane);
 }
 
-// Prompts of two to four rows (a batch of drafted tokens, the tail of a chunked prompt): the product is bound by the weights,
+// Prompts of two rows (up to four where GEMM_SKINNY_MAX_M is raised): the product is bound by the weights,
 // which the tile kernels above cannot stream at anything like the memory's rate (they take 100 us per layer whatever M
 // is).  This kernel walks W the way the single-row product does: a wavefront takes units of two whole rows, lanes across
 // K with 16-byte loads, in pieces of 4 sweeps x 2 rows = 8 loads per lane, two pieces in flight and the next one
@@ -549,11 +549,11 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(GemmArgs a, int
     }
 }
 
-// Prompts of five to 32 rows (a chat turn's new tokens, the tail of a chunked prompt): the product is bound by the
+// Prompts of three to 32 rows (a chat turn's new tokens, the tail of a chunked prompt): the product is bound by the
 // weights, and the tile kernels above take the same ~100 us per layer for 5 rows as for 128.  This kernel streams W once
 // and multiplies on the matrix cores without sharing anything between wavefronts: a wavefront owns 16 rows of W (a column
 // tile of C; N / 16 tiles spread evenly over the compute units where N / 32 would not) over a range of K and all
-// MT <= 2 row tiles of 16 rows of A.  It fetches 16 x 32 blocks of W (GS_DW blocks ahead: 16 KB per wavefront in flight,
+// MT <= 2 row tiles of 16 rows of A.  It fetches 16 x 32 blocks of W (8 or 16 blocks ahead: 16 KB per wavefront in flight,
 // what the single-row product keeps in flight) and 16 x 32 blocks of A (those come from L2) with coalesced 16-byte loads,
 // turns them into operand order through a wavefront-private LDS buffer (no barriers) and multiplies with the f32
 // matrix instruction (v_mfma_f32_16x16x4_f32: a sixteenth of the bf16 rate, but no splitting into bf16 parts on the
@@ -561,28 +561,26 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(GemmArgs a, int
 // further row tile costs 20 us per layer in f32 matrix instructions, so beyond 32 rows the tile kernels are as fast).  The four wavefronts of a
 // workgroup take consecutive K ranges of ONE column tile and add their accumulators through LDS in wavefront order; ranges
 // are split further over gridDim.z like the tile kernels' (partial tiles of M x 16).
-#define GS_KW 32           // k per block of W (128 and 256, longer visits to a row, measured no faster: 23.6 and 35 against 24.7 us)
-#define GS_LW (GS_KW + 4)  // floats per LDS row of a staged block of W: rows start 4 banks apart, 8 rows cover all banks
-#define GS_LA 36           // ... of a 32-wide block of A
-#define GS_DW 8            // blocks of W in flight per wavefront (16 KB)
-#define GS_DA 2            // 32-wide blocks of A in flight
+#define GS_LD 36  // floats per LDS row of a staged 16 x 32 block: rows start 4 banks apart, 8 rows cover all banks (blocks of
+                  // 128 and 256 k -- longer visits to a row of W -- measured no faster: 23.6 and 35 against 24.7 us)
+#define GS_DA 2   // blocks of A in flight
 typedef float v4acc __attribute__((ext_vector_type(4)));
-template <int MT, int EPI, bool PARTIAL>
+// BF16: W holds bf16 bits; widened by a shift on the way into the operand registers like src/loader.rs:58 widens them at
+// load time, so the products are those of f32 weights with the same values.
+template <int MT, bool BF16, int EPI, bool PARTIAL>
 __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmArgs a) {
-    constexpr int WP = GS_KW / 16;   // 16-byte pieces of a W block per lane: 16 rows x GS_KW / 4 pieces / 64 lanes
-    constexpr int SUB = GS_KW / 32;  // 32-wide blocks of A per block of W
-    constexpr int RL = 64 * 4 / GS_KW;  // rows of W one load instruction covers
-    __shared__ __align__(16) float stage_w[4][16 * GS_LW];
-    __shared__ __align__(16) float stage_a[4][MT][16 * GS_LA];
+    constexpr int DW = BF16 ? 16 : 8;  // blocks of W in flight per wavefront (16 KB)
+    constexpr int WP = BF16 ? 1 : 2;   // 16-byte pieces of a W block per lane
+    __shared__ __align__(16) float stage_w[4][16 * GS_LD];
+    __shared__ __align__(16) float stage_a[4][MT][16 * GS_LD];
     STAGE_T(0);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = lane & 15, g = lane >> 4;
     const int bn = blockIdx.x * 16;
     const int M = a.M, N = a.N, K = a.K;
     const float *A = a.A;
-    const float *W = (const float *)a.W;
-    // blocks of GS_KW k: this workgroup's share [z per_wg, (z + 1) per_wg), this wavefront's quarter of it
-    const int nblk = (K + GS_KW - 1) / GS_KW;
+    // blocks of 32 k: this workgroup's share [z per_wg, (z + 1) per_wg), this wavefront's quarter of it
+    const int nblk = (K + 31) / 32;
     const int per_wg = (nblk + (int)gridDim.z - 1) / (int)gridDim.z;
     const int per_wave = (per_wg + 3) / 4;
     const int wg0 = (int)blockIdx.z * per_wg;
@@ -593,87 +591,97 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmArgs a) {
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[t] = v4acc{0.f, 0.f, 0.f, 0.f};
 
-    // W: piece i of this lane in a 16 x GS_KW block is row RL i + lane / (64 / RL), k offset 4 * (lane % (64 / RL)):
-    // the lanes of a row read GS_KW * 4 contiguous bytes.  A: piece i (0, 1) of a 16 x 32 block is row 8 i + lane / 8,
-    // k offset 4 * (lane % 8).  K is a multiple of 4: a piece is inside or outside as a whole.  Rows past the end are
+    // Piece i (0, 1) of this lane in a 16 x 32 block of f32 values: row 8 i + lane / 8, k offset 4 * (lane % 8) -- the 8
+    // lanes of a row read 128 contiguous bytes; a block of bf16 weights is one piece per lane: row lane / 4, k offset
+    // 8 * (lane % 4).  K is a multiple of the piece: a piece is inside or outside as a whole.  Rows past the end are
     // clamped (their products are never stored).
-    const int wrow = lane / (64 / RL), wk = (lane % (64 / RL)) * 4;
     const int arow = lane >> 3, ak = (lane & 7) * 4;
-    const float *wp = W + (size_t)min(bn + wrow, N - 1) * K + wk;
-    const size_t wstep = (size_t)RL * K;  // (rows past N - 1: the loads of the last tile are clamped one by one below)
-    const bool wclamp = bn + 16 > N;
+    const int wrow = BF16 ? lane >> 2 : arow, wk = BF16 ? (lane & 3) * 8 : ak;
+    const char *wp[WP];
     const float *ap[MT][2];
+#pragma unroll
+    for (int i = 0; i < WP; ++i)
+        wp[i] = (const char *)a.W + ((size_t)min(bn + wrow + 8 * i, N - 1) * K + wk) * (BF16 ? 2 : 4);
 #pragma unroll
     for (int t = 0; t < MT; ++t)
 #pragma unroll
         for (int i = 0; i < 2; ++i) ap[t][i] = A + (size_t)min(t * 16 + arow + 8 * i, M - 1) * K + ak;
-    v4f vw[GS_DW][WP], va[GS_DA][MT][2];
+    v4u vw[DW][WP];
+    v4f va[GS_DA][MT][2];
     auto fetch_w = [&](int slot, int d) {
-        const bool in = d * GS_KW + wk < K;
+        const bool in = d * 32 + wk < K;
 #pragma unroll
         for (int i = 0; i < WP; ++i) {
-            vw[slot][i] = v4f{0.f, 0.f, 0.f, 0.f};
-            const float *q = wclamp ? W + (size_t)min(bn + wrow + RL * i, N - 1) * K + wk : wp + i * wstep;
-            if (in) vw[slot][i] = __builtin_nontemporal_load((const v4f *)(q + (size_t)d * GS_KW));
+            vw[slot][i] = v4u{0u, 0u, 0u, 0u};
+            if (in) vw[slot][i] = __builtin_nontemporal_load((const v4u *)(wp[i] + (size_t)d * (BF16 ? 64 : 128)));
         }
     };
-    auto fetch_a = [&](int slot, int e) {  // e: index of the 32-wide block of A
-        const bool in = e * 32 + ak < K;
+    auto fetch_a = [&](int slot, int d) {
+        const bool in = d * 32 + ak < K;
 #pragma unroll
         for (int t = 0; t < MT; ++t)
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
                 va[slot][t][i] = v4f{0.f, 0.f, 0.f, 0.f};
-                if (in) va[slot][t][i] = *(const v4f *)(ap[t][i] + e * 32);
+                if (in) va[slot][t][i] = *(const v4f *)(ap[t][i] + d * 32);
             }
     };
     float *sw = stage_w[wave];
-    auto block = [&](int ws, int d) {
+    auto block = [&](int ws, int as) {
+        if (BF16) {  // rows of 36 bf16 (72 bytes): 8-byte accesses
+            uint16_t *h = (uint16_t *)sw + wrow * GS_LD + wk;
+            *(v2u *)h = v2u{vw[ws][0].x, vw[ws][0].y};
+            *(v2u *)(h + 4) = v2u{vw[ws][0].z, vw[ws][0].w};
+        } else {
 #pragma unroll
-        for (int i = 0; i < WP; ++i) *(v4f *)(sw + (wrow + RL * i) * GS_LW + wk) = vw[ws][i];
-#pragma unroll
-        for (int u = 0; u < SUB; ++u) {
-            const int as = (ws * SUB + u) % GS_DA;
-#pragma unroll
-            for (int t = 0; t < MT; ++t)
-#pragma unroll
-                for (int i = 0; i < 2; ++i) *(v4f *)(stage_a[wave][t] + (arow + 8 * i) * GS_LA + ak) = va[as][t][i];
-            // The buffers are this wavefront's own and its LDS instructions execute in order: the reads below see the
-            // writes above without a workgroup barrier (the wave barrier emits no instruction; it keeps the compiler
-            // from moving LDS accesses across it).
-            __builtin_amdgcn_wave_barrier();
-            if (d * SUB + u + GS_DA < d1 * SUB) fetch_a(as, d * SUB + u + GS_DA);
-            // lane (c, g) takes the k = 16 j + 4 g + e of row c for both operands: instruction (j, e) multiplies four k
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const v4f wf = *(const v4f *)(sw + c * GS_LW + u * 32 + j * 16 + g * 4);
-                v4f af[MT];
-#pragma unroll
-                for (int t = 0; t < MT; ++t) af[t] = *(const v4f *)(stage_a[wave][t] + c * GS_LA + j * 16 + g * 4);
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-#pragma unroll
-                    for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[t][e], wf[e], acc[t], 0, 0, 0);
-            }
-            __builtin_amdgcn_wave_barrier();  // (the next block's writes come after these reads)
+            for (int i = 0; i < WP; ++i) *(v4u *)(sw + (wrow + 8 * i) * GS_LD + wk) = vw[ws][i];
         }
-    };
-    // block d + j of W sits in slot j % GS_DW; the 32-wide blocks of A rotate through GS_DA slots (a trip of the loop
-    // below is a whole number of turns of that ring); a slot is requested anew as soon as its block is used
-    static_assert((GS_DW * SUB) % GS_DA == 0, "the A ring must divide a trip of the loop");
 #pragma unroll
-    for (int j = 0; j < GS_DW; ++j)
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int i = 0; i < 2; ++i) *(v4f *)(stage_a[wave][t] + (arow + 8 * i) * GS_LD + ak) = va[as][t][i];
+        // The buffers are this wavefront's own and its LDS instructions execute in order: the reads below see the
+        // writes above without a workgroup barrier (the wave barrier emits no instruction; it keeps the compiler
+        // from moving LDS accesses across it).
+        __builtin_amdgcn_wave_barrier();
+        // lane (c, g) takes the k = 16 j + 4 g + e of row c for both operands: instruction (j, e) multiplies four k
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            v4f wf;
+            if (BF16) {
+                const v2u r = *(const v2u *)((const uint16_t *)sw + c * GS_LD + j * 16 + g * 4);
+                wf = v4f{__uint_as_float(r.x << 16), __uint_as_float(r.x & 0xffff0000u), __uint_as_float(r.y << 16),
+                         __uint_as_float(r.y & 0xffff0000u)};
+            } else {
+                wf = *(const v4f *)(sw + c * GS_LD + j * 16 + g * 4);
+            }
+            v4f af[MT];
+#pragma unroll
+            for (int t = 0; t < MT; ++t) af[t] = *(const v4f *)(stage_a[wave][t] + c * GS_LD + j * 16 + g * 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[t][e], wf[e], acc[t], 0, 0, 0);
+        }
+        __builtin_amdgcn_wave_barrier();  // (the next block's writes come after these reads)
+    };
+    // block d0 + j of W sits in slot j % DW, of A in slot j % GS_DA (a trip of the loop below is a whole number of turns
+    // of both rings); a slot is requested anew as soon as its block is used
+    static_assert(DW % GS_DA == 0, "the A ring must divide a trip of the loop");
+#pragma unroll
+    for (int j = 0; j < DW; ++j)
         if (d0 + j < d1) fetch_w(j, d0 + j);
 #pragma unroll
     for (int j = 0; j < GS_DA; ++j)
-        if (d0 * SUB + j < d1 * SUB) fetch_a(j, d0 * SUB + j);
+        if (d0 + j < d1) fetch_a(j, d0 + j);
     STAGE_T(1);
-    for (int d = d0; d < d1; d += GS_DW) {
+    for (int d = d0; d < d1; d += DW) {
 #pragma unroll
-        for (int j = 0; j < GS_DW; ++j)
+        for (int j = 0; j < DW; ++j)
             if (d + j < d1) {
-                block(j, d + j);
-                if (d + j + GS_DW < d1) fetch_w(j, d + j + GS_DW);
+                block(j, j % GS_DA);
+                if (d + j + DW < d1) fetch_w(j, d + j + DW);
+                if (d + j + GS_DA < d1) fetch_a(j % GS_DA, d + j + GS_DA);
                 if (d + j == d0) STAGE_T(2);
                 if (d + j == d0 + 7) STAGE_T(3);
             }
@@ -935,23 +943,26 @@ static int gemm_big_splits(const lumen_ctx *ctx, const GemmArgs &a) {
     return best;
 }
 
-// up to 4 rows of A the weight-streaming kernel wins (TinyLlama shape: prompt pass of 2 tokens 2.45 -> 1.48 ms, of 4
-// tokens 2.46 -> 1.89 ms); at 8 rows the two are level, beyond that the multiply-adds and LDS reads per piece cost more
-// than the tile kernels' fixed 100 us per layer
+// Two rows of A: the vector-ALU kernel above (TinyLlama shape: prompt pass of 2 tokens 1.43 ms against 1.57 with the
+// matrix-core kernel below; with three and four rows it is the other way round, 1.75 / 1.83 against 1.57 ms, and on the
+// Llama-2-7B shape with bf16 weights 8.1 / 8.3 against 5.7 ms)
 #ifndef GEMM_SKINNY_MAX_M
-#define GEMM_SKINNY_MAX_M 4
+#define GEMM_SKINNY_MAX_M 2
 #endif
-// The weight-streaming matrix-core kernel takes five to 32 rows of A with f32 weights.
+// The weight-streaming matrix-core kernel takes three to 32 rows of A, with bf16-stored weights three to 16: a bf16
+// weight is half the bytes for the same f32 matrix instructions, and the second row tile then costs more than the tile
+// kernels do (Llama-2-7B shape, prompt pass of 32 tokens: 7.7 against 6.0 ms; of 5-16 tokens 5.7 against 5.9).
 #define GEMM_STREAM_MAX_M 32
+static int gemm_stream_max_rows(int w_bf16) { return w_bf16 ? 16 : GEMM_STREAM_MAX_M; }
 static bool gemm_stream_applies(const GemmArgs &a) {
     const bool aligned = (((uintptr_t)a.A | (uintptr_t)a.W) & 15) == 0;
-    return !a.w_bf16 && aligned && a.K > 0 && a.K % 4 == 0 && a.M > GEMM_SKINNY_MAX_M && a.M <= GEMM_STREAM_MAX_M &&
+    return aligned && a.K > 0 && a.K % (a.w_bf16 ? 8 : 4) == 0 && a.M > GEMM_SKINNY_MAX_M && a.M <= gemm_stream_max_rows(a.w_bf16) &&
            !(a.epi == EPI_SWIGLU && (a.N & 1));
 }
 // Workgroups along K per column tile of 16: about three workgroups per compute unit over the chip, at least four
 // blocks of K per wavefront, 16 splits at most (the split sum takes that many).
 static int gemm_stream_splits(const lumen_ctx *ctx, const GemmArgs &a) {
-    const long tiles = (a.N + 15) / 16, nblk = (a.K + GS_KW - 1) / GS_KW;
+    const long tiles = (a.N + 15) / 16, nblk = (a.K + 31) / 32;
     long s = (3L * ctx->num_cus + tiles / 2) / tiles;
     while (s > 1 && nblk / (4 * s) < 4) --s;
     if (s > GEMM_MAX_SPLITS) s = GEMM_MAX_SPLITS;
@@ -974,7 +985,7 @@ size_t gemm_workspace_bytes(const lumen_ctx *ctx, int M, int N, int K, int w_bf1
     GemmArgs a = {};
     a.M = M; a.N = N; a.K = K; a.w_bf16 = w_bf16;
     if (M <= 0 || N <= 0 || K <= 0 || K % (w_bf16 ? 8 : 4)) return 0;
-    if (M > GEMM_SKINNY_MAX_M && M <= GEMM_STREAM_MAX_M && !w_bf16) {  // (alignment is the caller's: assume the streaming kernel)
+    if (M > GEMM_SKINNY_MAX_M && M <= gemm_stream_max_rows(w_bf16)) {  // (alignment is the caller's: assume the streaming kernel)
         const int st = gemm_stream_splits(ctx, a);
         return st > 1 ? (size_t)st * M * N * sizeof(float) : 0;
     }
@@ -1031,13 +1042,13 @@ static int gemm_skinny_rows(const GemmArgs &a, int *kpad_out) {
 }
 
 
-template <int MT>
+template <int MT, bool BF16>
 static void launch_gemm_stream(const GemmArgs &g, int splits, hipStream_t s) {
     dim3 grid((g.N + 15) / 16, 1, splits);
-    if (splits > 1) hipLaunchKernelGGL((gemm_stream_kernel<MT, EPI_STORE, true>), grid, dim3(256), 0, s, g);
-    else if (g.epi == EPI_STORE) hipLaunchKernelGGL((gemm_stream_kernel<MT, EPI_STORE, false>), grid, dim3(256), 0, s, g);
-    else if (g.epi == EPI_RESIDUAL) hipLaunchKernelGGL((gemm_stream_kernel<MT, EPI_RESIDUAL, false>), grid, dim3(256), 0, s, g);
-    else hipLaunchKernelGGL((gemm_stream_kernel<MT, EPI_SWIGLU, false>), grid, dim3(256), 0, s, g);
+    if (splits > 1) hipLaunchKernelGGL((gemm_stream_kernel<MT, BF16, EPI_STORE, true>), grid, dim3(256), 0, s, g);
+    else if (g.epi == EPI_STORE) hipLaunchKernelGGL((gemm_stream_kernel<MT, BF16, EPI_STORE, false>), grid, dim3(256), 0, s, g);
+    else if (g.epi == EPI_RESIDUAL) hipLaunchKernelGGL((gemm_stream_kernel<MT, BF16, EPI_RESIDUAL, false>), grid, dim3(256), 0, s, g);
+    else hipLaunchKernelGGL((gemm_stream_kernel<MT, BF16, EPI_SWIGLU, false>), grid, dim3(256), 0, s, g);
 }
 
 int launch_gemm(lumen_ctx *ctx, const GemmArgs &a) {
@@ -1049,7 +1060,7 @@ int launch_gemm(lumen_ctx *ctx, const GemmArgs &a) {
     int kpad = 0;
     const int ms = gemm_skinny_rows(a, &kpad);
     if (ms) {
-        // two to four rows of A: the weights are streamed the way the single-row product streams them, once per MS rows
+        // two rows of A: the weights are streamed the way the single-row product streams them, once per MS rows
         // of A (4, or 2 where 4 rows of K padded to whole pieces do not fit LDS)
         {
             if (a.splits_used) *a.splits_used = 1;
@@ -1086,8 +1097,12 @@ int launch_gemm(lumen_ctx *ctx, const GemmArgs &a) {
     }
     dim3 grid((a.N + BN - 1) / BN, (a.M + BM - 1) / BM, splits);
     if (stream) {
-        if (a.M <= 16) launch_gemm_stream<1>(g, splits, ctx->stream);
-        else launch_gemm_stream<2>(g, splits, ctx->stream);
+        if (a.w_bf16) {
+            launch_gemm_stream<1, true>(g, splits, ctx->stream);
+        } else {
+            if (a.M <= 16) launch_gemm_stream<1, false>(g, splits, ctx->stream);
+            else launch_gemm_stream<2, false>(g, splits, ctx->stream);
+        }
         stage_times_report(ctx, "weight-streaming prompt product", (a.N + 15) / 16 * splits,
                            "start, [1] requests out, [2] first block done, [3] eighth block done, [4] blocks done, [5] after the "
                            "barrier, [6] stores acknowledged");

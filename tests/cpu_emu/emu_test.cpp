@@ -240,9 +240,9 @@ static void case_bf16(lumen_ctx *ctx) {
 
 // the few-row product on its own: ragged N and K, all three epilogues through the operator-level entry points
 static void case_skinny(lumen_ctx *ctx) {
-    printf("skinny: lumen_matmul_f32 / lumen_gemm_bf16w with 2-4 rows, lumen_matmul_f32 with 5-32 rows, ragged shapes\n");
-    // (five to 32 rows: the weight-streaming kernel with the f32 matrix instruction, K split inside and across workgroups)
-    const int shapes[][3] = {{2, 37, 100}, {3, 64, 1032}, {4, 129, 264}, {4, 6, 4}, {5, 37, 100}, {17, 40, 1032}, {32, 18, 36}, {9, 16, 4}};
+    printf("skinny: lumen_matmul_f32 / lumen_gemm_bf16w with 2 rows (vector ALU) and 3-32 rows (f32 matrix instruction), ragged shapes\n");
+    // (three to 32 rows: the weight-streaming kernel with the f32 matrix instruction, K split inside and across workgroups)
+    const int shapes[][3] = {{2, 37, 100}, {2, 64, 1032}, {3, 64, 1032}, {4, 129, 264}, {4, 6, 4}, {5, 37, 100}, {16, 40, 1032}, {32, 18, 40}, {9, 16, 4}};
     for (const auto &sh : shapes) {
         const int M = sh[0], N = sh[1], K = sh[2];
         std::vector<float> A = randn((size_t)M * K, 1.f), W = randn((size_t)N * K, 0.05f), C((size_t)M * N), R((size_t)M * N);
@@ -258,7 +258,7 @@ static void case_skinny(lumen_ctx *ctx) {
         const double e = max_rel(C.data(), R.data(), C.size());
         printf("  %d x %d x %d f32: max rel err %.2e\n", M, N, K, e);
         CHECK(e <= 1e-5, "skinny %dx%dx%d: %.3g", M, N, K, e);
-        if (K % 8 == 0 && M <= 4) {  // (more rows with bf16 weights: the bf16 matrix instructions, not emulated)
+        if (K % 8 == 0 && M <= 16) {  // (more rows with bf16 weights: the bf16 matrix instructions, not emulated)
             std::vector<float> Wb = W;
             to_bf16_values(Wb);
             std::vector<uint16_t> bits(Wb.size());

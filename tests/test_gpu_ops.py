@@ -73,8 +73,8 @@ def test_matmul_shape_errors_and_empty():
 
 @pytest.mark.parametrize("M,N,K", [(2, 3, 4), (7, 33, 132), (128, 256, 2048), (130, 200, 64), (64, 5632, 512),
                                    (5, 9, 7), (300, 129, 260), (16, 2560, 2048),
-                                   # two to four rows: the weight-streaming kernel (whole rows per wavefront); ragged N,
-                                   # K not a whole number of pieces, K that needs the 2-row tile, one unit per wavefront
+                                   # two rows: the vector-ALU weight-streaming kernel (whole rows per wavefront), three
+                                   # and four: the matrix-core one; ragged N, K not a whole number of pieces / blocks
                                    (2, 2560, 2048), (3, 2047, 5632), (4, 11264, 2048), (4, 33, 8200), (2, 5, 1028),
                                    (4, 4096, 11008)])
 def test_gemm_against_oracle(M, N, K):
@@ -119,7 +119,7 @@ def test_gemm_keeps_f32_accuracy_across_magnitudes():
 @pytest.mark.parametrize("M,N,K", [(5, 40, 36), (17, 96, 4), (31, 2047, 2048), (32, 2560, 2048), (9, 100, 260),
                                    (24, 11264, 2048), (32, 2048, 5632), (20, 31, 8196), (16, 48, 64)])
 def test_gemm_five_to_32_rows(M, N, K):
-    """Five to 32 rows of A with f32 weights: the weight-streaming matrix-core kernel (a wavefront per 16 rows of W and
+    """Three to 32 rows of A with f32 weights: the weight-streaming matrix-core kernel (a wavefront per 16 rows of W and
     range of K, blocks of 32 k, the last one partial; one or two row tiles of A, f32 matrix instructions; ranges of K
     added inside the workgroup and, split further, in a second pass).  Values against the checker and the fp64 product, and -- rows of A and W
     scaled over 24 decades -- every output relative to the size of its own terms, as for the tile kernels."""
@@ -138,7 +138,9 @@ def test_gemm_five_to_32_rows(M, N, K):
     assert np.isfinite(C2).all() and err.max() <= 1e-6, err.max()
 
 
-@pytest.mark.parametrize("M,N,K", [(48, 300, 256), (3, 301, 1024), (4, 4096, 11008)])
+@pytest.mark.parametrize("M,N,K", [(48, 300, 256), (3, 301, 1024), (4, 4096, 11008),
+                                   # five to 32 rows: the weight-streaming matrix-core kernel, bf16 bits widened on the way
+                                   (5, 40, 40), (17, 301, 1032), (32, 4096, 2048), (16, 31, 8)])
 def test_gemm_bf16_weights(M, N, K):
     A = f32(RNG.normal(0, 1, (M, K)))
     bits = lo.f32_to_bf16(f32(RNG.normal(0, 0.02, (N, K))))
