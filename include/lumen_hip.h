@@ -80,7 +80,10 @@ int lumen_copy_d2d(lumen_ctx *ctx, void *dst_dev, const void *src_dev, size_t by
 /* --------------------------------------------------------------------- ops */
 /* ops::matmul::matmul forward, src/ops/matmul.rs:10-99.  A [M, K_a] @ W[N, K_w]^T
  * -> C [M, N].  K_a != K_w -> LUMEN_ERR_SHAPE (:33-38).  M == 1 takes the
- * memory-bound GEMV (:42-69), M > 1 the MFMA GEMM (:70-92). */
+ * memory-bound GEMV (:42-69), M > 1 the GEMM branch (:70-92): two rows stream W
+ * through the vector ALU, 3-32 rows through the f32 matrix instruction (both
+ * bound by the weights), more rows run on the bf16 matrix cores with every
+ * f32 value taken as three bf16 parts (f32 accuracy). */
 int lumen_matmul_f32(lumen_ctx *ctx, const float *A_dev, const float *W_dev, float *C_dev,
                      int M, int N, int K_a, int K_w);
 /* the two branches on their own.  The GEMM splits K over workgroups when its tile grid
