@@ -551,6 +551,15 @@ def test_tinyllama_1b_shape_prefill_128_decode_teacher_forced():
     # on-device greedy loop reproduces itself and advances the cache
     a = gpu.decode_greedy(int(ids[0]), 8)
     assert gpu.kv_len == 144 + 8 and a.shape == (8,)
+    # a follow-up turn of 12 and one of 20 tokens into the live cache: at this width the gate|up product of the
+    # weight-streaming prompt kernel runs unsplit, with the SwiGLU epilogue inside (one and two row tiles)
+    gpu.reset_kv_caches()
+    ora.reset()
+    turn = synth.make_tokens(12 + 20, cfg["vocab_size"], seed=3)
+    for lo_i, hi_i in ((0, 12), (12, 32)):
+        got = gpu.forward(turn[lo_i:hi_i], all_rows=True)
+        rc, ref = ora.forward(turn[lo_i:hi_i])
+        assert rc == lo.LO_OK and max_rel(got, ref) <= 1e-4
 
 
 def _stream_build(cfg, seed, bf16=False):
