@@ -424,6 +424,48 @@ static void selfcheck_oob(lumen_ctx *ctx) {
     fprintf(stderr, "selfcheck: the write past the array went unnoticed\n");
 }
 
+
+// the row-count dispatch of the products (2 rows: vector ALU; 3-32: f32 matrix instruction, bf16-stored weights up to
+// 16 rows) over pseudo-random ragged shapes: every access bounds-checked by the sanitizer, values against the checker
+static void case_shapes(lumen_ctx *ctx) {
+    printf("shapes: 48 pseudo-random products of 2-32 rows, f32 and bf16-stored weights\n");
+    unsigned long long st = 12345;
+    auto rnd = [&]() { st = st * 6364136223846793005ull + 1442695040888963407ull; return (double)(st >> 11) / 9007199254740992.0; };
+    double worst = 0.0;
+    for (int it = 0; it < 48; ++it) {
+        const int M = 2 + (int)(rnd() * 31), N = 1 + (int)(rnd() * 70), K = 4 * (1 + (int)(rnd() * (it % 3 == 0 ? 700 : 40)));
+        const bool bf16 = (it & 1) && K % 8 == 0 && M <= 16;
+        std::vector<float> A = randn((size_t)M * K, 1.f), W = randn((size_t)N * K, 0.05f), C((size_t)M * N), R((size_t)M * N);
+        std::vector<uint16_t> bits(W.size());
+        if (bf16) {
+            to_bf16_values(W);
+            for (size_t i = 0; i < W.size(); ++i) {
+                uint32_t u;
+                memcpy(&u, &W[i], 4);
+                bits[i] = (uint16_t)(u >> 16);
+            }
+        }
+        void *dA, *dW, *dC;
+        OK(lumen_malloc(ctx, A.size() * 4, &dA));
+        OK(lumen_malloc(ctx, bf16 ? bits.size() * 2 : W.size() * 4, &dW));
+        OK(lumen_malloc(ctx, C.size() * 4, &dC));
+        OK(lumen_upload(ctx, dA, A.data(), A.size() * 4));
+        if (bf16) OK(lumen_upload(ctx, dW, bits.data(), bits.size() * 2));
+        else OK(lumen_upload(ctx, dW, W.data(), W.size() * 4));
+        if (bf16) OK(lumen_gemm_bf16w(ctx, (const float *)dA, (const uint16_t *)dW, (float *)dC, M, N, K));
+        else OK(lumen_matmul_f32(ctx, (const float *)dA, (const float *)dW, (float *)dC, M, N, K, K));
+        OK(lumen_download(ctx, C.data(), dC, C.size() * 4));
+        lo_gemm_f32(A.data(), W.data(), R.data(), M, N, K);
+        const double e = max_rel(C.data(), R.data(), C.size());
+        worst = e > worst ? e : worst;
+        CHECK(e <= 1e-5, "product %d x %d x %d%s: %.3g", M, N, K, bf16 ? " bf16 weights" : "", e);
+        OK(lumen_free(ctx, dA));
+        OK(lumen_free(ctx, dW));
+        OK(lumen_free(ctx, dC));
+    }
+    printf("  worst max rel err %.2e\n", worst);
+}
+
 int main(int argc, char **argv) {
     lo_set_threads(4);
     lumen_ctx *ctx = nullptr;
@@ -433,7 +475,7 @@ int main(int argc, char **argv) {
         return 0;  // (reached only if nothing stopped the program: the test expects a sanitizer report instead)
     }
     struct { const char *name; void (*fn)(lumen_ctx *); } cases[] = {
-        {"chain", case_chain}, {"sliced", case_sliced}, {"qknorm", case_qknorm}, {"bf16", case_bf16}, {"skinny", case_skinny}, {"attn", case_attn}, {"layerop", case_layerop}};
+        {"chain", case_chain}, {"sliced", case_sliced}, {"qknorm", case_qknorm}, {"bf16", case_bf16}, {"skinny", case_skinny}, {"attn", case_attn}, {"layerop", case_layerop}, {"shapes", case_shapes}};
     for (const auto &c : cases) {
         bool run = argc <= 1;
         for (int i = 1; i < argc; ++i) run = run || !strcmp(argv[i], c.name);

@@ -24,7 +24,7 @@ def test_decode_kernels_on_the_cpu_under_sanitizers_match_the_checker(emu):
     r = subprocess.run([emu], capture_output=True, text=True, timeout=900)
     assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-3000:]
     assert "cpu emulation: all checks passed" in r.stdout
-    for case in ("chain:", "sliced:", "qknorm:", "bf16:", "skinny:", "attn:", "layerop:"):
+    for case in ("chain:", "sliced:", "qknorm:", "bf16:", "skinny:", "attn:", "layerop:", "shapes:"):
         assert case in r.stdout
     assert "ERROR" not in r.stderr and "runtime error" not in r.stderr, r.stderr[-3000:]
 
